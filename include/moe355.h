@@ -1,0 +1,217 @@
+/*
+ * moe355.h -- C ABI of libmoe355.so: the W8A8-dynamic fused-MoE layer of
+ * vllm-ascend as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - every call only enqueues work on `stream` (a hipStream_t passed as void*)
+ *     and returns; it never synchronises, allocates or frees;
+ *   - scratch memory comes from the caller: ask moe355_*_workspace() for the
+ *     byte count, pass a 256-byte aligned buffer of at least that size;
+ *   - return value 0 = enqueued; negative = rejected, nothing was enqueued
+ *     (see MOE355_E_*; moe355_strerror() gives the text);
+ *   - tensors are dense row-major; "bf16" means raw bfloat16 bits;
+ *   - `dtype` arguments use MOE355_DT_*.
+ *
+ * Each entry point names the interface of the reference tree (vllm-ascend,
+ * paths relative to its root) that it stands in for.
+ */
+#ifndef MOE355_H
+#define MOE355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE355_ABI_VERSION 1
+
+enum {
+    MOE355_OK = 0,
+    MOE355_E_ARG = -1,       /* null pointer, negative size, unknown enum value */
+    MOE355_E_SHAPE = -2,     /* shape outside what the kernels support (alignment, limits) */
+    MOE355_E_WORKSPACE = -3, /* workspace missing, misaligned or too small */
+    MOE355_E_LAUNCH = -4,    /* the HIP runtime refused the launch */
+    MOE355_E_UNSUPPORTED = -5
+};
+
+enum { MOE355_DT_F32 = 0, MOE355_DT_BF16 = 1, MOE355_DT_F16 = 2 };
+
+/* layouts accepted by moe355_format_cast_nz */
+enum {
+    MOE355_W_ENK = 0, /* [E, N, K]: one row of K per output channel (checkpoint order) */
+    MOE355_W_EKN = 1  /* [E, K, N]: the order the reference holds after its transpose
+                         (vllm_ascend/quantization/methods/w8a8_dynamic.py:346-347) */
+};
+
+/* meaning of a group list, as in the reference (vllm_ascend/ops/fused_moe/moe_mlp.py:54-83) */
+enum { MOE355_GL_CUMSUM = 0, MOE355_GL_COUNT = 1 };
+
+int moe355_abi_version(void);
+const char *moe355_strerror(int code);
+
+/* ---------------------------------------------------------------------------
+ * Per-token dynamic int8 quantisation.
+ * Stands in for torch_npu.npu_dynamic_quant as called from
+ * vllm_ascend/device/device_op.py:192-206 (moe_mlp.py:237-242) and the shared
+ * expert (vllm_ascend/ops/fused_moe/shared_experts.py:258).
+ *   a = max|row| ; scale = a/127 ; q = clamp(rint(v/scale), -128, 127) ; a == 0 -> q = 0, scale = 0
+ * x [rows, cols] bf16 -> q [rows, cols] int8, scale [rows] fp32.
+ */
+int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q, float *scale,
+                         void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Group-limited top-k gating.
+ * Stands in for aclnnMoeGatingTopK behind torch.ops._C_ascend.moe_gating_top_k
+ * (csrc/moe/moe_gating_top_k/moe_gating_top_k_torch_adpt.h:19-71, schema
+ * csrc/torch_binding.cpp:2135-2150).  Argument meaning is the reference's:
+ * norm_type 0 softmax / 1 sigmoid; group_select_mode 0 max / 1 sum of top-2;
+ * bias is used for selection only; renorm or sigmoid divides by (sum + eps).
+ * x [rows, E] (x_dtype), bias [E] (x_dtype) or NULL ->
+ * y [rows, k] (x_dtype), expert_idx [rows, k] int32, out [rows, E] fp32
+ * (written only when out_flag != 0; may be NULL otherwise).
+ * Limits: E <= 2048, k <= 64, group_count <= 64.
+ */
+int moe355_gating_top_k(const void *x, int x_dtype, const void *bias, int64_t rows, int64_t num_experts, int k,
+                        int k_group, int group_count, int group_select_mode, int renorm, int norm_type, int out_flag,
+                        float routed_scaling_factor, float eps, void *y, int32_t *expert_idx, float *out,
+                        void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Expert histogram + stable counting sort of the flattened [T*k] expert ids +
+ * token gather with fused per-row int8 quantisation.
+ * Stands in for torch_npu.npu_moe_init_routing_v2 as called from
+ * vllm_ascend/device/device_op.py:103-127 (token_dispatcher.py:424-435):
+ *   expanded_row_idx[t*k+j] = row of pair (t, j) in the expert-sorted array,
+ *   the sort being stable in the flat index (vllm_ascend/lora/fused_moe.py:190-204).
+ * quant_mode 1: expanded_x is int8 [R, H] and dynamic_scale [R] fp32 is written;
+ * quant_mode -1: expanded_x is a bf16 [R, H] copy and dynamic_scale is ignored.
+ * expert_tokens [E] int64: per-expert counts (tokens_num_type 1) or their
+ * running sum (tokens_num_type 0).
+ * x [T, H] bf16, expert_idx [T, k] int32 in [0, E).  Ids outside the range are
+ * dropped (their expanded_row_idx is -1).  R = T*k must be < 2^31.
+ */
+size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, int num_experts);
+int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t hidden, const int32_t *expert_idx,
+                        int top_k, int num_experts, int quant_mode, int tokens_num_type, void *expanded_x,
+                        int32_t *expanded_row_idx, int64_t *expert_tokens, float *dynamic_scale, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Weight format cast: dense int8 weights -> the MFMA-tiled storage the grouped
+ * GEMMs stream ("NZ" of this build).  Stands in for
+ * torch_npu.npu_format_cast(w, ACL_FORMAT_FRACTAL_NZ) in
+ * vllm_ascend/quantization/methods/w8a8_dynamic.py:350-351.
+ * Tiled storage: [E][N/32][K/32][64][16] bytes; inside a 1 KiB tile, entry
+ * (lane, b) holds w[e, 32*nb + lane%32, 32*kb + 16*(lane/32) + b].
+ * N and K must be multiples of 32.  out has E*N*K bytes and must not alias w.
+ */
+int moe355_format_cast_nz(const int8_t *w, int layout, int64_t num_experts, int64_t n, int64_t k, int8_t *out,
+                          void *stream);
+
+/* int4 variant: w holds two 4-bit two's-complement values per byte along N
+ * (low nibble = even channel; vllm_ascend/quantization/methods/w4a8.py:327-336),
+ * logical [E, K, N] stored as [E, K, N/2] bytes.  out: tiled int4 storage
+ * [E][N/32][K/64][64][16] bytes; entry (lane, b) holds the pair
+ * k = 64*kb + 32*(lane/32) + 2*b (low nibble) and k+1 (high nibble) of channel 32*nb + lane%32. */
+int moe355_format_cast_nz_int4(const uint8_t *w_packed, int64_t num_experts, int64_t n, int64_t k, uint8_t *out,
+                               void *stream);
+
+/* ---------------------------------------------------------------------------
+ * gate_up grouped GEMM (int8 x int8 -> int32) + dequant + SwiGLU + per-row int8
+ * re-quantisation.
+ * Stands in for aclnnGroupedMatmulSwigluQuantWeightNZ behind
+ * torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz
+ * (csrc/gmm/grouped_matmul_swiglu_quant_weight_nz_tensor_list/grouped_matmul_swiglu_quant_torch_adpt.h:20-51,
+ * schema csrc/torch_binding.cpp:2025-2037; math
+ * csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:370-522):
+ *   f = (float(acc) * x_scale[row]) * weight_scale[e, col]
+ *   y = silu(f[:, :N/2]) * f[:, N/2:] ; out_scale = max|y|/127 ; out = rint(y * (1/out_scale))
+ * x [R, K] int8; weight: tiled storage of [E, N, K] (moe355_format_cast_nz);
+ * weight_scale [E, N] fp32; x_scale [R] fp32; group_list [E] int64
+ * (group_list_type MOE355_GL_*); out [R, N/2] int8; out_scale [R] fp32.
+ * Rows at or beyond the last cumulative count are left untouched.
+ * swiglu_limit > 0 clamps gate to <= L and up to [-L, L].
+ * Limits: N % 64 == 0, K % 32 == 0.
+ */
+size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts);
+int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const float *weight_scale,
+                             const float *x_scale, const int64_t *group_list, int group_list_type, int64_t rows,
+                             int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
+                             float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
+
+/* W4A8 variant: int4 weights (moe355_format_cast_nz_int4 storage), fp32 scales
+ * per group of `group_size` along K: weight_scale [E, K/group_size, N]
+ * (group_size == K gives per-channel scales [E, 1, N]).
+ *   f = (sum_g float(acc_g) * weight_scale[e, g, col]) * x_scale[row]   (g ascending)
+ * Stands in for torch.ops._C_ascend.grouped_matmul_swiglu_quant with int4
+ * weights / grouped_matmul_swiglu_quant_v2 (csrc/torch_binding.cpp:2047-2053;
+ * golden tests/e2e/nightly/single_node/ops/singlecard_ops/test_grouped_matmul_swiglu_quant.py:22-109).
+ * bias [E, N] fp32 or NULL is added to f before the token scale. */
+int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *weight_scale,
+                                int64_t group_size, const float *bias, const float *x_scale,
+                                const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
+                                int num_experts, float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * down grouped GEMM (int8 x int8 -> int32) + dequant to bf16.
+ * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,
+ * group_type=0, split_item=2) as called from vllm_ascend/device/device_op.py:254-291:
+ *   out[row, col] = bf16( (float(acc) * per_token_scale[row]) * scale[e, col] )
+ * x [R, K] int8; weight tiled [E, N, K]; scale [E, N] fp32; out [R, N] bf16.
+ */
+size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts);
+int moe355_gmm2_dequant(const int8_t *x, const int8_t *weight_nz, const float *scale, const float *per_token_scale,
+                        const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
+                        int num_experts, void *out, int out_dtype, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
+/* W4A8 down projection (same scale convention as moe355_gmm1_swiglu_quant_w4). */
+int moe355_gmm2_dequant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *scale, int64_t group_size,
+                           const float *bias, const float *per_token_scale, const int64_t *group_list,
+                           int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, void *out,
+                           int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Raw int32 accumulators of the same grouped product (no epilogue):
+ * acc [R, N] int32.  The integer stage of both ops above, exposed so a caller
+ * can check it exactly (the reference keeps the same intermediate in a global
+ * workspace: grouped_matmul_swiglu_quant.h:119,234-265). */
+int moe355_gmm_i32(const int8_t *x, const int8_t *weight_nz, const int64_t *group_list, int group_list_type,
+                   int64_t rows, int64_t k, int64_t n, int num_experts, int32_t *acc, void *workspace,
+                   size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * int32 -> dequant -> SwiGLU -> dynamic int8 (the split-path twin of the fused
+ * epilogue).  Stands in for torch.ops._C_ascend.npu_dequant_swiglu_quant
+ * (schema csrc/torch_binding.cpp:2495-2512) with quant_mode = 1 (dynamic):
+ *   f = (float(x) * weight_scale[col]) * activation_scale[row]   (weight scale first:
+ *   csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant_dynamic_base.hpp:423-426)
+ * x [rows, N] int32; weight_scale [N] fp32; activation_scale [rows] fp32;
+ * y [rows, N/2] int8; scale [rows] fp32.  activate_left != 0: SiLU on the left half.
+ */
+int moe355_dequant_swiglu_quant(const int32_t *x, const float *weight_scale, const float *activation_scale,
+                                int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t *y,
+                                float *scale, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Weighted un-permute (finalize routing).
+ * Stands in for torch_npu.npu_moe_token_unpermute as called from
+ * vllm_ascend/device/device_op.py:950-954 (token_dispatcher.py:451-461; math
+ * csrc/mc2/dispatch_ffn_combine/op_kernel/unpermute/moe_token_unpermute.h:241-372):
+ *   out[t, :] = bf16( sum_{j=0..k-1, slot order} float(probs[t, j]) * float(permuted[|idx[t*k+j]|, :]) )
+ * permuted [R, H] bf16; sorted_indices [T*k] int32; probs [T, k] bf16 or NULL
+ * (NULL = weight 1); residual [T, H] bf16 or NULL is added last in fp32
+ * (the shared-expert output; the reference adds it in upstream vLLM).
+ */
+int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorted_indices, const void *probs,
+                           int64_t num_tokens, int top_k, int64_t hidden, int64_t permuted_rows,
+                           const void *residual, void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE355_H */

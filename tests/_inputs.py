@@ -1,0 +1,77 @@
+"""Seeded synthetic inputs for the configured MoE-layer shapes (generated on the CPU so
+the CPU checker and the GPU kernels see identical bits)."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+
+@dataclass
+class LayerCfg:
+    name: str
+    T: int
+    H: int
+    E: int
+    k: int
+    I: int
+    scoring: str = "softmax"  # or "sigmoid"
+    n_group: int = 1
+    topk_group: int = 1
+    renorm: int = 1
+    routed_scaling_factor: float = 1.0
+    bias: bool = False
+    shared: bool = False
+
+
+CONFIGS = {
+    # BASELINE configs (full sizes) and reduced variants for CPU-checkable parity
+    "c1_tiny": LayerCfg("c1_tiny", 64, 1024, 8, 2, 1408),
+    "c2_qwen3_decode": LayerCfg("c2_qwen3_decode", 64, 2048, 128, 8, 768),
+    "c3_qwen3_prefill": LayerCfg("c3_qwen3_prefill", 8192, 2048, 128, 8, 768),
+    "c4_dsv3_prefill": LayerCfg("c4_dsv3_prefill", 4096, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8,
+                                topk_group=4, routed_scaling_factor=2.5, bias=True, shared=True),
+    # reduced shapes with the same structure
+    "c2_small": LayerCfg("c2_small", 48, 512, 32, 4, 256),
+    "c3_small": LayerCfg("c3_small", 640, 512, 16, 4, 256),
+    "c4_small": LayerCfg("c4_small", 96, 512, 64, 8, 192, scoring="sigmoid", n_group=8, topk_group=4,
+                         routed_scaling_factor=2.5, bias=True, shared=True),
+}
+
+
+def make_layer(cfg: LayerCfg, seed: int = 0, device: str = "cpu"):
+    """Returns a dict of torch CPU tensors: x bf16, logits fp32, w13 int8 [E,2I,H], s13 fp32 [E,2I],
+    w2 int8 [E,H,I], s2 fp32 [E,H], optional bias fp32 [E] and shared-expert weights."""
+    g = torch.Generator().manual_seed(seed)
+    d = {}
+    d["x"] = torch.randn(cfg.T, cfg.H, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    d["logits"] = torch.randn(cfg.T, cfg.E, generator=g, dtype=torch.float32)
+    d["w13"] = torch.randint(-127, 128, (cfg.E, 2 * cfg.I, cfg.H), generator=g, dtype=torch.int8)
+    d["w2"] = torch.randint(-127, 128, (cfg.E, cfg.H, cfg.I), generator=g, dtype=torch.int8)
+    d["s13"] = torch.rand(cfg.E, 2 * cfg.I, generator=g, dtype=torch.float32) * 0.009 + 0.001
+    d["s2"] = torch.rand(cfg.E, cfg.H, generator=g, dtype=torch.float32) * 0.009 + 0.001
+    if cfg.bias:
+        d["bias"] = torch.randn(cfg.E, generator=g, dtype=torch.float32) * 0.01
+    if cfg.shared:
+        d["sw13"] = torch.randint(-127, 128, (1, 2 * cfg.I, cfg.H), generator=g, dtype=torch.int8)
+        d["sw2"] = torch.randint(-127, 128, (1, cfg.H, cfg.I), generator=g, dtype=torch.int8)
+        d["ss13"] = torch.rand(1, 2 * cfg.I, generator=g, dtype=torch.float32) * 0.009 + 0.001
+        d["ss2"] = torch.rand(1, cfg.H, generator=g, dtype=torch.float32) * 0.009 + 0.001
+    if device != "cpu":
+        d = {k: v.to(device) for k, v in d.items()}
+    return d
+
+
+def gating_kwargs(cfg: LayerCfg) -> dict:
+    return dict(k=cfg.k, k_group=cfg.topk_group, group_count=cfg.n_group, group_select_mode=1, renorm=cfg.renorm,
+                norm_type=0 if cfg.scoring == "softmax" else 1, routed_scaling_factor=cfg.routed_scaling_factor,
+                eps=1e-20)
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    """torch tensor -> numpy, 16-bit floats as raw uint16."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()

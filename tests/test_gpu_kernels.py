@@ -1,0 +1,232 @@
+"""GPU parity: every entry point of libmoe355.so against the CPU checker, bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from _inputs import CONFIGS, bits, gating_kwargs, make_layer
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from vllm_ascend_amd import kernels
+
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import oracle
+
+    return oracle
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (3, 1024), (64, 2048), (17, 7168), (5, 200), (2, 30)])
+def test_dynamic_quant(K, orc, rows, cols):
+    print(f"dynamic_quant rows={rows} cols={cols}", flush=True)
+    g = torch.Generator().manual_seed(rows * 1000 + cols)
+    x = torch.randn(rows, cols, generator=g).to(torch.bfloat16)
+    x[0, :] = 0  # an all-zero row
+    q, s = K.dynamic_quant(x.to(DEV))
+    torch.cuda.synchronize()
+    qo, so = orc.dynamic_quant(bits(x))
+    assert np.array_equal(q.cpu().numpy(), qo)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+GATING_CASES = [
+    # (T, E, k, k_group, G, mode, renorm, norm_type, rsf, bias, dtype)
+    (64, 128, 8, 1, 1, 1, 1, 0, 1.0, False, torch.float32),
+    (64, 8, 2, 1, 1, 1, 1, 0, 1.0, False, torch.float32),
+    (33, 256, 8, 4, 8, 1, 0, 1, 2.5, True, torch.float32),
+    (33, 256, 8, 4, 8, 0, 1, 1, 2.5, True, torch.float32),
+    (16, 64, 4, 1, 8, 1, 1, 0, 1.0, True, torch.float32),
+    (16, 256, 32, 1, 8, 0, 1, 1, 1.0, True, torch.float32),
+    (7, 128, 16, 2, 4, 1, 1, 0, 1.0, False, torch.bfloat16),
+    (7, 128, 16, 2, 4, 1, 1, 1, 1.0, True, torch.float16),
+    (5, 384, 6, 3, 6, 1, 1, 1, 1.0, True, torch.float32),
+    (3, 2048, 8, 1, 1, 1, 1, 0, 1.0, False, torch.float32),
+    (4097, 128, 8, 1, 1, 1, 1, 0, 1.0, False, torch.float32),
+]
+
+
+@pytest.mark.parametrize("case", GATING_CASES, ids=[str(i) for i in range(len(GATING_CASES))])
+def test_gating_top_k(K, orc, case):
+    T, E, k, k_group, G, mode, renorm, norm_type, rsf, use_bias, dtype = case
+    print(f"gating {case}", flush=True)
+    g = torch.Generator().manual_seed(45)
+    x = (torch.rand(T, E, generator=g) * 4 - 2).to(dtype)
+    bias = (torch.rand(E, generator=g) * 4 - 2).to(dtype) if use_bias else None
+    y, idx, out = K.gating_top_k(x.to(DEV), k, k_group, G, mode, renorm, norm_type, True, rsf, 1e-20,
+                                 bias.to(DEV) if use_bias else None)
+    torch.cuda.synchronize()
+    name = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[dtype]
+    yo, io, no = orc.gating_top_k(bits(x), k, bias=bits(bias) if use_bias else None, k_group=k_group, group_count=G,
+                                  group_select_mode=mode, renorm=renorm, norm_type=norm_type,
+                                  routed_scaling_factor=rsf, eps=1e-20, x_dtype=name, want_norm=True)
+    assert np.array_equal(idx.cpu().numpy(), io)
+    assert np.array_equal(bits(y).view(np.uint16 if dtype != torch.float32 else np.uint32),
+                          yo.view(np.uint16 if dtype != torch.float32 else np.uint32))
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), no.view(np.uint32))
+
+
+@pytest.mark.parametrize("T,k,E,H", [(3, 2, 2, 64), (64, 8, 128, 2048), (1, 1, 8, 64), (700, 8, 256, 512),
+                                     (2000, 4, 16, 128), (40, 6, 2048, 64)])
+@pytest.mark.parametrize("quant", [True, False])
+def test_init_routing(K, orc, T, k, E, H, quant):
+    print(f"init_routing T={T} k={k} E={E} H={H} quant={quant}", flush=True)
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    # distinct experts per token, like a real top-k
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    xs, dst, cnt, sx = K.init_routing(x.to(DEV), ids.to(DEV), E, 1 if quant else -1, 1)
+    torch.cuda.synchronize()
+    xo, do, co, so = orc.init_routing(bits(x), ids.numpy(), E, quant=quant)
+    assert np.array_equal(dst.cpu().numpy(), do)
+    assert np.array_equal(cnt.cpu().numpy(), co)
+    assert np.array_equal(bits(xs), xo)
+    if quant:
+        assert np.array_equal(sx.cpu().numpy().view(np.uint32), so.view(np.uint32))
+    # cumulative form of the token counts
+    _, _, cum, _ = K.init_routing(x.to(DEV), ids.to(DEV), E, 1 if quant else -1, 0)
+    assert np.array_equal(cum.cpu().numpy(), np.cumsum(co))
+
+
+def test_init_routing_known_answer(K):
+    """Permutation known-answer vector of the reference (tests/ut/lora/test_lora.py:151-165)."""
+    ids = torch.tensor([[1, 0], [0, 1], [1, 1]], dtype=torch.int32)
+    x = torch.zeros(3, 64, dtype=torch.bfloat16)
+    _, dst, cnt, _ = K.init_routing(x.to(DEV), ids.to(DEV), 2, 1, 1)
+    assert dst.cpu().tolist() == [2, 0, 1, 3, 4, 5]
+    assert cnt.cpu().tolist() == [2, 4]
+
+
+def _rand_groups(g, E, R, empty_some=True):
+    w = torch.rand(E, generator=g)
+    if empty_some and E > 2:
+        w[torch.randperm(E, generator=g)[: E // 4]] = 0
+    cnt = torch.floor(w / w.sum() * R).to(torch.int64)
+    cnt[int(torch.argmax(w))] += R - int(cnt.sum())
+    return cnt
+
+
+GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100, 16, 768, 2048),
+             (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256)]
+
+
+@pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
+@pytest.mark.parametrize("layout", ["enk", "ekn"])
+def test_gmm_i32(K, orc, R, E, Kd, N, layout):
+    print(f"gmm_i32 R={R} E={E} K={Kd} N={N} {layout}", flush=True)
+    from vllm_ascend_amd._lib import W_EKN, W_ENK
+
+    g = torch.Generator().manual_seed(R + E + Kd)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    cnt = _rand_groups(g, E, R)
+    cum = torch.cumsum(cnt, 0)
+    if layout == "enk":
+        wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    else:
+        wnz = K.format_cast_nz(w.transpose(1, 2).contiguous().to(DEV), W_EKN)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    acc = K.gmm_i32(x.to(DEV), wnz, cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    acc2 = K.gmm_i32(x.to(DEV), wnz, cnt.to(DEV), 1, N, Kd)
+    assert np.array_equal(acc2.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
+def test_gmm1_swiglu_quant(K, orc, R, E, Kd, N):
+    print(f"gmm1 R={R} E={E} K={Kd} N={N}", flush=True)
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(R + E + Kd + 1)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    cnt = _rand_groups(g, E, R)
+    covered = int(cnt.sum())
+    cum = torch.cumsum(cnt, 0)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    q = torch.full((R, N // 2), 77, dtype=torch.int8, device=DEV)
+    qs = torch.full((R,), -1.0, dtype=torch.float32, device=DEV)
+    K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd, out=q, out_scale=qs)
+    torch.cuda.synchronize()
+    acc = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    f = orc.dequant_acc(acc, sx.numpy(), sw.numpy(), cum.numpy())
+    qo, so = orc.swiglu_quant(f)
+    assert covered == R
+    assert np.array_equal(q.cpu().numpy(), qo)
+    assert np.array_equal(qs.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+def test_gmm1_rows_beyond_groups_untouched(K):
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(3)
+    R, E, Kd, N = 40, 4, 64, 128
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    cum = torch.tensor([5, 5, 20, 33], dtype=torch.int64)
+    q = torch.full((R, N // 2), 77, dtype=torch.int8, device=DEV)
+    qs = torch.full((R,), -1.0, dtype=torch.float32, device=DEV)
+    K.gmm1_swiglu_quant(x.to(DEV), K.format_cast_nz(w.to(DEV), W_ENK), torch.ones(E, N, device=DEV),
+                        torch.ones(R, device=DEV), cum.to(DEV), 0, N, Kd, out=q, out_scale=qs)
+    assert bool((q[33:] == 77).all()) and bool((qs[33:] == -1.0).all())
+    assert bool((qs[:33] >= 0).all())
+
+
+@pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
+def test_gmm2_dequant(K, orc, R, E, Kd, N):
+    print(f"gmm2 R={R} E={E} K={Kd} N={N}", flush=True)
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(R + E + Kd + 2)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    cnt = _rand_groups(g, E, R)
+    cum = torch.cumsum(cnt, 0)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    o = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt.to(DEV), 1, N, Kd)
+    torch.cuda.synchronize()
+    acc = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    oo = orc.gmm2_dequant(acc, sx.numpy(), sw.numpy(), cum.numpy())
+    assert np.array_equal(bits(o), oo)
+
+
+@pytest.mark.parametrize("T,k,H", [(64, 8, 2048), (5, 2, 1024), (33, 1, 64), (100, 8, 7168)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_token_unpermute(K, orc, T, k, H, residual):
+    print(f"unpermute T={T} k={k} H={H} residual={residual}", flush=True)
+    g = torch.Generator().manual_seed(T + H)
+    R = T * k
+    o = torch.randn(R, H, generator=g).to(torch.bfloat16)
+    idx = torch.randperm(R, generator=g).to(torch.int32)
+    p = torch.rand(T, k, generator=g).to(torch.bfloat16)
+    res = torch.randn(T, H, generator=g).to(torch.bfloat16) if residual else None
+    out = K.token_unpermute(o.to(DEV), idx.to(DEV), p.to(DEV), res.to(DEV) if residual else None)
+    torch.cuda.synchronize()
+    ref = orc.unpermute(bits(o), idx.numpy(), bits(p), bits(res) if residual else None)
+    assert np.array_equal(bits(out), ref)
+
+
+@pytest.mark.parametrize("rows,n", [(2, 192), (4, 192), (8, 384), (1, 256), (300, 2048)])
+@pytest.mark.parametrize("left", [True, False])
+def test_dequant_swiglu_quant(K, orc, rows, n, left):
+    g = torch.Generator().manual_seed(rows + n)
+    x = torch.randint(-100, 100, (rows, n), generator=g, dtype=torch.int32)
+    ws = torch.randn(n, generator=g) * 0.1
+    a = torch.randn(rows, generator=g) * 0.5
+    y, s = K.dequant_swiglu_quant(x.to(DEV), ws.to(DEV), a.to(DEV), left, 0.0)
+    torch.cuda.synchronize()
+    yo, so = orc.dequant_swiglu_quant(x.numpy(), ws.numpy(), a.numpy(), left, 0.0)
+    assert np.array_equal(y.cpu().numpy(), yo)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))

@@ -1,0 +1,86 @@
+// Weighted un-permute (finalize routing): one workgroup per token, each lane
+// owns runs of 8 hidden elements (16-byte loads), accumulating the k expert
+// rows in fp32 in slot order.
+#include "moe355_common.h"
+
+namespace moe355 {
+
+__global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __restrict__ permuted,
+                                                              const int32_t* __restrict__ idx,
+                                                              const uint16_t* __restrict__ probs, int top_k,
+                                                              int64_t H, int64_t permuted_rows,
+                                                              const uint16_t* __restrict__ residual,
+                                                              uint16_t* __restrict__ out)
+{
+    __shared__ int32_t srow[64];
+    __shared__ float sw[64];
+    const int64_t t = blockIdx.x;
+    if (threadIdx.x < top_k) {
+        int32_t d = idx[t * top_k + threadIdx.x];
+        d = d < 0 ? -d : d;
+        srow[threadIdx.x] = ((int64_t)d < permuted_rows) ? d : -1;
+        sw[threadIdx.x] = probs ? bf16_to_f32(probs[t * top_k + threadIdx.x]) : 1.0f;
+    }
+    __syncthreads();
+    const int64_t nv = H >> 3;
+    for (int64_t i = threadIdx.x; i < nv; i += 256) {
+        float acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+        for (int s = 0; s < top_k; ++s) {
+            const int32_t d = srow[s];
+            if (d < 0) continue;
+            const float w = sw[s];
+            const v8u16 v = ((const v8u16*)(permuted + (int64_t)d * H))[i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float pr = w * bf16_to_f32(v[j]);
+                acc[j] = acc[j] + pr;
+            }
+        }
+        if (residual) {
+            const v8u16 r = ((const v8u16*)(residual + t * H))[i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = acc[j] + bf16_to_f32(r[j]);
+        }
+        v8u16 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = f32_to_bf16(acc[j]);
+        ((v8u16*)(out + t * H))[i] = o;
+    }
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+extern "C" int moe355_token_unpermute(const void* permuted, int dtype, const int32_t* sorted_indices,
+                                      const void* probs, int64_t num_tokens, int top_k, int64_t hidden,
+                                      int64_t permuted_rows, const void* residual, void* out, void* stream)
+{
+    if (num_tokens < 0 || top_k <= 0 || hidden <= 0 || permuted_rows < 0) return MOE355_E_ARG;
+    if (dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (top_k > 64 || hidden % 8 != 0 || num_tokens > 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (num_tokens == 0) return MOE355_OK;
+    if (!permuted || !sorted_indices || !out) return MOE355_E_ARG;
+    if (((uintptr_t)permuted & 15) || ((uintptr_t)out & 15) || ((uintptr_t)residual & 15)) return MOE355_E_SHAPE;
+    hipLaunchKernelGGL(token_unpermute_kernel, dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,
+                       permuted_rows, (const uint16_t*)residual, (uint16_t*)out);
+    return launch_status();
+}
+
+extern "C" int moe355_abi_version(void) { return MOE355_ABI_VERSION; }
+
+extern "C" const char* moe355_strerror(int code)
+{
+    switch (code) {
+        case MOE355_OK: return "ok";
+        case MOE355_E_ARG: return "invalid argument (null pointer, negative size or unknown enum value)";
+        case MOE355_E_SHAPE: return "shape or alignment outside what the kernels support";
+        case MOE355_E_WORKSPACE: return "workspace missing, misaligned or too small";
+        case MOE355_E_LAUNCH: return "the HIP runtime refused the kernel launch";
+        case MOE355_E_UNSUPPORTED: return "option not supported by this build";
+        default: return "unknown error code";
+    }
+}

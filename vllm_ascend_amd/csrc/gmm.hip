@@ -1,0 +1,326 @@
+// Grouped int8 x int8 -> int32 GEMM for the expert MLPs, with the three
+// epilogues (raw int32, dequant+SwiGLU, dequant to bf16), the weight format
+// cast, and the per-row re-quantisation that finishes the SwiGLU op.
+//
+// Weight-streaming kernel: few rows per expert (decode), where the time is the
+// HBM stream of the weights.  Work unit = (expert, pair of 32-channel tiles).
+// The weights of a unit are contiguous 1 KiB tiles along K and go straight from
+// HBM into MFMA operand registers with one 16-byte load per lane (no LDS: each
+// weight byte is used by exactly one wavefront).  The expert's tokens are
+// processed 32 at a time as the MFMA's second operand.  With KSPLIT = 4 the
+// four wavefronts of a workgroup split K and add their int32 partials through
+// LDS (integer addition: exact, order free).
+#include "gmm_common.h"
+
+namespace moe355 {
+
+// ------------------------------------------------------------------ format cast
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void format_cast_nz_kernel(const int8_t* __restrict__ w, int64_t E, int64_t N,
+                                                             int64_t K, int8_t* __restrict__ out)
+{
+    const int64_t total = E * N * K / 16;
+    const int64_t KB = K / 32, NB = N / 32;
+    for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+        const int lane = (int)(id & 63);
+        const int64_t tile = id >> 6;
+        const int64_t kb = tile % KB;
+        const int64_t nb = (tile / KB) % NB;
+        const int64_t e = tile / (KB * NB);
+        const int64_t n = nb * 32 + (lane & 31);
+        const int64_t k0 = kb * 32 + (lane >> 5) * 16;
+        v4i v;
+        if constexpr (LAYOUT == MOE355_W_ENK) {
+            v = *(const v4i*)(w + (e * N + n) * K + k0);
+        } else {
+            uint32_t p[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int b = 0; b < 16; ++b)
+                p[b >> 2] |= (uint32_t)(uint8_t)w[(e * K + k0 + b) * N + n] << (8 * (b & 3));
+            v = {(int)p[0], (int)p[1], (int)p[2], (int)p[3]};
+        }
+        *(v4i*)(out + id * 16) = v;
+    }
+}
+
+// ------------------------------------------------------------------ streaming GEMM
+template <int EPI, int KSPLIT, int UN>
+__global__ __launch_bounds__(256) void gmm_stream_kernel(GmmArgs a)
+{
+    static_assert(KSPLIT == 1 || KSPLIT == 4, "workgroup barriers need all four wavefronts on one unit");
+    __shared__ int32_t red[(KSPLIT > 1) ? (KSPLIT - 1) * 32 * 64 : 1];
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int NB = a.N >> 5, KB = a.K >> 5;
+    const int upe = NB >> 1;  // units per expert
+    const int64_t unit = (KSPLIT == 1) ? (int64_t)blockIdx.x * 4 + wave : (int64_t)blockIdx.x;
+    if (unit >= (int64_t)a.E * upe) return;  // KSPLIT == 1: no barriers below; KSPLIT == 4: whole workgroup leaves
+    const int e = (int)(unit / upe);
+    const int p = (int)(unit % upe);
+    const int nb0 = (EPI == EPI_SWIGLU) ? p : 2 * p;
+    const int nb1 = (EPI == EPI_SWIGLU) ? p + upe : 2 * p + 1;
+
+    int64_t row0, row1;
+    expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
+    if (row1 > a.R) row1 = a.R;
+    if (row1 <= row0) return;
+
+    const int ks = (KSPLIT == 1) ? 0 : wave;
+    const int kb_begin = (KB * ks) / KSPLIT;
+    const int kb_end = (KB * (ks + 1)) / KSPLIT;
+
+    const int8_t* w0 = a.w + (((int64_t)e * NB + nb0) * KB) * 1024 + lane * 16;
+    const int8_t* w1 = a.w + (((int64_t)e * NB + nb1) * KB) * 1024 + lane * 16;
+    const int tok = lane & 31;
+    const int kh = lane >> 5;
+
+    for (int64_t r0 = row0; r0 < row1; r0 += 32) {
+        const int64_t row = r0 + tok;
+        const bool valid = row < row1;
+        const int8_t* xr = a.x + row * a.K + kh * 16;
+        v16i c0 = {0}, c1 = {0};
+        for (int kb = kb_begin; kb < kb_end; kb += UN) {
+            v4i a0[UN], a1[UN], b[UN];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const int k = kb + u;
+                if (k < kb_end) {
+                    a0[u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
+                    a1[u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
+                    b[u] = valid ? *(const v4i*)(xr + k * 32) : (v4i){0, 0, 0, 0};
+                } else {
+                    a0[u] = (v4i){0, 0, 0, 0};
+                    a1[u] = (v4i){0, 0, 0, 0};
+                    b[u] = (v4i){0, 0, 0, 0};
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                c0 = mfma_i8(a0[u], b[u], c0);
+                c1 = mfma_i8(a1[u], b[u], c1);
+            }
+        }
+        if constexpr (KSPLIT > 1) {
+            if (wave > 0) {
+                int32_t* dstp = red + (wave - 1) * 32 * 64;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    dstp[v * 64 + lane] = c0[v];
+                    dstp[(16 + v) * 64 + lane] = c1[v];
+                }
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int s = 0; s < KSPLIT - 1; ++s) {
+                    const int32_t* srcp = red + s * 32 * 64;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        c0[v] += srcp[v * 64 + lane];
+                        c1[v] += srcp[(16 + v) * 64 + lane];
+                    }
+                }
+                epilogue_pair<EPI>(a, e, row, valid, nb0 * 32, nb1 * 32, c0, c1, lane);
+            }
+            __syncthreads();
+        } else {
+            epilogue_pair<EPI>(a, e, row, valid, nb0 * 32, nb1 * 32, c0, c1, lane);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ SwiGLU re-quantisation
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = v;
+}
+
+// One wavefront per row: y fp32 [R, I] + row absmax -> int8 + scale.
+__global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __restrict__ y,
+                                                             const uint32_t* __restrict__ rowmax, int64_t R, int I,
+                                                             int8_t* __restrict__ q, float* __restrict__ qs)
+{
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= R) return;
+    const uint32_t mb = rowmax[row];
+    if (mb == 0u) return;  // row belongs to no expert: left untouched
+    const float amax = __uint_as_float(mb - 1u);
+    const float s = amax / 127.0f;
+    const float inv = 1.0f / s;
+    if (lane == 0) qs[row] = (amax == 0.0f) ? 0.0f : s;
+    const v4f* yr = (const v4f*)(y + row * I);
+    uint32_t* qr = (uint32_t*)(q + row * I);
+    for (int i = lane; i < (I >> 2); i += 64) {
+        const v4f v = yr[i];
+        uint32_t pk = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int8_t b = (amax == 0.0f) ? (int8_t)0 : sat_rint_i8(v[j] * inv);
+            pk |= (uint32_t)(uint8_t)b << (8 * j);
+        }
+        qr[i] = pk;
+    }
+}
+
+static int check_gmm(const void* x, const void* w, const int64_t* gl, int gl_type, int64_t rows, int64_t k, int64_t n,
+                     int E)
+{
+    if (rows < 0 || k <= 0 || n <= 0 || E <= 0) return MOE355_E_ARG;
+    if (gl_type != MOE355_GL_CUMSUM && gl_type != MOE355_GL_COUNT) return MOE355_E_ARG;
+    if (n % 64 != 0 || k % 32 != 0) return MOE355_E_SHAPE;
+    if (rows >= 0x7fffffffLL || n >= 0x7fffffffLL || k >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if ((int64_t)E * (n / 64) >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (rows > 0 && (!x || !w || !gl)) return MOE355_E_ARG;
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return MOE355_E_SHAPE;
+    return MOE355_OK;
+}
+
+template <int EPI>
+static int launch_stream(const GmmArgs& a, hipStream_t st)
+{
+    const int64_t units = (int64_t)a.E * (a.N / 64);
+    // K split over the four wavefronts when one wavefront per unit would leave the chip short of work
+    const bool split = units < 8192;
+    if (split)
+        hipLaunchKernelGGL((gmm_stream_kernel<EPI, 4, 4>), dim3((unsigned)units), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((gmm_stream_kernel<EPI, 1, 4>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a);
+    return launch_status();
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+extern "C" int moe355_format_cast_nz(const int8_t* w, int layout, int64_t num_experts, int64_t n, int64_t k,
+                                     int8_t* out, void* stream)
+{
+    if (num_experts <= 0 || n <= 0 || k <= 0 || !w || !out) return MOE355_E_ARG;
+    if (layout != MOE355_W_ENK && layout != MOE355_W_EKN) return MOE355_E_ARG;
+    if (n % 32 != 0 || k % 32 != 0) return MOE355_E_SHAPE;
+    if (((uintptr_t)w & 15) || ((uintptr_t)out & 15)) return MOE355_E_SHAPE;
+    const int64_t total = num_experts * n * k / 16;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipStream_t st = (hipStream_t)stream;
+    if (layout == MOE355_W_ENK)
+        hipLaunchKernelGGL(format_cast_nz_kernel<MOE355_W_ENK>, dim3((unsigned)blocks), dim3(256), 0, st, w,
+                           num_experts, n, k, out);
+    else
+        hipLaunchKernelGGL(format_cast_nz_kernel<MOE355_W_EKN>, dim3((unsigned)blocks), dim3(256), 0, st, w,
+                           num_experts, n, k, out);
+    return launch_status();
+}
+
+extern "C" int moe355_gmm_i32(const int8_t* x, const int8_t* weight_nz, const int64_t* group_list,
+                              int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, int32_t* acc,
+                              void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
+    if (rc != MOE355_OK) return rc;
+    if (rows == 0) return MOE355_OK;
+    if (!acc || ((uintptr_t)acc & 15)) return MOE355_E_ARG;
+    GmmArgs a = {};
+    a.x = x;
+    a.w = weight_nz;
+    a.gl = group_list;
+    a.gl_type = group_list_type;
+    a.R = rows;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    a.acc = acc;
+    return launch_stream<EPI_I32>(a, (hipStream_t)stream);
+}
+
+extern "C" size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
+{
+    (void)k;
+    (void)num_experts;
+    if (rows <= 0 || n <= 0) return 256;
+    size_t ybytes = ((size_t)rows * (size_t)(n / 2) * 4 + 255) & ~(size_t)255;
+    size_t mbytes = ((size_t)rows * 4 + 255) & ~(size_t)255;
+    return ybytes + mbytes;
+}
+
+extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz, const float* weight_scale,
+                                        const float* x_scale, const int64_t* group_list, int group_list_type,
+                                        int64_t rows, int64_t k, int64_t n, int num_experts, float swiglu_limit,
+                                        int8_t* out, float* out_scale, void* workspace, size_t workspace_bytes,
+                                        void* stream)
+{
+    int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
+    if (rc != MOE355_OK) return rc;
+    if (rows == 0) return MOE355_OK;
+    if (!weight_scale || !x_scale || !out || !out_scale) return MOE355_E_ARG;
+    if (((uintptr_t)weight_scale & 15) || ((uintptr_t)out & 3)) return MOE355_E_SHAPE;
+    if (!workspace || ((uintptr_t)workspace & 255) ||
+        workspace_bytes < moe355_gmm1_swiglu_quant_workspace(rows, n, k, num_experts))
+        return MOE355_E_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const int I = (int)(n / 2);
+    float* y = (float*)workspace;
+    uint32_t* rowmax = (uint32_t*)((char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255));
+    int fb = (int)((rows + 255) / 256);
+    if (fb > 1024) fb = 1024;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(fb), dim3(256), 0, st, rowmax, rows, 0u);
+    GmmArgs a = {};
+    a.x = x;
+    a.w = weight_nz;
+    a.gl = group_list;
+    a.gl_type = group_list_type;
+    a.R = rows;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    a.row_scale = x_scale;
+    a.ch_scale = weight_scale;
+    a.limit = swiglu_limit;
+    a.y = y;
+    a.rowmax = rowmax;
+    rc = launch_stream<EPI_SWIGLU>(a, st);
+    if (rc != MOE355_OK) return rc;
+    hipLaunchKernelGGL(swiglu_requant_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, y, rowmax, rows, I,
+                       out, out_scale);
+    return launch_status();
+}
+
+extern "C" size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
+{
+    (void)rows;
+    (void)n;
+    (void)k;
+    (void)num_experts;
+    return 256;
+}
+
+extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, const float* scale,
+                                   const float* per_token_scale, const int64_t* group_list, int group_list_type,
+                                   int64_t rows, int64_t k, int64_t n, int num_experts, void* out, int out_dtype,
+                                   void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
+    if (rc != MOE355_OK) return rc;
+    if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (rows == 0) return MOE355_OK;
+    if (!scale || !per_token_scale || !out) return MOE355_E_ARG;
+    if (((uintptr_t)scale & 15) || ((uintptr_t)out & 7)) return MOE355_E_SHAPE;
+    GmmArgs a = {};
+    a.x = x;
+    a.w = weight_nz;
+    a.gl = group_list;
+    a.gl_type = group_list_type;
+    a.R = rows;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    a.row_scale = per_token_scale;
+    a.ch_scale = scale;
+    a.out = (uint16_t*)out;
+    return launch_stream<EPI_DEQUANT>(a, (hipStream_t)stream);
+}

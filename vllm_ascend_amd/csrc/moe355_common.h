@@ -1,0 +1,164 @@
+// Shared device helpers for the gfx950 MoE kernels.
+//
+// Arithmetic contract shared by every kernel: IEEE binary32, round to nearest
+// even, no fused multiply-add (the library is compiled with -ffp-contract=off),
+// one exp() built from explicit multiplies and adds.  A CPU program executing
+// the same operation sequence produces the same bits.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/moe355.h"
+
+#define MOE355_WAVE 64
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short v8u16 __attribute__((ext_vector_type(8)));
+typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
+
+namespace moe355 {
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uint(f); }
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// fp32 -> bf16, round to nearest even, NaN stays quiet NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float f16_to_f32(uint16_t h)
+{
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16(float f)
+{
+    _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+
+// exp(x): n = rint(x*log2e), two-part ln2 reduction, degree-5 polynomial,
+// result scaled by 2^n in two exact steps.  Mul/add only, no contraction.
+__device__ __forceinline__ float m_expf(float x)
+{
+    if (x != x) return x;
+    if (x > 88.72283f) return __builtin_inff();
+    if (x < -87.33654f) return 0.0f;
+    float n = __builtin_rintf(x * 1.44269504088896341f);
+    float r = x - n * 0.693359375f;
+    r = r - n * -2.12194440e-4f;
+    float p = 1.9875691500e-4f;
+    p = p * r + 1.3981999507e-3f;
+    p = p * r + 8.3334519073e-3f;
+    p = p * r + 4.1665795894e-2f;
+    p = p * r + 1.6666665459e-1f;
+    p = p * r + 5.0000001201e-1f;
+    float r2 = r * r;
+    float y = p * r2 + r;
+    y = y + 1.0f;
+    int ni = (int)n;
+    int n1 = ni / 2;
+    int n2 = ni - n1;
+    float s1 = __uint_as_float((uint32_t)(n1 + 127) << 23);
+    float s2 = __uint_as_float((uint32_t)(n2 + 127) << 23);
+    return (y * s1) * s2;
+}
+
+__device__ __forceinline__ float m_silu(float g) { return g / (1.0f + m_expf(-g)); }
+
+// clamp(rint(v), -128, 127) as int8
+__device__ __forceinline__ int8_t sat_rint_i8(float v)
+{
+    float r = __builtin_rintf(v);
+    r = r > 127.0f ? 127.0f : r;
+    r = r < -128.0f ? -128.0f : r;
+    return (int8_t)(int)r;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        float o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// Butterfly sum: after the loop every lane holds the same value; the order of
+// additions is part of the arithmetic contract (partial[l] + partial[l ^ off]).
+__device__ __forceinline__ float wave_tree_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum_i32(int v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// "a ranks before b": larger value first, ties to the lower index.
+__device__ __forceinline__ bool ranks_before(float va, int ia, float vb, int ib)
+{
+    if (va > vb) return true;
+    if (va < vb) return false;
+    return ia < ib;
+}
+
+template <int DT>
+__device__ __forceinline__ float load_as_f32(const void* p, int64_t i)
+{
+    if constexpr (DT == MOE355_DT_F32) return ((const float*)p)[i];
+    if constexpr (DT == MOE355_DT_BF16) return bf16_to_f32(((const uint16_t*)p)[i]);
+    return f16_to_f32(((const uint16_t*)p)[i]);
+}
+
+template <int DT>
+__device__ __forceinline__ void store_from_f32(void* p, int64_t i, float v)
+{
+    if constexpr (DT == MOE355_DT_F32) ((float*)p)[i] = v;
+    else if constexpr (DT == MOE355_DT_BF16) ((uint16_t*)p)[i] = f32_to_bf16(v);
+    else ((uint16_t*)p)[i] = f32_to_f16(v);
+}
+
+// Row range [row0, row1) of expert e from a group list held as counts or as a
+// running sum.  Called by one full wave; every lane returns the same pair.
+__device__ __forceinline__ void expert_rows(const int64_t* gl, int gl_type, int e, int lane, int64_t& row0,
+                                            int64_t& row1)
+{
+    if (gl_type == MOE355_GL_CUMSUM) {
+        row0 = e > 0 ? gl[e - 1] : 0;
+        row1 = gl[e];
+    } else {
+        int s = 0;
+        for (int i = lane; i < e; i += 64) s += (int)gl[i];
+        s = wave_sum_i32(s);
+        row0 = s;
+        row1 = s + gl[e];
+    }
+}
+
+inline int launch_status()
+{
+    return hipGetLastError() == hipSuccess ? MOE355_OK : MOE355_E_LAUNCH;
+}
+
+}  // namespace moe355

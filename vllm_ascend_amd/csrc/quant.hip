@@ -1,0 +1,152 @@
+// Per-token dynamic int8 quantisation and the int32 -> SwiGLU -> int8 split op.
+//
+// One workgroup (256 lanes = 4 wavefronts) per row.  The row absmax is reduced
+// with wavefront shuffles, then across the four wavefronts through LDS; the
+// row is read twice (the second read hits L2) in 16-byte vectors.
+#include "moe355_common.h"
+
+namespace moe355 {
+
+__device__ __forceinline__ float block_max_256(float v, float* lds4)
+{
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+    __syncthreads();
+    float m = lds4[0];
+    m = lds4[1] > m ? lds4[1] : m;
+    m = lds4[2] > m ? lds4[2] : m;
+    m = lds4[3] > m ? lds4[3] : m;
+    __syncthreads();
+    return m;
+}
+
+// x [rows, cols] bf16 -> q int8, scale fp32.  VEC: cols % 8 == 0 and 16-byte aligned rows.
+template <bool VEC>
+__global__ __launch_bounds__(256) void dynamic_quant_bf16_kernel(const uint16_t* __restrict__ x, int64_t cols,
+                                                                 int8_t* __restrict__ q, float* __restrict__ scale)
+{
+    __shared__ float lds4[4];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * cols;
+    int8_t* qr = q + row * cols;
+    float a = 0.0f;
+    if constexpr (VEC) {
+        const int64_t nv = cols >> 3;
+        const v8u16* xv = (const v8u16*)xr;
+        for (int64_t i = threadIdx.x; i < nv; i += 256) {
+            v8u16 v = xv[i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float f = __builtin_fabsf(bf16_to_f32(v[j]));
+                a = f > a ? f : a;
+            }
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < cols; i += 256) {
+            float f = __builtin_fabsf(bf16_to_f32(xr[i]));
+            a = f > a ? f : a;
+        }
+    }
+    a = block_max_256(a, lds4);
+    const float s = a / 127.0f;
+    if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
+    if constexpr (VEC) {
+        const int64_t nv = cols >> 3;
+        const v8u16* xv = (const v8u16*)xr;
+        uint2* qv = (uint2*)qr;
+        for (int64_t i = threadIdx.x; i < nv; i += 256) {
+            v8u16 v = xv[i];
+            uint32_t w[2] = {0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(v[j]) / s);
+                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+            }
+            qv[i] = make_uint2(w[0], w[1]);
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < cols; i += 256)
+            qr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(xr[i]) / s);
+    }
+}
+
+// x [rows, n] int32 -> dequant (weight scale, then activation scale) -> SwiGLU -> dynamic int8.
+__global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t* __restrict__ x,
+                                                                   const float* __restrict__ w_scale,
+                                                                   const float* __restrict__ a_scale, int64_t n,
+                                                                   int activate_left, float limit,
+                                                                   int8_t* __restrict__ y, float* __restrict__ scale)
+{
+    __shared__ float lds4[4];
+    const int64_t row = blockIdx.x;
+    const int64_t half = n >> 1;
+    const int32_t* xr = x + row * n;
+    const float as = a_scale[row];
+    const int64_t goff = activate_left ? 0 : half;
+    const int64_t uoff = activate_left ? half : 0;
+    float a = 0.0f;
+    for (int64_t i = threadIdx.x; i < half; i += 256) {
+        float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
+        float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
+        if (limit > 0.0f) {
+            g = g > limit ? limit : g;
+            u = u > limit ? limit : u;
+            u = u < -limit ? -limit : u;
+        }
+        float v = __builtin_fabsf(m_silu(g) * u);
+        a = v > a ? v : a;
+    }
+    a = block_max_256(a, lds4);
+    const float s = a / 127.0f;
+    const float inv = 1.0f / s;
+    if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
+    int8_t* yr = y + row * half;
+    for (int64_t i = threadIdx.x; i < half; i += 256) {
+        float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
+        float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
+        if (limit > 0.0f) {
+            g = g > limit ? limit : g;
+            u = u > limit ? limit : u;
+            u = u < -limit ? -limit : u;
+        }
+        float v = m_silu(g) * u;
+        yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(v * inv);
+    }
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q, float* scale,
+                                    void* stream)
+{
+    if (rows < 0 || cols <= 0) return MOE355_E_ARG;
+    if (rows == 0) return MOE355_OK;
+    if (!x || !q || !scale) return MOE355_E_ARG;
+    if (x_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = (cols % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)q & 7) == 0);
+    if (vec)
+        hipLaunchKernelGGL(dynamic_quant_bf16_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st,
+                           (const uint16_t*)x, cols, q, scale);
+    else
+        hipLaunchKernelGGL(dynamic_quant_bf16_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st,
+                           (const uint16_t*)x, cols, q, scale);
+    return launch_status();
+}
+
+extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight_scale, const float* activation_scale,
+                                           int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t* y,
+                                           float* scale, void* stream)
+{
+    if (rows < 0 || n <= 0 || (n & 1)) return MOE355_E_ARG;
+    if (rows == 0) return MOE355_OK;
+    if (!x || !weight_scale || !activation_scale || !y || !scale) return MOE355_E_ARG;
+    if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
+    hipLaunchKernelGGL(dequant_swiglu_quant_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
+                       weight_scale, activation_scale, n, activate_left, clamp_limit, y, scale);
+    return launch_status();
+}

@@ -1,0 +1,252 @@
+// Token dispatch: expert histogram, prefix-scan offsets, stable counting-sort
+// permutation of the flattened (token, slot) pairs, and the token gather with
+// fused per-row int8 quantisation.
+//
+// The flat index space [0, R) is cut into chunks of 1024.  Stability needs
+//   dst[f] = off[e] + #{f' < f : ids[f'] == e},
+// which is built in three launches:
+//   1. per-chunk expert histograms (LDS atomics; counts are order independent);
+//   2. one workgroup turns them into per-(chunk, expert) start rows and the
+//      per-expert offsets (exclusive scans);
+//   3. one wavefront per chunk walks its 1024 indices in order, 64 at a time:
+//      lanes with equal expert ids find each other with ballots, rank
+//      themselves by lane number, and the lowest lane advances the running
+//      per-expert cursor kept in LDS.
+// A fourth launch quantises every token row once and writes it to its k
+// destination rows.
+#include "moe355_common.h"
+
+namespace moe355 {
+
+constexpr int kChunk = 1024;
+
+struct RouteWs {
+    int32_t* chunk_hist;  // [nchunks][E]   histogram, then start row of (chunk, expert)
+    int32_t* off;         // [E + 1]        first row of each expert
+};
+
+__host__ __device__ inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+__global__ __launch_bounds__(256) void route_hist_kernel(const int32_t* __restrict__ ids, int64_t R, int E,
+                                                         int32_t* __restrict__ chunk_hist)
+{
+    extern __shared__ int32_t hist[];  // [E]
+    for (int e = threadIdx.x; e < E; e += 256) hist[e] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kChunk;
+    for (int i = threadIdx.x; i < kChunk; i += 256) {
+        int64_t f = base + i;
+        if (f < R) {
+            int e = ids[f];
+            if (e >= 0 && e < E) atomicAdd(&hist[e], 1);
+        }
+    }
+    __syncthreads();
+    int32_t* dstp = chunk_hist + (int64_t)blockIdx.x * E;
+    for (int e = threadIdx.x; e < E; e += 256) dstp[e] = hist[e];
+}
+
+// One workgroup of 256.  Thread t owns experts [t*seg, (t+1)*seg).
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E,
+                                                         int tokens_num_type, int32_t* __restrict__ off,
+                                                         int64_t* __restrict__ expert_tokens)
+{
+    extern __shared__ int32_t cnt[];  // [E] counts, then [256] partials
+    int32_t* partial = cnt + E;
+    // column scan over chunks: chunk_hist[c][e] <- number of rows of expert e in chunks before c
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int32_t run = 0;
+        for (int c = 0; c < nchunks; ++c) {
+            int32_t v = chunk_hist[(int64_t)c * E + e];
+            chunk_hist[(int64_t)c * E + e] = run;
+            run += v;
+        }
+        cnt[e] = run;
+    }
+    __syncthreads();
+    const int seg = (E + 255) / 256;
+    const int e0 = threadIdx.x * seg;
+    int32_t s = 0;
+    for (int j = 0; j < seg; ++j)
+        if (e0 + j < E) s += cnt[e0 + j];
+    partial[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t run = 0;
+        for (int t = 0; t < 256; ++t) {
+            int32_t v = partial[t];
+            partial[t] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    int32_t run = partial[threadIdx.x];
+    for (int j = 0; j < seg; ++j) {
+        int e = e0 + j;
+        if (e < E) {
+            off[e] = run;
+            run += cnt[e];
+            expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
+            if (e == E - 1) off[E] = run;
+        }
+    }
+}
+
+// One wavefront per chunk.
+__global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __restrict__ ids, int64_t R, int E,
+                                                           int nbits, const int32_t* __restrict__ chunk_start,
+                                                           const int32_t* __restrict__ off,
+                                                           int32_t* __restrict__ dst)
+{
+    extern __shared__ int32_t cursor[];  // [E] next free row of each expert for this chunk
+    const int lane = threadIdx.x;
+    const int32_t* cs = chunk_start + (int64_t)blockIdx.x * E;
+    for (int e = lane; e < E; e += 64) cursor[e] = off[e] + cs[e];
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kChunk;
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int it = 0; it < kChunk / 64; ++it) {
+        const int64_t f = base + it * 64 + lane;
+        int e = -1;
+        if (f < R) {
+            e = ids[f];
+            if (e < 0 || e >= E) e = -1;
+        }
+        const bool valid = e >= 0;
+        unsigned long long same = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (e >> b) & 1;
+            unsigned long long bal = __ballot(valid && bit);
+            same &= bit ? bal : ~bal;
+        }
+        int32_t start = 0;
+        if (valid) {
+            const int rank = __popcll(same & below);
+            const int leader = __ffsll((long long)same) - 1;
+            if (lane == leader) {
+                start = cursor[e];
+                cursor[e] = start + __popcll(same);
+            }
+            start = __shfl(start, leader, 64);
+            dst[f] = start + rank;
+        } else if (f < R) {
+            dst[f] = -1;
+        }
+        __syncthreads();
+    }
+}
+
+// One workgroup per token: quantise the row once, write it to its k destinations.
+template <bool QUANT>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
+                                                          const int32_t* __restrict__ dst, void* __restrict__ xs,
+                                                          float* __restrict__ sx)
+{
+    __shared__ float lds4[4];
+    __shared__ int32_t drow[64];
+    const int64_t t = blockIdx.x;
+    const uint16_t* xr = x + t * H;
+    if (threadIdx.x < top_k) drow[threadIdx.x] = dst[t * top_k + threadIdx.x];
+    const int64_t nv = H >> 3;
+    const v8u16* xv = (const v8u16*)xr;
+    if constexpr (!QUANT) {
+        __syncthreads();
+        for (int64_t i = threadIdx.x; i < nv; i += 256) {
+            v8u16 v = xv[i];
+            for (int j = 0; j < top_k; ++j)
+                if (drow[j] >= 0) ((v8u16*)((uint16_t*)xs + (int64_t)drow[j] * H))[i] = v;
+        }
+        return;
+    } else {
+        float a = 0.0f;
+        for (int64_t i = threadIdx.x; i < nv; i += 256) {
+            v8u16 v = xv[i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float f = __builtin_fabsf(bf16_to_f32(v[j]));
+                a = f > a ? f : a;
+            }
+        }
+        a = wave_max(a);
+        if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = a;
+        __syncthreads();
+        a = lds4[0];
+        a = lds4[1] > a ? lds4[1] : a;
+        a = lds4[2] > a ? lds4[2] : a;
+        a = lds4[3] > a ? lds4[3] : a;
+        const float s = a / 127.0f;
+        if (threadIdx.x < top_k && drow[threadIdx.x] >= 0) sx[drow[threadIdx.x]] = (a == 0.0f) ? 0.0f : s;
+        for (int64_t i = threadIdx.x; i < nv; i += 256) {
+            v8u16 v = xv[i];
+            uint32_t w[2] = {0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(v[j]) / s);
+                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+            }
+            const uint2 pk = make_uint2(w[0], w[1]);
+            for (int j = 0; j < top_k; ++j)
+                if (drow[j] >= 0) ((uint2*)((int8_t*)xs + (int64_t)drow[j] * H))[i] = pk;
+        }
+    }
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+static int nchunks_of(int64_t R) { return (int)((R + kChunk - 1) / kChunk); }
+
+extern "C" size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, int num_experts)
+{
+    if (num_tokens < 0 || top_k <= 0 || num_experts <= 0) return 0;
+    const int64_t R = num_tokens * top_k;
+    size_t n = nchunks_of(R > 0 ? R : 1);
+    return align256(n * (size_t)num_experts * 4) + align256(((size_t)num_experts + 1) * 4);
+}
+
+extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
+                                   const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
+                                   int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
+                                   int64_t* expert_tokens, float* dynamic_scale, void* workspace,
+                                   size_t workspace_bytes, void* stream)
+{
+    if (num_tokens < 0 || hidden <= 0 || top_k <= 0 || num_experts <= 0) return MOE355_E_ARG;
+    if (quant_mode != 1 && quant_mode != -1) return MOE355_E_UNSUPPORTED;
+    if (tokens_num_type != 0 && tokens_num_type != 1) return MOE355_E_UNSUPPORTED;
+    if (x_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (top_k > 64 || num_experts > 2048) return MOE355_E_SHAPE;
+    const int64_t R = num_tokens * top_k;
+    if (R >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (hidden % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)expanded_x & 15)) return MOE355_E_SHAPE;
+    if (!expert_tokens) return MOE355_E_ARG;
+    if (!workspace || ((uintptr_t)workspace & 255) ||
+        workspace_bytes < moe355_init_routing_workspace(num_tokens, top_k, num_experts))
+        return MOE355_E_WORKSPACE;
+    if (R > 0 && (!x || !expert_idx || !expanded_x || !expanded_row_idx)) return MOE355_E_ARG;
+    if (R > 0 && quant_mode == 1 && !dynamic_scale) return MOE355_E_ARG;
+
+    hipStream_t st = (hipStream_t)stream;
+    const int E = num_experts;
+    const int nch = nchunks_of(R > 0 ? R : 1);
+    RouteWs ws;
+    ws.chunk_hist = (int32_t*)workspace;
+    ws.off = (int32_t*)((char*)workspace + align256((size_t)nch * E * 4));
+    int nbits = 0;
+    while ((1 << nbits) < E) ++nbits;
+
+    hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E, ws.chunk_hist);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), ((size_t)E + 256) * 4, st, ws.chunk_hist, nch, E,
+                       tokens_num_type, ws.off, expert_tokens);
+    if (R > 0) {
+        hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
+                           ws.chunk_hist, ws.off, expanded_row_idx);
+        if (quant_mode == 1)
+            hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, st,
+                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+        else
+            hipLaunchKernelGGL(gather_rows_kernel<false>, dim3((unsigned)num_tokens), dim3(256), 0, st,
+                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+    }
+    return launch_status();
+}

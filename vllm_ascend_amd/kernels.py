@@ -1,0 +1,201 @@
+"""Tensor-level launchers: allocate outputs and scratch with torch, pass raw device
+pointers and the current HIP stream to the C ABI.  PyTorch is only the owner of
+device memory and streams here; all arithmetic happens in ``libmoe355.so``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import DT_BF16, DT_F16, DT_F32, GL_COUNT, GL_CUMSUM, W_EKN, W_ENK, check
+
+_DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _dev(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got device {t.device}); this path has no CPU implementation")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _dt(t: torch.Tensor, name: str) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"{name}: float16, float32 or bfloat16 tensor expected but got {t.dtype}") from None
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    # torch's caching allocator hands out 512-byte aligned blocks
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def dynamic_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 [..., H] -> (int8 [..., H], fp32 [...]) per-row absmax/127 quantisation."""
+    x = _dev(x, "x")
+    lib = _lib.load()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    check(lib.moe355_dynamic_quant(_ptr(x), _dt(x, "x"), rows, cols, _ptr(q), _ptr(s), _stream(x)),
+          "moe355_dynamic_quant")
+    return q, s
+
+
+def gating_top_k(x, k, k_group, group_count, group_select_mode, renorm, norm_type, out_flag, routed_scaling_factor,
+                 eps, bias):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows, E = x.shape
+    if bias is not None:
+        bias = _dev(bias, "bias")
+    y = torch.empty((rows, k), dtype=x.dtype, device=x.device)
+    idx = torch.empty((rows, k), dtype=torch.int32, device=x.device)
+    out = torch.empty((rows, E), dtype=torch.float32, device=x.device)
+    check(lib.moe355_gating_top_k(_ptr(x), _dt(x, "x"), _ptr(bias), rows, E, k, k_group, group_count,
+                                  group_select_mode, renorm, norm_type, int(bool(out_flag)),
+                                  float(routed_scaling_factor), float(eps), _ptr(y), _ptr(idx), _ptr(out),
+                                  _stream(x)), "moe355_gating_top_k")
+    return y, idx, out
+
+
+def init_routing(x, expert_idx, num_experts, quant_mode, tokens_num_type):
+    x = _dev(x, "x")
+    expert_idx = _dev(expert_idx, "expert_idx")
+    if expert_idx.dtype != torch.int32:
+        expert_idx = expert_idx.to(torch.int32)
+    lib = _lib.load()
+    T, k = expert_idx.shape
+    H = x.shape[-1]
+    R = T * k
+    dev = x.device
+    xs = torch.empty((R, H), dtype=torch.int8 if quant_mode == 1 else x.dtype, device=dev)
+    row_idx = torch.empty((R,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((num_experts,), dtype=torch.int64, device=dev)
+    scale = torch.empty((R,), dtype=torch.float32, device=dev) if quant_mode == 1 else None
+    nbytes = lib.moe355_init_routing_workspace(T, k, num_experts)
+    ws = _workspace(nbytes, dev)
+    check(lib.moe355_init_routing(_ptr(x), _dt(x, "x"), T, H, _ptr(expert_idx), k, num_experts, quant_mode,
+                                  tokens_num_type, _ptr(xs), _ptr(row_idx), _ptr(tokens), _ptr(scale), _ptr(ws),
+                                  ws.numel(), _stream(x)), "moe355_init_routing")
+    return xs, row_idx, tokens, scale
+
+
+def format_cast_nz(w: torch.Tensor, layout: int) -> torch.Tensor:
+    """int8 [E, N, K] (layout W_ENK) or [E, K, N] (W_EKN) -> same shape, MFMA-tiled storage."""
+    w = _dev(w, "weight")
+    if w.dtype != torch.int8 or w.dim() != 3:
+        raise TypeError("format_cast_nz expects a 3-D int8 weight")
+    lib = _lib.load()
+    E = w.shape[0]
+    n, k = (w.shape[1], w.shape[2]) if layout == W_ENK else (w.shape[2], w.shape[1])
+    out = torch.empty_like(w)
+    check(lib.moe355_format_cast_nz(_ptr(w), layout, E, n, k, _ptr(out), _stream(w)), "moe355_format_cast_nz")
+    return out
+
+
+def _gl_type(group_list_type: int) -> int:
+    if group_list_type == 0:
+        return GL_CUMSUM
+    if group_list_type == 1:
+        return GL_COUNT
+    raise NotImplementedError(f"group_list_type {group_list_type} is not supported on this path")
+
+
+def _gl(group_list: torch.Tensor) -> torch.Tensor:
+    group_list = _dev(group_list, "group_list")
+    return group_list if group_list.dtype == torch.int64 else group_list.to(torch.int64)
+
+
+def gmm1_swiglu_quant(x, weight_nz, weight_scale, x_scale, group_list, group_list_type, n, k, swiglu_limit=0.0,
+                      out=None, out_scale=None):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows = x.shape[0]
+    E = weight_nz.shape[0]
+    dev = x.device
+    if out is None:
+        out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
+    if out_scale is None:
+        out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.moe355_gmm1_swiglu_quant_workspace(rows, n, k, E), dev)
+    check(lib.moe355_gmm1_swiglu_quant(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_dev(weight_scale, "scale")),
+                                       _ptr(_dev(x_scale, "x_scale")), _ptr(_gl(group_list)),
+                                       _gl_type(group_list_type), rows, k, n, E, float(swiglu_limit), _ptr(out),
+                                       _ptr(out_scale), _ptr(ws), ws.numel(), _stream(x)),
+          "moe355_gmm1_swiglu_quant")
+    return out, out_scale
+
+
+def gmm2_dequant(x, weight_nz, scale, per_token_scale, group_list, group_list_type, n, k, out_dtype=torch.bfloat16):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows = x.shape[0]
+    E = weight_nz.shape[0]
+    out = torch.empty((rows, n), dtype=out_dtype, device=x.device)
+    ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
+    check(lib.moe355_gmm2_dequant(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_dev(scale, "scale")),
+                                  _ptr(_dev(per_token_scale, "per_token_scale")), _ptr(_gl(group_list)),
+                                  _gl_type(group_list_type), rows, k, n, E, _ptr(out), _dt(out, "out"), _ptr(ws),
+                                  ws.numel(), _stream(x)), "moe355_gmm2_dequant")
+    return out
+
+
+def gmm_i32(x, weight_nz, group_list, group_list_type, n, k):
+    """Raw int32 accumulators of the grouped product (rows outside every group are zero)."""
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows = x.shape[0]
+    E = weight_nz.shape[0]
+    acc = torch.zeros((rows, n), dtype=torch.int32, device=x.device)
+    ws = _workspace(256, x.device)
+    check(lib.moe355_gmm_i32(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_gl(group_list)),
+                             _gl_type(group_list_type), rows, k, n, E, _ptr(acc), _ptr(ws), ws.numel(), _stream(x)),
+          "moe355_gmm_i32")
+    return acc
+
+
+def dequant_swiglu_quant(x, weight_scale, activation_scale, activate_left=True, clamp_limit=0.0):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    n = x.shape[-1]
+    rows = x.numel() // n if n else 0
+    y = torch.empty(x.shape[:-1] + (n // 2,), dtype=torch.int8, device=x.device)
+    s = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    check(lib.moe355_dequant_swiglu_quant(_ptr(x), _ptr(_dev(weight_scale, "weight_scale")),
+                                          _ptr(_dev(activation_scale, "activation_scale")), rows, n,
+                                          int(bool(activate_left)), float(clamp_limit), _ptr(y), _ptr(s), _stream(x)),
+          "moe355_dequant_swiglu_quant")
+    return y, s
+
+
+def token_unpermute(permuted, sorted_indices, probs, residual=None):
+    permuted = _dev(permuted, "permuted_tokens")
+    sorted_indices = _dev(sorted_indices, "sorted_indices")
+    if sorted_indices.dtype != torch.int32:
+        sorted_indices = sorted_indices.to(torch.int32)
+    lib = _lib.load()
+    R, H = permuted.shape
+    if probs is not None:
+        probs = _dev(probs, "probs")
+        if probs.dtype != permuted.dtype:
+            probs = probs.to(permuted.dtype)
+        T, k = probs.shape
+    else:
+        T, k = sorted_indices.numel(), 1
+    if residual is not None:
+        residual = _dev(residual, "residual")
+    out = torch.empty((T, H), dtype=permuted.dtype, device=permuted.device)
+    check(lib.moe355_token_unpermute(_ptr(permuted), _dt(permuted, "permuted_tokens"), _ptr(sorted_indices),
+                                     _ptr(probs), T, k, H, R, _ptr(residual), _ptr(out), _stream(permuted)),
+          "moe355_token_unpermute")
+    return out
