@@ -211,6 +211,16 @@ int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorte
                            int64_t num_tokens, int top_k, int64_t hidden, int64_t permuted_rows,
                            const void *residual, void *out, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Measurement hook (no counterpart in the reference; for benchmarks).
+ * The next grouped-GEMM kernel launched from the calling thread by
+ * moe355_gmm1_swiglu_quant / moe355_gmm2_dequant / moe355_gmm_i32 is bracketed
+ * by the two hipEvent_t handles (recorded immediately before and after that
+ * one kernel, not the small helper kernels around it).  One-shot: the pair is
+ * consumed by that launch.  Pass two NULLs to cancel.
+ */
+int moe355_profile_next_gemm(void *start_event, void *stop_event);
+
 #ifdef __cplusplus
 }
 #endif

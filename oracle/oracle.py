@@ -359,3 +359,17 @@ def fp32_dequant_reference(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2) -> n
         o = act @ wd.T
         np.add.at(out, tok, o * w[tok, slot][:, None])
     return out.astype(np.float32)
+
+
+def quantized_fp64_reference(tr: LayerTrace, s2) -> np.ndarray:
+    """The same quantised pipeline (identical int8 activations and int32 accumulators) with the
+    final dequantisation and the weighted combine evaluated in float64 and no bf16 rounding:
+    isolates the rounding error of the floating-point tail from the quantisation noise."""
+    E = tr.expert_tokens.size
+    cum = np.cumsum(tr.expert_tokens)
+    row_expert = np.searchsorted(cum, np.arange(tr.acc2.shape[0]), side="right")
+    o = tr.acc2.astype(np.float64) * tr.s1.astype(np.float64)[:, None] * s2.astype(np.float64)[row_expert]
+    w = bf16_to_f32(tr.topk_weights).astype(np.float64)
+    T, k = w.shape
+    dst = tr.expanded_row_idx.reshape(T, k)
+    return (o[dst] * w[:, :, None]).sum(axis=1).astype(np.float32)

@@ -39,6 +39,7 @@ PROTOTYPES = {
                                c_void_p, c_size_t, c_void_p]),
     "moe355_dequant_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p,
                                             c_void_p, c_void_p]),
+    "moe355_profile_next_gemm": (c_int, [c_void_p, c_void_p]),
     "moe355_token_unpermute": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p,
                                        c_void_p, c_void_p]),
 }

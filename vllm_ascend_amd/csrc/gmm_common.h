@@ -29,7 +29,6 @@ struct GmmArgs {
     // outputs
     int32_t* acc;           // EPI_I32   [R, N]
     float* y;               // EPI_SWIGLU [R, N/2] fp32 SwiGLU values
-    uint32_t* rowmax;       // EPI_SWIGLU [R] bits(max|y|) + 1, 0 = row untouched
     uint16_t* out;          // EPI_DEQUANT [R, N] bf16
 };
 
@@ -38,76 +37,75 @@ __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c)
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
 }
 
-// Epilogue for one pair of 32x32 accumulator tiles held by one wavefront.
-// c0/c1: channel tile columns n0/n1 (first channel of each tile); row is the
-// lane's token row, valid says whether it exists.
-template <int EPI>
-__device__ __forceinline__ void epilogue_pair(const GmmArgs& a, int e, int64_t row, bool valid, int n0, int n1,
-                                              const v16i& c0, const v16i& c1, int lane)
+// v_mfma_i32_16x16x64_i8: A = 16 channels x 64 K (lane l: channel l%16, K slice 16*(l/16)..+15),
+// B = 16 tokens x 64 K with the same K mapping; result 4 VGPRs: token l%16, channels 4*(l/16)+0..3.
+__device__ __forceinline__ v4i mfma_i8_16(v4i a, v4i b, v4i c)
 {
-    const int hi = lane >> 5;
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+}
+
+// One token row, one run of four consecutive channels starting at c0 (tile 0) and c1 (tile 1).
+template <int EPI>
+__device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t row, bool valid, int c0, int c1,
+                                             const int* g, const int* u)
+{
+    const int n0 = c0, n1 = c1;
+    constexpr int ch = 0;
     if constexpr (EPI == EPI_I32) {
         if (!valid) return;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ch = 8 * q + 4 * hi;
-            v4i o0 = {c0[4 * q], c0[4 * q + 1], c0[4 * q + 2], c0[4 * q + 3]};
-            v4i o1 = {c1[4 * q], c1[4 * q + 1], c1[4 * q + 2], c1[4 * q + 3]};
-            *(v4i*)(a.acc + row * a.N + n0 + ch) = o0;
-            *(v4i*)(a.acc + row * a.N + n1 + ch) = o1;
-        }
+        v4i o0 = {g[0], g[1], g[2], g[3]};
+        v4i o1 = {u[0], u[1], u[2], u[3]};
+        *(v4i*)(a.acc + row * a.N + n0 + ch) = o0;
+        *(v4i*)(a.acc + row * a.N + n1 + ch) = o1;
     } else if constexpr (EPI == EPI_DEQUANT) {
         if (!valid) return;
         const float rs = a.row_scale[row];
         const float* cs = a.ch_scale + (int64_t)e * a.N;
+        const v4f s0 = *(const v4f*)(cs + n0 + ch);
+        const v4f s1 = *(const v4f*)(cs + n1 + ch);
+        v4u16 o0, o1;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ch = 8 * q + 4 * hi;
-            const v4f s0 = *(const v4f*)(cs + n0 + ch);
-            const v4f s1 = *(const v4f*)(cs + n1 + ch);
-            v4u16 o0, o1;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                o0[j] = f32_to_bf16(((float)c0[4 * q + j] * rs) * s0[j]);
-                o1[j] = f32_to_bf16(((float)c1[4 * q + j] * rs) * s1[j]);
-            }
-            *(v4u16*)(a.out + row * a.N + n0 + ch) = o0;
-            *(v4u16*)(a.out + row * a.N + n1 + ch) = o1;
+        for (int j = 0; j < 4; ++j) {
+            o0[j] = f32_to_bf16(((float)g[j] * rs) * s0[j]);
+            o1[j] = f32_to_bf16(((float)u[j] * rs) * s1[j]);
         }
+        *(v4u16*)(a.out + row * a.N + n0 + ch) = o0;
+        *(v4u16*)(a.out + row * a.N + n1 + ch) = o1;
     } else {
-        // c0 = gate tile, c1 = matching up tile (n1 = n0 + N/2)
+        // tile 0 = gate, tile 1 = the matching up tile (n1 = n0 + N/2)
         if (!valid) return;
         const int I = a.N >> 1;
         const float rs = a.row_scale[row];
         const float* cs = a.ch_scale + (int64_t)e * a.N;
-        float m = 0.0f;
+        const v4f sg = *(const v4f*)(cs + n0 + ch);
+        const v4f su = *(const v4f*)(cs + n1 + ch);
+        v4f yv;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ch = 8 * q + 4 * hi;
-            const v4f sg = *(const v4f*)(cs + n0 + ch);
-            const v4f su = *(const v4f*)(cs + n1 + ch);
-            v4f yv;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float g = ((float)c0[4 * q + j] * rs) * sg[j];
-                float u = ((float)c1[4 * q + j] * rs) * su[j];
-                if (a.limit > 0.0f) {
-                    g = g > a.limit ? a.limit : g;
-                    u = u > a.limit ? a.limit : u;
-                    u = u < -a.limit ? -a.limit : u;
-                }
-                float yy = m_silu(g) * u;
-                yv[j] = yy;
-                float ab = __builtin_fabsf(yy);
-                m = ab > m ? ab : m;
+        for (int j = 0; j < 4; ++j) {
+            float gg = ((float)g[j] * rs) * sg[j];
+            float uu = ((float)u[j] * rs) * su[j];
+            if (a.limit > 0.0f) {
+                gg = gg > a.limit ? a.limit : gg;
+                uu = uu > a.limit ? a.limit : uu;
+                uu = uu < -a.limit ? -a.limit : uu;
             }
-            *(v4f*)(a.y + row * I + n0 + ch) = yv;
+            float yy = m_silu(gg) * uu;
+            yv[j] = yy;
         }
-        // lanes l and l^32 hold the same token (and the same `valid`)
-        const float mo = __shfl_xor(m, 32, 64);
-        m = mo > m ? mo : m;
-        if (hi == 0) atomicMax(a.rowmax + row, __float_as_uint(m) + 1u);
+        *(v4f*)(a.y + row * I + n0 + ch) = yv;
     }
+}
+
+// Epilogue for one quarter of a pair of 32x32 accumulator tiles: the lane's token row and the
+// run of four consecutive channels  8*q + 4*(lane/32) + 0..3  of both tiles.
+// g[4]/u[4]: the int32 accumulators of that run in tile 0 / tile 1 (first channels n0 / n1).
+template <int EPI>
+__device__ __forceinline__ void epilogue_quad(const GmmArgs& a, int e, int64_t row, bool valid, int n0, int n1,
+                                              int q, const int* g, const int* u, int lane)
+{
+    const int hi = lane >> 5;
+    const int ch = 8 * q + 4 * hi;
+    epilogue_run<EPI>(a, e, row, valid, n0 + ch, n1 + ch, g, u);
 }
 
 }  // namespace moe355

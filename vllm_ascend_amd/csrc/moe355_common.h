@@ -108,11 +108,17 @@ __device__ __forceinline__ float wave_tree_sum(float v)
     return v;
 }
 
+// Integer sum over the wavefront with DPP row shifts and row broadcasts (no LDS traffic);
+// every lane returns the total.
 __device__ __forceinline__ int wave_sum_i32(int v)
 {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // "a ranks before b": larger value first, ties to the lower index.

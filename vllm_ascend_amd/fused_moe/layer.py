@@ -1,0 +1,54 @@
+"""Owner of one MoE layer's expert weights and the runner that strings the stages
+together: router -> ``quant_method.apply`` -> result.  Counterpart of
+``AscendRoutedExperts.forward_impl`` (``vllm_ascend/ops/fused_moe/routed_experts.py:496-609``)
+and of the weight registration in ``AscendFusedMoEMethod.create_weights``
+(``vllm_ascend/quantization/method_adapters.py:214-245``), without vLLM."""
+from __future__ import annotations
+
+import torch
+
+from ..quantization.base import AscendMoEScheme
+from .contracts import FusedExpertsResult, FusedMoEConfig
+from .moe_comm_method import setup_moe_comm_method
+from .router import AscendFusedTopKRouter
+
+
+class AscendRoutedExperts(torch.nn.Module):
+    def __init__(self, moe_config: FusedMoEConfig, quant_method: AscendMoEScheme, router: AscendFusedTopKRouter,
+                 params_dtype: torch.dtype = torch.bfloat16, device="cuda"):
+        super().__init__()
+        self.moe_config = moe_config
+        self.quant_method = quant_method
+        self.router = router
+        self.activation = moe_config.activation
+        self.apply_router_weight_on_input = False
+        self.ascend_expert_map = None
+        self.global_redundant_expert_num = 0
+        self.ascend_mc2_mask = None
+        self.ascend_pertoken_scale = None
+        specs = dict(quant_method.get_weight(moe_config.num_experts, moe_config.intermediate_size_per_partition,
+                                             moe_config.hidden_dim, params_dtype))
+        specs.update(quant_method.get_dynamic_quant_param(moe_config.num_experts,
+                                                          moe_config.intermediate_size_per_partition,
+                                                          moe_config.hidden_dim, params_dtype))
+        for name, t in specs.items():
+            self.register_parameter(name, torch.nn.Parameter(t.to(device), requires_grad=False))
+        self.moe_comm_method = setup_moe_comm_method(moe_config)
+
+    def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Copy checkpoint-layout tensors into the registered parameters, then run the scheme's
+        post-load processing (format cast, scale reshapes)."""
+        for name, t in tensors.items():
+            p = getattr(self, name)
+            p.data.copy_(t.reshape(p.data.shape).to(p.data.dtype))
+        self.quant_method.process_weights_after_loading(self)
+
+    def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
+        hidden_states, router_logits, _, _ = self.moe_comm_method.prepare(hidden_states, router_logits)
+        topk_weights, topk_ids = self.router.select_experts(hidden_states, router_logits)
+        result = self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, None, None)
+        result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
+        return result
+
+    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+        return self.forward_impl(hidden_states, router_logits).routed_out

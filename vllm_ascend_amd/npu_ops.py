@@ -1,0 +1,94 @@
+"""Stand-ins for the ``torch_npu.npu_*`` operators the fused-MoE path calls, with
+the reference's keyword arguments (call sites: ``vllm_ascend/device/device_op.py:103-127,
+192-206, 254-291, 950-954``, ``vllm_ascend/quantization/methods/w8a8_dynamic.py:350-351``).
+Each one is a thin launcher over libmoe355.so; unsupported options raise."""
+from __future__ import annotations
+
+import torch
+
+from . import kernels
+from ._lib import W_EKN, W_ENK
+
+ACL_FORMAT_FRACTAL_NZ = 29  # vllm_ascend/utils.py:61
+
+
+def npu_format_cast(weight: torch.Tensor, acl_format: int = ACL_FORMAT_FRACTAL_NZ) -> torch.Tensor:
+    """int8 ``[E, K, N]`` (or ``[K, N]``) -> same logical shape, MFMA-tiled storage.
+    The result must only be handed to the grouped-matmul operators."""
+    if acl_format != ACL_FORMAT_FRACTAL_NZ:
+        raise NotImplementedError(f"npu_format_cast: only FRACTAL_NZ ({ACL_FORMAT_FRACTAL_NZ}) is supported")
+    if weight.dim() == 2:
+        return kernels.format_cast_nz(weight.unsqueeze(0), W_EKN).squeeze(0)
+    return kernels.format_cast_nz(weight, W_EKN)
+
+
+def format_cast_from_checkpoint(weight_enk: torch.Tensor) -> torch.Tensor:
+    """int8 ``[E, N, K]`` (checkpoint order) -> tiled storage, returned with the logical
+    shape ``[E, K, N]`` the operators expect.  Same result as transposing and calling
+    ``npu_format_cast``, without materialising the transpose."""
+    tiled = kernels.format_cast_nz(weight_enk, W_ENK)
+    e, n, k = weight_enk.shape
+    return tiled.view(e, k, n)
+
+
+def npu_dynamic_quant(x: torch.Tensor, dst_type: torch.dtype | None = None):
+    if dst_type not in (None, torch.int8):
+        raise NotImplementedError(f"npu_dynamic_quant: dst_type {dst_type} is not supported (int8 only)")
+    return kernels.dynamic_quant(x)
+
+
+def npu_moe_init_routing_v2(x, expert_idx, *, scale=None, offset=None, active_num=-1, expert_capacity=-1,
+                            expert_num=-1, drop_pad_mode=0, expert_tokens_num_type=0, expert_tokens_num_flag=False,
+                            quant_mode=-1, active_expert_range=None, row_idx_type=0):
+    """-> (expanded_x, expanded_row_idx, expert_tokens, dynamic_scale)."""
+    if scale is not None or offset is not None:
+        raise NotImplementedError("npu_moe_init_routing_v2: smooth `scale`/`offset` inputs are not supported")
+    if drop_pad_mode != 0 or expert_capacity not in (-1, 0) or row_idx_type != 0:
+        raise NotImplementedError("npu_moe_init_routing_v2: drop/pad mode is not supported")
+    if quant_mode not in (-1, 1):
+        raise NotImplementedError(f"npu_moe_init_routing_v2: quant_mode {quant_mode} is not supported (-1 or 1)")
+    if expert_tokens_num_type not in (0, 1):
+        raise NotImplementedError("npu_moe_init_routing_v2: expert_tokens_num_type must be 0 (cumsum) or 1 (count)")
+    num_rows = expert_idx.numel()
+    if active_num not in (-1, 0, num_rows):
+        raise NotImplementedError("npu_moe_init_routing_v2: active_num must cover every (token, slot) pair")
+    if active_expert_range is not None and list(active_expert_range) != [0, expert_num]:
+        raise NotImplementedError("npu_moe_init_routing_v2: a partial active_expert_range (expert parallelism) "
+                                  "is not supported on one GPU")
+    x2 = x.reshape(-1, x.shape[-1])
+    xs, row_idx, tokens, dyn = kernels.init_routing(x2, expert_idx.reshape(x2.shape[0], -1), expert_num, quant_mode,
+                                                    expert_tokens_num_type)
+    return xs, row_idx, tokens, dyn
+
+
+def npu_grouped_matmul(x, weight, *, bias=None, scale=None, offset=None, antiquant_scale=None, antiquant_offset=None,
+                       per_token_scale=None, group_list=None, activation_input=None, activation_quant_scale=None,
+                       activation_quant_offset=None, split_item=0, group_type=None, group_list_type=0, act_type=0,
+                       output_dtype=None, tuning_config=None):
+    """Quantised grouped matmul, the form the down projection uses: one int8 ``x`` [M, K],
+    one tiled weight [E, K, N], per-channel ``scale`` [E, N], ``per_token_scale`` [M],
+    ``group_type=0`` (split along M), ``split_item`` 2 or 3 (single output).  Returns ``[out]``."""
+    if bias is not None or offset is not None or antiquant_scale is not None or antiquant_offset is not None:
+        raise NotImplementedError("npu_grouped_matmul: bias / offset / antiquant operands are not supported")
+    if group_type != 0 or split_item not in (2, 3) or act_type != 0:
+        raise NotImplementedError("npu_grouped_matmul: only group_type=0 with split_item 2/3 is supported")
+    xs = x if isinstance(x, (list, tuple)) else [x]
+    ws = weight if isinstance(weight, (list, tuple)) else [weight]
+    ss = scale if isinstance(scale, (list, tuple)) else [scale]
+    ps = per_token_scale if isinstance(per_token_scale, (list, tuple)) else [per_token_scale]
+    if len(xs) != 1 or len(ws) != 1 or len(ss) != 1 or len(ps) != 1 or ss[0] is None or ps[0] is None:
+        raise NotImplementedError("npu_grouped_matmul: expects exactly one x, weight, scale and per_token_scale")
+    a, w, s, p = xs[0], ws[0], ss[0], ps[0]
+    if a.dtype != torch.int8 or w.dtype != torch.int8:
+        raise NotImplementedError("npu_grouped_matmul: only the int8 x int8 form is supported")
+    if output_dtype not in (None, torch.bfloat16):
+        raise NotImplementedError(f"npu_grouped_matmul: output_dtype {output_dtype} is not supported (bfloat16 only)")
+    k, n = w.shape[1], w.shape[2]
+    out = kernels.gmm2_dequant(a, w, s.to(torch.float32), p, group_list, group_list_type, n, k)
+    return [out]
+
+
+def npu_moe_token_unpermute(permuted_tokens, sorted_indices, probs=None, padded_mode=False, restore_shape=None):
+    if padded_mode:
+        raise NotImplementedError("npu_moe_token_unpermute: padded_mode is not supported")
+    return kernels.token_unpermute(permuted_tokens, sorted_indices, probs)

@@ -1,0 +1,3 @@
+"""Quantisation schemes of the MoE layer (plugin-facing ``apply()`` contract)."""
+from .base import AscendMoEScheme, get_scheme_class, register_scheme  # noqa: F401
+from .w8a8_dynamic import AscendW8A8DynamicFusedMoEMethod  # noqa: F401

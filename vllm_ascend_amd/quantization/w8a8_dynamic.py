@@ -1,0 +1,96 @@
+"""W8A8-dynamic fused-MoE scheme: int8 per-channel weights, int8 per-token activations
+quantised on the fly.  Same contract as ``AscendW8A8DynamicFusedMoEMethod``
+(``vllm_ascend/quantization/methods/w8a8_dynamic.py:165-399``): parameter names and
+shapes, ``process_weights_after_loading`` and ``apply(layer, x, topk_weights, topk_ids,
+shared_experts, shared_experts_input)``."""
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from .. import npu_ops
+from ..fused_moe.contracts import build_fused_experts_input
+from ..fused_moe.forward_context import _EXTRA_CTX
+from ..quant_type import QuantType
+from .base import AscendMoEScheme, register_scheme
+
+
+@register_scheme("W8A8_DYNAMIC", "moe")
+class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
+    supports_eplb = True
+    quant_type: QuantType = QuantType.W8A8
+
+    def __init__(self, in_dtype: torch.dtype = torch.bfloat16, dynamic_eplb: bool = False):
+        # The reference reads these from the vLLM / Ascend configs (w8a8_dynamic.py:173-196);
+        # there is no vLLM here, so they are constructor arguments with the 1-GPU defaults.
+        if dynamic_eplb:
+            raise NotImplementedError("dynamic EPLB (per-expert weight lists) is not built yet")
+        self.in_dtype = in_dtype
+        self.dynamic_eplb = False
+        self.use_expert_weight_list = False
+        self.use_aclgraph = False
+        self.moe_all_to_all_group_name = ""  # no MC2 group on one device
+
+    def get_weight(self, num_experts: int, intermediate_size_per_partition: int, hidden_sizes: int,
+                   params_dtype: torch.dtype) -> dict[str, Any]:
+        return {
+            "w13_weight": torch.empty(num_experts, 2 * intermediate_size_per_partition, hidden_sizes,
+                                      dtype=torch.int8),
+            "w2_weight": torch.empty(num_experts, hidden_sizes, intermediate_size_per_partition, dtype=torch.int8),
+        }
+
+    def get_dynamic_quant_param(self, num_experts: int, intermediate_size_per_partition: int, hidden_sizes: int,
+                                params_dtype: torch.dtype) -> dict[str, Any]:
+        two_i = 2 * intermediate_size_per_partition
+        return {
+            "w13_weight_scale": torch.empty(num_experts, two_i, 1, dtype=params_dtype),
+            "w13_weight_offset": torch.empty(num_experts, two_i, 1, dtype=params_dtype),
+            "w2_weight_scale": torch.empty(num_experts, hidden_sizes, 1, dtype=params_dtype),
+            "w2_weight_offset": torch.empty(num_experts, hidden_sizes, 1, dtype=params_dtype),
+        }
+
+    def process_weights_after_loading(self, layer) -> None:
+        """Checkpoint order ``[E, N, K]`` -> logical ``[E, K, N]`` in the MFMA-tiled storage the
+        grouped GEMMs stream (the reference transposes, then casts to FRACTAL_NZ:
+        w8a8_dynamic.py:345-357); scales squeezed to ``[E, N]``; fp32 copies of both scales
+        (the reference keeps the w2 scale in the model dtype; the kernels take fp32)."""
+        layer.w13_weight.data = npu_ops.format_cast_from_checkpoint(layer.w13_weight.data)
+        layer.w2_weight.data = npu_ops.format_cast_from_checkpoint(layer.w2_weight.data)
+        for name in ("w13_weight_scale", "w13_weight_offset", "w2_weight_scale", "w2_weight_offset"):
+            p = getattr(layer, name, None)
+            if p is not None:
+                p.data = p.data.view(p.data.shape[0], -1)
+        layer.w13_weight_scale_fp32 = layer.w13_weight_scale.data.to(torch.float32)
+        layer.w2_weight_scale_fp32 = layer.w2_weight_scale.data.to(torch.float32)
+
+    def apply(self, layer, x: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+              shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
+        assert topk_ids is not None
+        assert topk_weights is not None
+        topk_weights = topk_weights.to(self.in_dtype)
+        moe_comm_method = _EXTRA_CTX.moe_comm_method
+        if moe_comm_method is None:
+            raise RuntimeError("no MoE communication method is set up (call setup_moe_comm_method first)")
+        return moe_comm_method.fused_experts(
+            fused_experts_input=build_fused_experts_input(
+                hidden_states=x,
+                topk_weights=topk_weights,
+                topk_ids=topk_ids,
+                w1=[layer.w13_weight],
+                w2=[layer.w2_weight],
+                quant_type=self.quant_type,
+                dynamic_eplb=self.use_expert_weight_list,
+                expert_map=getattr(layer, "ascend_expert_map", None),
+                global_redundant_expert_num=getattr(layer, "global_redundant_expert_num", 0),
+                mc2_mask=getattr(layer, "ascend_mc2_mask", None),
+                apply_router_weight_on_input=getattr(layer, "apply_router_weight_on_input", False),
+                pertoken_scale=getattr(layer, "ascend_pertoken_scale", None),
+                activation=getattr(layer, "activation", "silu"),
+                w1_scale=[layer.w13_weight_scale_fp32],
+                w2_scale=[layer.w2_weight_scale_fp32],
+            ))
+
+    @staticmethod
+    def get_eplb_weight_views(layer) -> list:
+        return [layer.w13_weight, layer.w2_weight, layer.w13_weight_scale_fp32, layer.w2_weight_scale_fp32]
