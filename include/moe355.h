@@ -73,12 +73,15 @@ int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols,
  * x [rows, E] (x_dtype), bias [E] (x_dtype) or NULL ->
  * y [rows, k] (x_dtype), expert_idx [rows, k] int32, out [rows, E] fp32
  * (written only when out_flag != 0; may be NULL otherwise).
+ * y_alt (optional, NULL to skip): a second copy of y, narrowed from the value stored
+ * in y to y_alt_dtype -- the cast the reference's caller applies next
+ * (topk_weights.to(hidden dtype), vllm_ascend/ops/fused_moe/routed_experts.py:482).
  * Limits: E <= 2048, k <= 64, group_count <= 64.
  */
 int moe355_gating_top_k(const void *x, int x_dtype, const void *bias, int64_t rows, int64_t num_experts, int k,
                         int k_group, int group_count, int group_select_mode, int renorm, int norm_type, int out_flag,
                         float routed_scaling_factor, float eps, void *y, int32_t *expert_idx, float *out,
-                        void *stream);
+                        void *y_alt, int y_alt_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Expert histogram + stable counting sort of the flattened [T*k] expert ids +
@@ -112,14 +115,6 @@ int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t 
 int moe355_format_cast_nz(const int8_t *w, int layout, int64_t num_experts, int64_t n, int64_t k, int8_t *out,
                           void *stream);
 
-/* int4 variant: w holds two 4-bit two's-complement values per byte along N
- * (low nibble = even channel; vllm_ascend/quantization/methods/w4a8.py:327-336),
- * logical [E, K, N] stored as [E, K, N/2] bytes.  out: tiled int4 storage
- * [E][N/32][K/64][64][16] bytes; entry (lane, b) holds the pair
- * k = 64*kb + 32*(lane/32) + 2*b (low nibble) and k+1 (high nibble) of channel 32*nb + lane%32. */
-int moe355_format_cast_nz_int4(const uint8_t *w_packed, int64_t num_experts, int64_t n, int64_t k, uint8_t *out,
-                               void *stream);
-
 /* ---------------------------------------------------------------------------
  * gate_up grouped GEMM (int8 x int8 -> int32) + dequant + SwiGLU + per-row int8
  * re-quantisation.
@@ -143,20 +138,6 @@ int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const flo
                              int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
                              float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
 
-/* W4A8 variant: int4 weights (moe355_format_cast_nz_int4 storage), fp32 scales
- * per group of `group_size` along K: weight_scale [E, K/group_size, N]
- * (group_size == K gives per-channel scales [E, 1, N]).
- *   f = (sum_g float(acc_g) * weight_scale[e, g, col]) * x_scale[row]   (g ascending)
- * Stands in for torch.ops._C_ascend.grouped_matmul_swiglu_quant with int4
- * weights / grouped_matmul_swiglu_quant_v2 (csrc/torch_binding.cpp:2047-2053;
- * golden tests/e2e/nightly/single_node/ops/singlecard_ops/test_grouped_matmul_swiglu_quant.py:22-109).
- * bias [E, N] fp32 or NULL is added to f before the token scale. */
-int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *weight_scale,
-                                int64_t group_size, const float *bias, const float *x_scale,
-                                const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
-                                int num_experts, float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
-                                size_t workspace_bytes, void *stream);
-
 /* ---------------------------------------------------------------------------
  * down grouped GEMM (int8 x int8 -> int32) + dequant to bf16.
  * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,
@@ -169,12 +150,6 @@ int moe355_gmm2_dequant(const int8_t *x, const int8_t *weight_nz, const float *s
                         const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
                         int num_experts, void *out, int out_dtype, void *workspace, size_t workspace_bytes,
                         void *stream);
-
-/* W4A8 down projection (same scale convention as moe355_gmm1_swiglu_quant_w4). */
-int moe355_gmm2_dequant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *scale, int64_t group_size,
-                           const float *bias, const float *per_token_scale, const int64_t *group_list,
-                           int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, void *out,
-                           int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Raw int32 accumulators of the same grouped product (no epilogue):
  * acc [R, N] int32.  The integer stage of both ops above, exposed so a caller

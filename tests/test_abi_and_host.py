@@ -1,0 +1,188 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares, the host
+mirror of the reference interface behaves like the reference for argument handling, and nothing in
+the package reaches into the checker."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KATS = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_kats.json")))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "moe355.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from vllm_ascend_amd import _lib
+
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared_symbols()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/moe355.h but not exported"
+    # the ctypes prototypes cover the same set
+    assert sorted(_lib.PROTOTYPES) == names
+
+
+def test_abi_version_and_strerror():
+    from vllm_ascend_amd import _lib
+
+    lib = _lib.load()
+    assert lib.moe355_abi_version() == _lib.ABI_VERSION
+    assert lib.moe355_strerror(0) == b"ok"
+    assert b"workspace" in lib.moe355_strerror(-3)
+
+
+def test_argument_validation_without_gpu():
+    """Rejections happen on the host before any launch, so they can be exercised without a GPU."""
+    from vllm_ascend_amd import _lib
+
+    lib = _lib.load()
+    one = ctypes.c_void_p(256)  # never dereferenced: every call below is refused first
+    assert lib.moe355_dynamic_quant(one, 1, -1, 8, one, one, None) == -1
+    assert lib.moe355_dynamic_quant(one, 0, 4, 8, one, one, None) == -5  # fp32 input not supported
+    assert lib.moe355_gating_top_k(one, 0, None, 4, 4096, 8, 1, 1, 1, 1, 0, 0, 1.0, 1e-20, one, one, None, None, 0,
+                                   None) == -2  # E > 2048
+    assert lib.moe355_gating_top_k(one, 0, None, 4, 64, 8, 1, 3, 1, 1, 0, 0, 1.0, 1e-20, one, one, None, None, 0,
+                                   None) == -2  # E % group_count
+    assert lib.moe355_gating_top_k(one, 0, None, 4, 64, 8, 1, 1, 1, 1, 2, 0, 1.0, 1e-20, one, one, None, None, 0,
+                                   None) == -1  # norm_type
+    assert lib.moe355_gmm_i32(one, one, one, 0, 4, 48, 64, 2, one, one, 256, None) == -2  # K % 32
+    assert lib.moe355_gmm_i32(one, one, one, 7, 4, 64, 64, 2, one, one, 256, None) == -1  # group list type
+    assert lib.moe355_gmm1_swiglu_quant(one, one, one, one, one, 0, 4, 64, 64, 2, 0.0, one, one, None, 0,
+                                        None) == -3  # no workspace
+    assert lib.moe355_init_routing(one, 1, 4, 64, one, 2, 8, 5, 1, one, one, one, one, one, 1 << 20, None) == -5
+    assert lib.moe355_format_cast_nz(one, 0, 2, 48, 64, one, None) == -2
+    assert lib.moe355_token_unpermute(one, 0, one, one, 4, 2, 64, 8, None, one, None) == -5
+    assert lib.moe355_init_routing_workspace(64, 8, 128) >= 128 * 4 + 129 * 4
+    assert lib.moe355_gmm1_swiglu_quant_workspace(512, 1536, 2048, 128) >= 512 * 768 * 4
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from vllm_ascend_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmoe355.so"))
+    with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
+        _lib.load()
+
+
+def test_package_never_touches_the_checker():
+    pkg = os.path.join(ROOT, "vllm_ascend_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f"{f} mentions the checker"
+
+
+def test_custom_ops_schemas_and_meta():
+    from vllm_ascend_amd.custom_ops import enable_custom_op
+
+    assert enable_custom_op()
+    ops = torch.ops._C_ascend
+    x = torch.empty(5, 128, device="meta")
+    y, idx, out = ops.moe_gating_top_k(x, k=8, k_group=1, group_count=1, group_select_mode=1, renorm=1, norm_type=0,
+                                       out_flag=False, routed_scaling_factor=1.0, eps=1e-20, bias_opt=None)
+    assert y.shape == (5, 8) and idx.dtype == torch.int32 and out.shape == (5, 128) and out.dtype == torch.float32
+    xi = torch.empty(16, 64, dtype=torch.int8, device="meta")
+    w = torch.empty(4, 64, 128, dtype=torch.int8, device="meta")
+    o, s, off = ops.grouped_matmul_swiglu_quant_weight_nz(
+        x=xi, weight=w, weight_scale=torch.empty(4, 128, device="meta"), x_scale=torch.empty(16, device="meta"),
+        group_list=torch.empty(4, dtype=torch.int64, device="meta"))
+    assert o.shape == (16, 64) and o.dtype == torch.int8 and s.shape == (16,) and s.dtype == torch.float32
+    o, s = ops.npu_dequant_swiglu_quant(torch.empty(3, 256, dtype=torch.int32, device="meta"), quant_mode=1)
+    assert o.shape == (3, 128) and s.shape == (3,)
+    # CPU tensors are refused: only the HIP kernels exist
+    with pytest.raises(NotImplementedError):
+        ops.moe_gating_top_k(torch.zeros(5, 128), k=8, k_group=1, group_count=1, group_select_mode=1, renorm=1,
+                             norm_type=0, out_flag=False, routed_scaling_factor=1.0, eps=1e-20)
+
+
+def test_gating_argument_checks_match_the_reference_adapter():
+    """Messages of csrc/moe/moe_gating_top_k/moe_gating_top_k_torch_adpt.h:33-48."""
+    from vllm_ascend_amd.custom_ops import _check_gating
+
+    with pytest.raises(RuntimeError, match="The x should be 2D"):
+        _check_gating(torch.zeros(8), None)
+    with pytest.raises(RuntimeError, match="tensor expected but got a tensor with dtype"):
+        _check_gating(torch.zeros(2, 8, dtype=torch.int32), None)
+    with pytest.raises(RuntimeError, match="The dtype of x and bias should be same"):
+        _check_gating(torch.zeros(2, 8), torch.zeros(8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="The bias should be 1D"):
+        _check_gating(torch.zeros(2, 8), torch.zeros(1, 8))
+    with pytest.raises(RuntimeError, match="The bias first dim should be same as x second dim"):
+        _check_gating(torch.zeros(2, 8), torch.zeros(4))
+
+
+def test_cumsum_group_list_known_answers():
+    """Vectors of tests/ut/ops/test_moe_mlp.py:31-62."""
+    from vllm_ascend_amd.fused_moe.moe_mlp import cumsum_group_list
+
+    k = KATS["cumsum_group_list"]
+    lists = {0: torch.tensor(k["type0_cumsum"]), 1: torch.tensor(k["type1_count"]),
+             2: torch.tensor([[1, 2], [2, 1], [0, 0], [0, 0]])}
+    for src, dst in k["supported"]:
+        assert torch.equal(cumsum_group_list(lists[src], src, dst, expert_num=4), lists[dst])
+    with pytest.raises(ValueError, match=r"group_list_type should be in \[0, 1, 2\], but received"):
+        cumsum_group_list(lists[0], 4, 0)
+    for src, dst in k["unsupported"]:
+        with pytest.raises(NotImplementedError, match="This feature is under development."):
+            cumsum_group_list(lists[0], src, dst)
+    # sparse pairs -> running sum
+    sparse = torch.tensor([[1, 2], [3, 1]])
+    assert cumsum_group_list(sparse, 2, 0, active_num=3, expert_num=4).tolist() == [0, 2, 2, 3]
+
+
+def test_scheme_weight_specs_match_the_reference():
+    """Names and shapes of vllm_ascend/quantization/methods/w8a8_dynamic.py:198-222."""
+    from vllm_ascend_amd.quant_type import QuantType
+    from vllm_ascend_amd.quantization import get_scheme_class
+
+    scheme = get_scheme_class("W8A8_DYNAMIC", "moe")()
+    assert scheme.quant_type == QuantType.W8A8 and scheme.supports_eplb
+    w = scheme.get_weight(8, 1408, 1024, torch.bfloat16)
+    assert w["w13_weight"].shape == (8, 2816, 1024) and w["w13_weight"].dtype == torch.int8
+    assert w["w2_weight"].shape == (8, 1024, 1408) and w["w2_weight"].dtype == torch.int8
+    q = scheme.get_dynamic_quant_param(8, 1408, 1024, torch.bfloat16)
+    assert q["w13_weight_scale"].shape == (8, 2816, 1) and q["w13_weight_scale"].dtype == torch.bfloat16
+    assert q["w2_weight_scale"].shape == (8, 1024, 1) and q["w13_weight_offset"].shape == (8, 2816, 1)
+    with pytest.raises(NotImplementedError):
+        get_scheme_class("W8A8_MXFP8", "moe")
+
+
+def test_unsupported_options_raise_by_name():
+    from vllm_ascend_amd.fused_moe.contracts import FusedMoEConfig, build_fused_experts_input, build_token_dispatch_input
+    from vllm_ascend_amd.fused_moe.token_dispatcher import TokenDispatcherWithAllGather
+    from vllm_ascend_amd.quant_type import QuantType
+
+    with pytest.raises(NotImplementedError, match="one GPU"):
+        FusedMoEConfig(num_experts=8, experts_per_token=2, hidden_dim=64, intermediate_size_per_partition=64,
+                       ep_size=2)
+    disp = TokenDispatcherWithAllGather(top_k=2, num_experts=8, num_local_experts=8)
+    base = dict(hidden_states=torch.zeros(4, 64, dtype=torch.bfloat16), topk_weights=torch.zeros(4, 2),
+                topk_ids=torch.zeros(4, 2, dtype=torch.int32), w1=[None], w2=[None], quant_type=QuantType.W8A8)
+    for kw, pat in ((dict(expert_map=torch.arange(8)), "expert_map"), (dict(mc2_mask=torch.ones(4)), "mc2_mask"),
+                    (dict(pertoken_scale=torch.ones(4)), "pertoken_scale")):
+        inp = build_token_dispatch_input(fused_experts_input=build_fused_experts_input(**base, **kw))
+        with pytest.raises(NotImplementedError, match=pat):
+            disp.token_dispatch(inp)
+    from vllm_ascend_amd.fused_moe.moe_mlp import quant_apply_mlp
+
+    with pytest.raises(NotImplementedError, match="gelu"):
+        quant_apply_mlp(torch.zeros(1, 8), None, None, None, None, torch.zeros(1), activation="gelu")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "ONE GPU" in r.stderr

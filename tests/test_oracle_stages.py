@@ -1,0 +1,299 @@
+"""Pins for the checker's permutation, quantiser, grouped GEMM, epilogues and combine (CPU only).
+Each check compares the C checker with something that is not its own code: the reference's
+known-answer vectors, numpy renderings of the reference's golden functions, library routines
+(stable argsort, bincount, integer matmul) or closed forms."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+
+
+def bf16(a):
+    return orc.f32_to_bf16(np.asarray(a, dtype=np.float32))
+
+
+# ------------------------------------------------------------------ conversions
+def test_bf16_rounding_closed_forms():
+    # exactly representable values survive; ties go to even; NaN stays NaN
+    v = np.array([1.0, -2.5, 0.0, 3.140625], dtype=np.float32)
+    assert np.array_equal(orc.bf16_to_f32(bf16(v)), v)
+    one_plus_half_ulp = np.float32(1.0 + 2.0 ** -8)  # halfway between 1.0 and the next bf16
+    assert orc.bf16_to_f32(bf16([one_plus_half_ulp]))[0] == 1.0  # tie -> even mantissa
+    three_halves_ulp = np.float32(1.0 + 3 * 2.0 ** -8)
+    assert orc.bf16_to_f32(bf16([three_halves_ulp]))[0] == np.float32(1.0 + 2.0 ** -6)
+    assert np.isnan(orc.bf16_to_f32(bf16([np.nan]))[0])
+    import torch
+
+    x = torch.randn(4096, dtype=torch.float32)
+    assert np.array_equal(bf16(x.numpy()), orc.to_np(x.to(torch.bfloat16)))
+    assert np.array_equal(orc.f32_to_f16(x.numpy()), x.numpy().astype(np.float16).view(np.uint16))
+    big = np.array([65504.0, 65519.9, 65520.0, 1e-8, 6e-8, -1e-5], dtype=np.float32)
+    assert np.array_equal(orc.f32_to_f16(big), big.astype(np.float16).view(np.uint16))
+    h = np.arange(0, 65536, 7, dtype=np.uint16)
+    ref = h.view(np.float16).astype(np.float32)
+    got = orc.f16_to_f32(h)
+    assert np.array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])
+
+
+# ------------------------------------------------------------------ permutation
+def test_permutation_known_answer_of_the_reference():
+    k = KATS["permutation"]
+    ids = np.array(k["topk_ids"], dtype=np.int32)
+    x = np.zeros((3, 8), dtype=np.uint16)
+    _, dst, cnt, _ = orc.init_routing(x, ids, 2)
+    assert dst.tolist() == k["expanded_row_idx"]
+    # the reference recovers the expert of each sorted row through the inverse permutation
+    inv = np.argsort(dst)
+    assert ids.reshape(-1)[inv].tolist() == k["expert_of_sorted_row"]
+    assert cnt.tolist() == [2, 4]
+
+
+@pytest.mark.parametrize("T,k,E", [(1, 1, 4), (64, 8, 128), (333, 6, 64), (40, 2, 2048)])
+def test_permutation_is_the_inverse_of_a_stable_argsort(T, k, E):
+    rng = np.random.RandomState(T + E)
+    ids = rng.randint(0, E, size=(T, k)).astype(np.int32)
+    x = orc.f32_to_bf16(rng.normal(size=(T, 16)).astype(np.float32))
+    xp, dst, cnt, _ = orc.init_routing(x, ids, E, quant=False)
+    order = np.argsort(ids.reshape(-1), kind="stable")  # sorted position -> flat index
+    assert np.array_equal(dst[order], np.arange(T * k))
+    assert np.array_equal(cnt, np.bincount(ids.reshape(-1), minlength=E))
+    assert np.array_equal(xp, x[order // k])  # sorted row i holds the token of flat pair order[i]
+    with pytest.raises(ValueError):
+        orc.init_routing(x, ids + E, E)
+
+
+def test_cumsum_group_list_vectors():
+    k = KATS["cumsum_group_list"]
+    c0, c1 = np.array(k["type0_cumsum"]), np.array(k["type1_count"])
+    assert np.array_equal(orc.cumsum_group_list(c1, 1, 0), c0)
+    assert np.array_equal(orc.cumsum_group_list(c0, 0, 1), c1)
+    assert orc.cumsum_group_list(c0, 0, 0) is c0
+
+
+# ------------------------------------------------------------------ quantiser
+def test_quantiser_closed_forms():
+    # a row of -127..127 times c quantises to itself with scale c (c a power of two: exact)
+    c = np.float32(0.25)
+    row = (np.arange(-127, 128, dtype=np.float32) * c)[None, :]
+    row = np.concatenate([row, np.zeros((1, 1), np.float32)], axis=1)  # 256 columns
+    q, s = orc.dynamic_quant(bf16(row))
+    assert s[0] == c and np.array_equal(q[0, :255], np.arange(-127, 128))
+    # all-zero row -> zeros, scale 0
+    q, s = orc.dynamic_quant(bf16(np.zeros((2, 64))))
+    assert s.tolist() == [0.0, 0.0] and not q.any()
+    # single non-zero element is the absmax -> +-127
+    z = np.zeros((1, 64), np.float32)
+    z[0, 5] = -3.0
+    q, s = orc.dynamic_quant(bf16(z))
+    assert q[0, 5] == -127 and s[0] == np.float32(3.0) / np.float32(127.0)
+    # halves round to even: scale 1 (absmax 127), values k + 0.5
+    v = np.array([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, 3.5, 0.0]], dtype=np.float32)
+    q, s = orc.dynamic_quant(bf16(v))
+    assert s[0] == 1.0 and q[0].tolist() == [127, 0, 2, 2, 0, -2, 4, 0]
+    # invariants on random rows
+    rng = np.random.RandomState(0)
+    x = bf16(rng.normal(size=(50, 512)).astype(np.float32))
+    q, s = orc.dynamic_quant(x)
+    assert np.all(np.abs(q.astype(np.int32)).max(axis=1) == 127)
+    xf = orc.bf16_to_f32(x)
+    assert np.allclose(s, np.abs(xf).max(axis=1) / 127.0, rtol=1e-7)
+    assert np.max(np.abs(q * s[:, None] - xf)) <= 0.5001 * s.max()
+
+
+def test_fused_quant_in_the_gather_equals_the_standalone_quantiser():
+    rng = np.random.RandomState(1)
+    T, k, E, H = 20, 4, 16, 64
+    x = bf16(rng.normal(size=(T, H)).astype(np.float32))
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    xs, dst, _, sx = orc.init_routing(x, ids, E)
+    q, s = orc.dynamic_quant(x)
+    for t in range(T):
+        for j in range(k):
+            assert np.array_equal(xs[dst[t * k + j]], q[t]) and sx[dst[t * k + j]] == s[t]
+
+
+# ------------------------------------------------------------------ integer GEMM
+@pytest.mark.parametrize("R,E,K,N", [(17, 3, 64, 32), (100, 8, 256, 96), (5, 4, 7168, 64)])
+def test_grouped_gemm_is_an_exact_integer_matmul(R, E, K, N):
+    rng = np.random.RandomState(R)
+    x = rng.randint(-128, 128, size=(R, K)).astype(np.int8)
+    w = rng.randint(-128, 128, size=(E, N, K)).astype(np.int8)
+    cnt = np.bincount(rng.randint(0, E, size=R - 2), minlength=E)  # two trailing rows belong to no expert
+    cum = np.cumsum(cnt)
+    acc = orc.gmm_i32(x, w, cum)
+    ref = np.zeros((R, N), dtype=np.int64)
+    r = 0
+    for e in range(E):
+        ref[r:r + cnt[e]] = x[r:r + cnt[e]].astype(np.int64) @ w[e].astype(np.int64).T
+        r += cnt[e]
+    assert np.array_equal(acc.astype(np.int64), ref)
+    assert not acc[cum[-1]:].any()
+    # worst case magnitude stays inside int32: 7168 * 128 * 128 < 2^31
+    assert 7168 * 128 * 128 < 2 ** 31
+
+
+# ------------------------------------------------------------------ gate_up epilogue
+def golden_gmm_swiglu_quant(x, w_kn, per_channel, per_token):
+    """numpy rendering of gmm_swiglu_quant, tests/e2e/nightly/single_node/ops/singlecard_ops/
+    test_gmm_swiglu_quant_weight_nz_tensor_list.py:14-55 (channel scale first, sigmoid form, 127/max)."""
+    c = (x.astype(np.int64) @ w_kn.astype(np.int64)).astype(np.float32)
+    c = c * per_channel[None, :]
+    c = c * per_token[:, None]
+    a, gate = np.split(c, 2, axis=-1)
+    a = a * (1.0 / (1.0 + np.exp(-a.astype(np.float64)))).astype(np.float32)
+    y = a * gate
+    mx = np.abs(y).max(axis=-1)
+    qscale = 127.0 / mx
+    q = np.round(y * qscale[:, None]).astype(np.int8)
+    return q, (1.0 / qscale).astype(np.float32)
+
+
+def test_gate_up_epilogue_against_the_reference_golden():
+    """Shapes scaled down from the reference case (M=8192,K=7168,E=4,N=4096); same value ranges and the
+    reference's tolerances: int8 +-1, scale rtol 1e-6 (test file :135-136)."""
+    c = KATS["gmm_swiglu_quant_case"]
+    rng = np.random.RandomState(0)
+    M, K, E, N = 256, 512, 4, 256
+    x = rng.randint(-128, 127, size=(M, K)).astype(np.int8)
+    w = rng.randint(-128, 127, size=(E, K, N)).astype(np.int8)  # reference layout [E,K,N]
+    ws = (rng.rand(E, N) * 0.9 + 0.1).astype(np.float32)
+    xs = (rng.rand(M) * 0.9 + 0.1).astype(np.float32)
+    cum = np.array([64, 128, 192, 256], dtype=np.int64)
+    acc = orc.gmm_i32(x, np.ascontiguousarray(w.transpose(0, 2, 1)), cum)
+    q, s = orc.swiglu_quant(orc.dequant_acc(acc, xs, ws, cum))
+    for e in range(E):
+        lo, hi = e * 64, (e + 1) * 64
+        qg, sg = golden_gmm_swiglu_quant(x[lo:hi], w[e], ws[e], xs[lo:hi])
+        assert np.max(np.abs(q[lo:hi].astype(np.int32) - qg.astype(np.int32))) <= c["int8_atol"]
+        assert np.allclose(s[lo:hi], sg, rtol=c["scale_rtol"], atol=1e-9)
+
+
+def test_swiglu_quant_closed_forms():
+    # gate 0 -> silu 0 -> y 0 ; large gate -> silu(g) = g ; clamp
+    f = np.array([[0.0, 100.0, -100.0, 2.0, 3.0, 5.0, 7.0, 11.0]], dtype=np.float32)  # I = 4
+    q, s, y = orc.swiglu_quant(f, want_y=True)
+    assert y[0, 0] == 0.0 and y[0, 1] == 500.0 and abs(y[0, 2]) == 0.0
+    assert np.isclose(y[0, 3], 2.0 / (1.0 + np.exp(-2.0)) * 11.0, rtol=1e-6)
+    assert s[0] == np.float32(500.0) / np.float32(127.0) and q[0, 1] == 127
+    q2, s2, y2 = orc.swiglu_quant(f, swiglu_limit=4.0, want_y=True)
+    # gate 100 clamped to 4, up 5 clamped to 4: silu(4) * 4
+    assert np.isclose(y2[0, 1], 4.0 / (1.0 + np.exp(-4.0)) * 4.0, rtol=1e-6)
+    assert np.isclose(y2[0, 3], 2.0 / (1.0 + np.exp(-2.0)) * 4.0, rtol=1e-6)  # up 11 clamped to 4
+    # all-zero row
+    q3, s3 = orc.swiglu_quant(np.zeros((1, 8), np.float32))
+    assert s3[0] == 0 and not q3.any()
+
+
+def test_token_scale_is_applied_before_the_channel_scale():
+    """csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:387-399 then :448-459.
+    Chosen so that the two orders differ in the last bit."""
+    acc = np.array([[16777217]], dtype=np.int32)  # 2^24 + 1: float(acc) rounds to 2^24 (RNE)
+    sx = np.array([np.float32(1.0 / 3.0)])
+    sw = np.array([[np.float32(3.0)]])
+    f = orc.dequant_acc(acc, sx, sw, np.array([1], dtype=np.int64))
+    a = np.float32(16777216.0)
+    assert f[0, 0] == np.float32(np.float32(a * sx[0]) * sw[0, 0])
+
+
+# ------------------------------------------------------------------ down GEMM dequant, combine
+def test_gmm2_dequant_against_float64():
+    rng = np.random.RandomState(4)
+    R, E, N = 40, 4, 64
+    acc = rng.randint(-2 ** 22, 2 ** 22, size=(R, N)).astype(np.int32)
+    s1 = (rng.rand(R) * 0.05).astype(np.float32)
+    s2 = (rng.rand(E, N) * 0.01).astype(np.float32)
+    cum = np.array([10, 10, 25, 40], dtype=np.int64)
+    o = orc.bf16_to_f32(orc.gmm2_dequant(acc, s1, s2, cum))
+    e_of = np.searchsorted(cum, np.arange(R), side="right")
+    ref = acc.astype(np.float64) * s1[:, None].astype(np.float64) * s2[e_of].astype(np.float64)
+    assert np.allclose(o, ref, rtol=2 ** -8, atol=0)
+
+
+def test_unpermute_against_a_dense_reference():
+    """Restates torch_moe (tests/e2e/nightly/single_node/ops/singlecard_ops/test_fused_moe.py:85-97):
+    out[t] = sum_j w[t,j] * expert_out(t, j)."""
+    rng = np.random.RandomState(5)
+    T, k, H = 12, 4, 32
+    R = T * k
+    o = bf16(rng.normal(size=(R, H)).astype(np.float32))
+    w = bf16(rng.rand(T, k).astype(np.float32))
+    dst = rng.permutation(R).astype(np.int32)
+    out = orc.bf16_to_f32(orc.unpermute(o, dst, w))
+    of, wf = orc.bf16_to_f32(o).astype(np.float64), orc.bf16_to_f32(w).astype(np.float64)
+    ref = (of[dst.reshape(T, k)] * wf[:, :, None]).sum(axis=1)
+    assert np.allclose(out, ref, rtol=2 ** -7, atol=1e-6)
+    # weight 1, k = 1 is a pure gather; negative indices are taken by magnitude
+    ones = bf16(np.ones((R, 1), np.float32))
+    g = orc.unpermute(o, -dst, ones)
+    assert np.array_equal(g, o[dst])
+    # exact small case: slot order matters in fp32
+    o2 = bf16(np.array([[2.0 ** 24], [1.0], [-(2.0 ** 24)]], dtype=np.float32))
+    w2 = bf16(np.ones((1, 3), np.float32))
+    assert orc.bf16_to_f32(orc.unpermute(o2, np.array([0, 1, 2], np.int32), w2))[0, 0] == 0.0  # (2^24+1)-2^24 -> 0
+    assert orc.bf16_to_f32(orc.unpermute(o2, np.array([0, 2, 1], np.int32), w2))[0, 0] == 1.0
+
+
+def golden_dequant_swiglu_quant(x, w_scale, a_scale):
+    """numpy rendering of _shared_dequant_swiglu_quant (test_dequant_swiglu_quant.py:16-45) up to the
+    SwiGLU values (the golden then calls the closed npu_dynamic_quant on a bf16 copy)."""
+    gu = x.astype(np.float32) * w_scale[None, :] * a_scale[:, None]
+    half = gu.shape[-1] // 2
+    g, u = gu[:, :half].astype(np.float64), gu[:, half:].astype(np.float64)
+    return (g / (1 + np.exp(-g)) * u).astype(np.float32)
+
+
+@pytest.mark.parametrize("shape", KATS["dequant_swiglu_quant_shapes"]["shapes"][1:])
+def test_dequant_swiglu_quant_against_the_reference_golden(shape):
+    rng = np.random.RandomState(shape[0])
+    x = rng.randint(-100, 100, size=shape).astype(np.int32)
+    ws = (rng.normal(size=shape[1]) * 0.1).astype(np.float32)
+    a = (rng.normal(size=shape[0]) * 0.5).astype(np.float32)
+    q, s = orc.dequant_swiglu_quant(x, ws, a)
+    y = golden_dequant_swiglu_quant(x, ws, a)
+    assert np.allclose(s, np.abs(y).max(axis=1) / 127.0, rtol=1e-5)
+    assert np.max(np.abs(q - np.round(y / s[:, None]))) <= 1
+
+
+# ------------------------------------------------------------------ W4A8 integer stage
+def test_w4_grouped_against_the_reference_golden():
+    """custom_mm per-group branch of test_grouped_matmul_swiglu_quant.py:22-55, in fp32."""
+    rng = np.random.RandomState(6)
+    M, K, N, E, g = 16, 512, 32, 2, 256
+    x = rng.randint(-128, 128, size=(M, K)).astype(np.int8)
+    w = rng.randint(-8, 8, size=(E, N, K)).astype(np.int8)
+    sg = rng.normal(size=(E, K // g, N)).astype(np.float32)
+    cum = np.array([10, 16], dtype=np.int64)
+    f = orc.gmm_w4_grouped(x, w, sg, cum, g)
+    for e, (lo, hi) in enumerate([(0, 10), (10, 16)]):
+        xg = x[lo:hi].reshape(hi - lo, K // g, g).astype(np.int64)
+        wg = w[e].reshape(N, K // g, g).astype(np.int64)
+        part = np.einsum("mgk,ngk->gmn", xg, wg).astype(np.float64)
+        ref = (part * sg[e][:, None, :].astype(np.float64)).sum(axis=0)
+        assert np.allclose(f[lo:hi], ref, rtol=1e-5, atol=1e-3)
+
+
+# ------------------------------------------------------------------ whole layer
+def test_layer_matches_the_dense_reference_within_quantisation_noise():
+    import sys
+
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _inputs import CONFIGS, bits, make_layer
+    from _layer_utils import oracle_layer, rel_err
+
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=0)
+    tr = oracle_layer(cfg, d)
+    got = orc.bf16_to_f32(tr.out)
+    ref = orc.fp32_dequant_reference(bits(d["x"]), tr.topk_weights, tr.topk_ids, d["w13"].numpy(), d["s13"].numpy(),
+                                     d["w2"].numpy(), d["s2"].numpy())
+    assert rel_err(got, ref) <= 5e-2
+    assert rel_err(got, orc.quantized_fp64_reference(tr, d["s2"].numpy())) <= 1e-2
+    # linearity of the combine in the routing weights: doubling every weight doubles the output exactly
+    w2 = orc.f32_to_bf16(orc.bf16_to_f32(tr.topk_weights) * 2)
+    out2 = orc.unpermute(tr.o, tr.expanded_row_idx, w2)
+    assert np.array_equal(orc.bf16_to_f32(out2), orc.bf16_to_f32(tr.out) * 2)

@@ -5,15 +5,19 @@
 
 namespace moe355 {
 
+// TOPK > 0: the slot loop is unrolled and all TOPK row loads are issued before the first add,
+// so their latencies overlap; TOPK == 0: generic loop.
+template <int TOPK>
 __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __restrict__ permuted,
                                                               const int32_t* __restrict__ idx,
-                                                              const uint16_t* __restrict__ probs, int top_k,
+                                                              const uint16_t* __restrict__ probs, int top_k_rt,
                                                               int64_t H, int64_t permuted_rows,
                                                               const uint16_t* __restrict__ residual,
                                                               uint16_t* __restrict__ out)
 {
     __shared__ int32_t srow[64];
     __shared__ float sw[64];
+    const int top_k = TOPK > 0 ? TOPK : top_k_rt;
     const int64_t t = blockIdx.x;
     if (threadIdx.x < top_k) {
         int32_t d = idx[t * top_k + threadIdx.x];
@@ -27,15 +31,34 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
         float acc[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-        for (int s = 0; s < top_k; ++s) {
-            const int32_t d = srow[s];
-            if (d < 0) continue;
-            const float w = sw[s];
-            const v8u16 v = ((const v8u16*)(permuted + (int64_t)d * H))[i];
+        if constexpr (TOPK > 0) {
+            v8u16 v[TOPK];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float pr = w * bf16_to_f32(v[j]);
-                acc[j] = acc[j] + pr;
+            for (int s = 0; s < TOPK; ++s) {
+                const int32_t d = srow[s];
+                v[s] = (d >= 0) ? ((const v8u16*)(permuted + (int64_t)d * H))[i] : (v8u16){0, 0, 0, 0, 0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int s = 0; s < TOPK; ++s) {
+                if (srow[s] < 0) continue;
+                const float w = sw[s];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    float pr = w * bf16_to_f32(v[s][j]);
+                    acc[j] = acc[j] + pr;
+                }
+            }
+        } else {
+            for (int s = 0; s < top_k; ++s) {
+                const int32_t d = srow[s];
+                if (d < 0) continue;
+                const float w = sw[s];
+                const v8u16 v = ((const v8u16*)(permuted + (int64_t)d * H))[i];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    float pr = w * bf16_to_f32(v[j]);
+                    acc[j] = acc[j] + pr;
+                }
             }
         }
         if (residual) {
@@ -64,9 +87,19 @@ extern "C" int moe355_token_unpermute(const void* permuted, int dtype, const int
     if (num_tokens == 0) return MOE355_OK;
     if (!permuted || !sorted_indices || !out) return MOE355_E_ARG;
     if (((uintptr_t)permuted & 15) || ((uintptr_t)out & 15) || ((uintptr_t)residual & 15)) return MOE355_E_SHAPE;
-    hipLaunchKernelGGL(token_unpermute_kernel, dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream,
-                       (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,
-                       permuted_rows, (const uint16_t*)residual, (uint16_t*)out);
+#define MOE355_UNPERMUTE(K)                                                                                    \
+    hipLaunchKernelGGL(token_unpermute_kernel<K>, dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream, \
+                       (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,       \
+                       permuted_rows, (const uint16_t*)residual, (uint16_t*)out)
+    switch (top_k) {
+        case 1: MOE355_UNPERMUTE(1); break;
+        case 2: MOE355_UNPERMUTE(2); break;
+        case 4: MOE355_UNPERMUTE(4); break;
+        case 6: MOE355_UNPERMUTE(6); break;
+        case 8: MOE355_UNPERMUTE(8); break;
+        default: MOE355_UNPERMUTE(0); break;
+    }
+#undef MOE355_UNPERMUTE
     return launch_status();
 }
 

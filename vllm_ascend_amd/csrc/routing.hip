@@ -136,6 +136,112 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
     }
 }
 
+// Small batches (R <= 2048 pairs): histogram, scan and stable ranks in ONE workgroup, ids held
+// in registers.  Wavefronts take their turn in order when they advance the per-expert cursors,
+// which keeps the permutation stable in the flat index.
+constexpr int kSmallMaxIters = 8;  // 8 * 256 = 2048 pairs
+
+__global__ __launch_bounds__(256) void route_small_kernel(const int32_t* __restrict__ ids, int R, int E, int nbits,
+                                                          int tokens_num_type, int32_t* __restrict__ off,
+                                                          int64_t* __restrict__ expert_tokens,
+                                                          int32_t* __restrict__ dst)
+{
+    extern __shared__ int32_t sm[];  // [E] counts, [E] cursors, [256] partials
+    int32_t* cnt = sm;
+    int32_t* cursor = sm + E;
+    int32_t* partial = sm + 2 * E;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    for (int e = tid; e < E; e += 256) cnt[e] = 0;
+    int my_e[kSmallMaxIters];
+#pragma unroll
+    for (int it = 0; it < kSmallMaxIters; ++it) {
+        const int f = it * 256 + tid;
+        int e = -1;
+        if (f < R) {
+            e = ids[f];
+            if (e < 0 || e >= E) e = -1;
+        }
+        my_e[it] = e;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kSmallMaxIters; ++it)
+        if (my_e[it] >= 0) atomicAdd(&cnt[my_e[it]], 1);
+    __syncthreads();
+    // exclusive scan of the counts: thread t owns experts [t*seg, (t+1)*seg)
+    const int seg = (E + 255) / 256;
+    const int e0 = tid * seg;
+    int32_t s = 0;
+    for (int j = 0; j < seg; ++j)
+        if (e0 + j < E) s += cnt[e0 + j];
+    partial[tid] = s;
+    __syncthreads();
+    if (wave == 0) {
+        // 256 partials, four per lane, scanned with the wavefront
+        int32_t v[4], run = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[j] = partial[lane * 4 + j];
+            run += v[j];
+        }
+        int32_t incl = run;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            int32_t t = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += t;
+        }
+        int32_t base = incl - run;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            partial[lane * 4 + j] = base;
+            base += v[j];
+        }
+    }
+    __syncthreads();
+    int32_t run = partial[tid];
+    for (int j = 0; j < seg; ++j) {
+        const int e = e0 + j;
+        if (e < E) {
+            off[e] = run;
+            cursor[e] = run;
+            run += cnt[e];
+            expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
+            if (e == E - 1) off[E] = run;
+        }
+    }
+    __syncthreads();
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int iters = (R + 255) / 256;
+    for (int it = 0; it < iters; ++it) {
+        int e = -1;
+#pragma unroll
+        for (int j = 0; j < kSmallMaxIters; ++j)
+            if (j == it) e = my_e[j];
+        const bool valid = e >= 0;
+        unsigned long long same = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (e >> b) & 1;
+            unsigned long long bal = __ballot(valid && bit);
+            same &= bit ? bal : ~bal;
+        }
+        const int rank = __popcll(same & below);
+        const int leader = valid ? (__ffsll((long long)same) - 1) : lane;
+        int32_t start = 0;
+        for (int w = 0; w < 4; ++w) {
+            if (wave == w && valid && lane == leader) {
+                start = cursor[e];
+                cursor[e] = start + __popcll(same);
+            }
+            __syncthreads();
+        }
+        start = __shfl(start, leader, 64);
+        const int f = it * 256 + tid;
+        if (f < R) dst[f] = valid ? start + rank : -1;
+    }
+}
+
 // One workgroup per token: quantise the row once, write it to its k destinations.
 template <bool QUANT>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
@@ -235,12 +341,18 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     int nbits = 0;
     while ((1 << nbits) < E) ++nbits;
 
-    hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E, ws.chunk_hist);
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), ((size_t)E + 256) * 4, st, ws.chunk_hist, nch, E,
-                       tokens_num_type, ws.off, expert_tokens);
-    if (R > 0) {
+    if (R <= kSmallMaxIters * 256) {
+        hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(256), ((size_t)2 * E + 256) * 4, st, expert_idx, (int)R, E,
+                           nbits, tokens_num_type, ws.off, expert_tokens, expanded_row_idx);
+    } else {
+        hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E,
+                           ws.chunk_hist);
+        hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), ((size_t)E + 256) * 4, st, ws.chunk_hist, nch, E,
+                           tokens_num_type, ws.off, expert_tokens);
         hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
                            ws.chunk_hist, ws.off, expanded_row_idx);
+    }
+    if (R > 0) {
         if (quant_mode == 1)
             hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, st,
                                (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);

@@ -23,8 +23,18 @@ class MI355XDeviceAdaptor:
     @staticmethod
     def moe_gating_top_k(x, *, k: int, k_group: int, group_count: int, group_select_mode: int, renorm: int,
                          norm_type: int, out_flag: bool, routed_scaling_factor: float = 1.0, eps: float = 1e-20,
-                         bias_opt=None):
+                         bias_opt=None, weights_dtype: torch.dtype | None = None):
+        """``weights_dtype`` (not in the reference): also have the kernel write the weights in that
+        dtype -- the ``topk_weights.to(hidden dtype)`` the caller does next -- and return those."""
         enable_custom_op()
+        if weights_dtype is not None and weights_dtype != x.dtype:
+            from . import custom_ops, kernels
+
+            custom_ops._check_gating(x, bias_opt)
+            _, topk_ids, out, cast = kernels.gating_top_k(x, k, k_group, group_count, group_select_mode, renorm,
+                                                          norm_type, out_flag, routed_scaling_factor, eps, bias_opt,
+                                                          alt_dtype=weights_dtype)
+            return cast, topk_ids, out
         topk_weights, topk_ids, out = torch.ops._C_ascend.moe_gating_top_k(
             x, k=k, k_group=k_group, group_count=group_count, group_select_mode=group_select_mode, renorm=renorm,
             norm_type=norm_type, out_flag=out_flag, routed_scaling_factor=routed_scaling_factor, eps=eps,
@@ -43,10 +53,19 @@ class MI355XDeviceAdaptor:
     @staticmethod
     def npu_grouped_matmul_swiglu_quant(*, x, weight, group_list, weight_scale, x_scale, bias=None,
                                         use_mxfp_quant: bool = False, act_quant_type=None, weight_quant_type=None,
-                                        swiglu_limit: float = 0.0, mxfp_quant_dtype=None):
+                                        swiglu_limit: float = 0.0, mxfp_quant_dtype=None, group_list_type: int = 0):
+        """``group_list_type`` (not in the reference, whose op only takes a running sum): 1 hands the
+        per-expert counts of the dispatcher to the kernel as they are, which saves the cumsum launch."""
         if use_mxfp_quant:
             raise RuntimeError("MXFP MoE quantization is not available on MI355X in this build.")
         enable_custom_op()
+        if group_list_type == 1:
+            from . import custom_ops, kernels
+
+            custom_ops._reject_unsupported(bias, None)
+            out, out_scale = kernels.gmm1_swiglu_quant(x, weight, weight_scale, x_scale, group_list, 1,
+                                                       weight.shape[2], weight.shape[1], swiglu_limit)
+            return out, out_scale, None
         return torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz(
             x=x, weight=weight, weight_scale=weight_scale, x_scale=x_scale, group_list=group_list, bias=bias,
             swiglu_limit=swiglu_limit)

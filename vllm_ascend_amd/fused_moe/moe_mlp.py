@@ -71,7 +71,9 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
         raise NotImplementedError("per-expert weight lists (dynamic EPLB) are not built yet")
     # gmm1: gate_up_proj + dequant + SwiGLU + dynamic re-quant in one op
     hidden_states, swiglu_out_scale, _ = DeviceOperator.npu_grouped_matmul_swiglu_quant(
-        x=hidden_states, weight=_single(w1, "w1"), group_list=cumsum_group_list(group_list, group_list_type, 0),
+        x=hidden_states, weight=_single(w1, "w1"),
+        group_list=group_list if group_list_type in (0, 1) else cumsum_group_list(group_list, group_list_type, 0),
+        group_list_type=group_list_type if group_list_type in (0, 1) else 0,
         weight_scale=_single(w1_scale, "w1_scale"), x_scale=pertoken_scale, bias=None, swiglu_limit=swiglu_limit)
     before_gmm2_evt = torch.cuda.current_stream().record_event() if hidden_states.is_cuda else None
     # gmm2: down_proj + dequant

@@ -28,10 +28,11 @@ class AscendFusedTopKRouter:
                        indices_type: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
         """-> (topk_weights in the hidden-state dtype, topk_ids int32)
         (``vllm_ascend/ops/fused_moe/routed_experts.py:438-494``)."""
-        topk_weights, topk_ids = self._compute_routing(hidden_states, router_logits, indices_type)
+        topk_weights, topk_ids = self._compute_routing(hidden_states, router_logits, indices_type,
+                                                       weights_dtype=hidden_states.dtype)
         return topk_weights.to(hidden_states.dtype), topk_ids
 
-    def _compute_routing(self, hidden_states, router_logits, indices_type=None):
+    def _compute_routing(self, hidden_states, router_logits, indices_type=None, weights_dtype=None):
         bias = self.e_score_correction_bias
         if bias is not None and bias.dtype != router_logits.dtype:
             bias = self.e_score_correction_bias = bias.to(router_logits.dtype)
@@ -47,6 +48,7 @@ class AscendFusedTopKRouter:
             routed_scaling_factor=self.routed_scaling_factor,
             eps=1e-20,
             bias_opt=bias,
+            weights_dtype=weights_dtype,
         )
         if indices_type is not None and topk_ids.dtype != indices_type:
             topk_ids = topk_ids.to(indices_type)

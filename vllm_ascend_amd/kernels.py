@@ -52,7 +52,8 @@ def dynamic_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 
 
 def gating_top_k(x, k, k_group, group_count, group_select_mode, renorm, norm_type, out_flag, routed_scaling_factor,
-                 eps, bias):
+                 eps, bias, alt_dtype=None):
+    """-> (y, expert_idx, out[, y_alt]); ``alt_dtype`` asks for a second copy of y cast to that dtype."""
     x = _dev(x, "x")
     lib = _lib.load()
     rows, E = x.shape
@@ -61,10 +62,16 @@ def gating_top_k(x, k, k_group, group_count, group_select_mode, renorm, norm_typ
     y = torch.empty((rows, k), dtype=x.dtype, device=x.device)
     idx = torch.empty((rows, k), dtype=torch.int32, device=x.device)
     out = torch.empty((rows, E), dtype=torch.float32, device=x.device)
+    y_alt = None
+    if alt_dtype is not None and alt_dtype != x.dtype:
+        y_alt = torch.empty((rows, k), dtype=alt_dtype, device=x.device)
     check(lib.moe355_gating_top_k(_ptr(x), _dt(x, "x"), _ptr(bias), rows, E, k, k_group, group_count,
                                   group_select_mode, renorm, norm_type, int(bool(out_flag)),
                                   float(routed_scaling_factor), float(eps), _ptr(y), _ptr(idx), _ptr(out),
-                                  _stream(x)), "moe355_gating_top_k")
+                                  _ptr(y_alt), _DT[alt_dtype] if y_alt is not None else 0, _stream(x)),
+          "moe355_gating_top_k")
+    if alt_dtype is not None:
+        return y, idx, out, (y if y_alt is None else y_alt)
     return y, idx, out
 
 
