@@ -113,8 +113,11 @@ def _rand_groups(g, E, R, empty_some=True):
     return cnt
 
 
+# (rows, experts, K, N).  rows/experts picks the kernel: < 48 weight streaming, >= 48 LDS-tiled with
+# 128-row tiles, >= 192 with 256-row tiles; K % 64 != 0 always streams.
 GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100, 16, 768, 2048),
-             (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256)]
+             (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256), (3000, 4, 768, 2048),
+             (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)

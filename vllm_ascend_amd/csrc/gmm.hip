@@ -14,6 +14,7 @@
 #include <stdlib.h>
 
 #include "gmm_common.h"
+#include "gmm_tiled.h"
 
 namespace moe355 {
 
@@ -223,21 +224,37 @@ static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs
     }
 }
 
-template <int EPI>
-static int launch_stream(const GmmArgs& a, hipStream_t st)
+// Rows per expert decide the kernel: few rows -> weight streaming; many -> LDS-tiled MFMA kernel.
+static int tiled_bm(const GmmArgs& a)
 {
-    const int64_t units = (int64_t)a.E * (a.N / 64);
-    static const char* force = getenv("MOE355_GEMM");  // development knob
-    const char v = force ? force[0] : 'a';
-    const dim3 g4((unsigned)units), g1((unsigned)((units + 3) / 4));
-    switch (v) {
-        case 'b': launch_gemm(gmm_stream_kernel<EPI, 1, 4, 4>, g1, st, a); break;
-        case 'c': launch_gemm(gmm_stream_kernel<EPI, 4, 8, 2>, g4, st, a); break;
-        case 'd': launch_gemm(gmm_stream_kernel<EPI, 1, 8, 2>, g1, st, a); break;
-        case 'e': launch_gemm(gmm_stream_kernel<EPI, 4, 6, 3>, g4, st, a); break;
-        case 'f': launch_gemm(gmm_stream_kernel<EPI, 4, 2, 4>, g4, st, a); break;
-        default: launch_gemm(gmm_stream_kernel<EPI, 4, 4, 4>, g4, st, a); break;
+    static const char* force = getenv("MOE355_GEMM");  // development knob: 's' stream, 't' tiled 128, 'T' tiled 256
+    if (a.K % 64 != 0) return 0;
+    if (force && force[0] == 's') return 0;
+    if (force && force[0] == 't') return 128;
+    if (force && force[0] == 'T') return 256;
+    if (force && force[0] == 'u') return 64;
+    const int64_t avg = a.R / a.E;
+    if (avg >= 48) return 128;
+    return 0;
+}
+
+static size_t tiled_ws_max(int64_t rows, int E)
+{
+    return tiled_workspace_bytes(rows, E, 64);  // the smallest tile needs the longest tile list
+}
+
+template <int EPI>
+static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
+{
+    const int bm = tile_ws ? tiled_bm(a) : 0;
+    if (bm) {
+        launch_tiled_any(EPI, bm, a, tile_ws, st, t_ev_start, t_ev_stop);
+        t_ev_start = nullptr;
+        t_ev_stop = nullptr;
+        return launch_status();
     }
+    const int64_t units = (int64_t)a.E * (a.N / 64);
+    launch_gemm(gmm_stream_kernel<EPI, 4, 4, 4>, dim3((unsigned)units), st, a);
     return launch_status();
 }
 
@@ -277,12 +294,14 @@ extern "C" int moe355_gmm_i32(const int8_t* x, const int8_t* weight_nz, const in
                               int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, int32_t* acc,
                               void* workspace, size_t workspace_bytes, void* stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
     if (rc != MOE355_OK) return rc;
     if (rows == 0) return MOE355_OK;
     if (!acc || ((uintptr_t)acc & 15)) return MOE355_E_ARG;
+    // the tile map is optional here: without (enough) scratch the streaming kernel is used
+    void* tile_ws = (workspace && !((uintptr_t)workspace & 255) && workspace_bytes >= tiled_ws_max(rows, num_experts))
+                        ? workspace
+                        : nullptr;
     GmmArgs a = {};
     a.x = x;
     a.w = weight_nz;
@@ -293,7 +312,7 @@ extern "C" int moe355_gmm_i32(const int8_t* x, const int8_t* weight_nz, const in
     a.N = (int)n;
     a.E = num_experts;
     a.acc = acc;
-    return launch_stream<EPI_I32>(a, (hipStream_t)stream);
+    return launch_gemm_auto<EPI_I32>(a, tile_ws, (hipStream_t)stream);
 }
 
 extern "C" size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
@@ -301,7 +320,7 @@ extern "C" size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, in
     (void)k;
     (void)num_experts;
     if (rows <= 0 || n <= 0) return 256;
-    return ((size_t)rows * (size_t)(n / 2) * 4 + 255) & ~(size_t)255;
+    return (((size_t)rows * (size_t)(n / 2) * 4 + 255) & ~(size_t)255) + tiled_ws_max(rows, num_experts);
 }
 
 extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz, const float* weight_scale,
@@ -334,7 +353,8 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
     a.ch_scale = weight_scale;
     a.limit = swiglu_limit;
     a.y = y;
-    rc = launch_stream<EPI_SWIGLU>(a, st);
+    void* tile_ws = (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
+    rc = launch_gemm_auto<EPI_SWIGLU>(a, tile_ws, st);
     if (rc != MOE355_OK) return rc;
     hipLaunchKernelGGL(swiglu_requant_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, y, group_list,
                        group_list_type, num_experts, rows, I, out, out_scale);
@@ -343,11 +363,10 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
 
 extern "C" size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
 {
-    (void)rows;
     (void)n;
     (void)k;
-    (void)num_experts;
-    return 256;
+    if (rows <= 0 || num_experts <= 0) return 256;
+    return tiled_ws_max(rows, num_experts);
 }
 
 extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, const float* scale,
@@ -355,11 +374,12 @@ extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, con
                                    int64_t rows, int64_t k, int64_t n, int num_experts, void* out, int out_dtype,
                                    void* workspace, size_t workspace_bytes, void* stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
     if (rc != MOE355_OK) return rc;
     if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (rows > 0 && (!workspace || ((uintptr_t)workspace & 255) ||
+                     workspace_bytes < moe355_gmm2_dequant_workspace(rows, n, k, num_experts)))
+        return MOE355_E_WORKSPACE;
     if (rows == 0) return MOE355_OK;
     if (!scale || !per_token_scale || !out) return MOE355_E_ARG;
     if (((uintptr_t)scale & 15) || ((uintptr_t)out & 7)) return MOE355_E_SHAPE;
@@ -375,5 +395,5 @@ extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, con
     a.row_scale = per_token_scale;
     a.ch_scale = scale;
     a.out = (uint16_t*)out;
-    return launch_stream<EPI_DEQUANT>(a, (hipStream_t)stream);
+    return launch_gemm_auto<EPI_DEQUANT>(a, workspace, (hipStream_t)stream);
 }

@@ -1,0 +1,357 @@
+// Grouped int8 GEMM for many rows per expert (prefill): MFMA-bound, LDS-staged tokens.
+//
+// Workgroup tile: BM tokens x 256 channels, K consumed 64 at a time.  The four wavefronts own 64
+// channels each (two 32-channel storage tiles: for the gate_up GEMM a gate tile and its up tile,
+// so SwiGLU pairs meet in one lane).  Weights never touch LDS: a storage tile is one MFMA A
+// operand and is loaded straight into registers, two iterations ahead.  Tokens are shared by the
+// four wavefronts: global -> registers (three iterations ahead) -> LDS in MFMA-operand order
+// (every B operand is one conflict-free 1 KiB ds_read_b128 sweep) -> MFMA.
+// Tiles are enumerated (expert, row block) by a small map kernel from the group list; the 1-D
+// grid is remapped so that all column blocks of a row block, and the row blocks of one expert,
+// run on the same XCD (workgroup i goes to XCD i % 8) and share its L2.
+#include <hip/hip_ext.h>
+
+#include "gmm_common.h"
+#include "gmm_tiled.h"
+
+namespace moe355 {
+
+// One workgroup.  Thread t owns experts [t*seg, (t+1)*seg).  Tiles are numbered expert by expert.
+__global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict__ gl, int gl_type, int E, int BM,
+                                                       int max_tiles, TileMap tm)
+{
+    __shared__ int32_t part_rows[256];
+    __shared__ int32_t part_tiles[256];
+    const int tid = threadIdx.x;
+    const int seg = (E + 255) / 256;
+    const int e0 = tid * seg;
+    auto rows_of = [&](int e) -> int64_t {
+        int64_t m = (gl_type == MOE355_GL_COUNT) ? gl[e] : gl[e] - (e > 0 ? gl[e - 1] : 0);
+        return m < 0 ? 0 : m;
+    };
+    int32_t rows = 0, tiles = 0;
+    for (int j = 0; j < seg; ++j) {
+        const int e = e0 + j;
+        if (e < E) {
+            const int64_t m = rows_of(e);
+            rows += (int32_t)m;
+            tiles += (int32_t)((m + BM - 1) / BM);
+        }
+    }
+    part_rows[tid] = rows;
+    part_tiles[tid] = tiles;
+    __syncthreads();
+    if (tid == 0) {
+        int32_t r = 0, t = 0;
+        for (int i = 0; i < 256; ++i) {
+            const int32_t a = part_rows[i], b = part_tiles[i];
+            part_rows[i] = r;
+            part_tiles[i] = t;
+            r += a;
+            t += b;
+        }
+        tm.count[0] = t < max_tiles ? t : max_tiles;
+    }
+    __syncthreads();
+    int64_t row = part_rows[tid];
+    int32_t t = part_tiles[tid];
+    for (int j = 0; j < seg; ++j) {
+        const int e = e0 + j;
+        if (e < E) {
+            const int64_t m = rows_of(e);
+            for (int64_t r0 = row; r0 < row + m; r0 += BM) {
+                if (t < max_tiles) {
+                    tm.expert[t] = e;
+                    tm.row_begin[t] = (int32_t)r0;
+                    tm.row_end[t] = (int32_t)(row + m);
+                }
+                ++t;
+            }
+            row += m;
+        }
+    }
+}
+
+constexpr int kBN = 256;  // channels per workgroup (4 wavefronts x 2 storage tiles)
+constexpr int kBK = 64;   // K per pipeline stage (2 MFMA K steps)
+
+template <int EPI, int BMT>  // BMT = token blocks of 32 per workgroup tile (BM = 32 * BMT)
+__global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+{
+    constexpr int BM = 32 * BMT;
+    constexpr int STAGE_BYTES = BM * kBK;                 // tokens of one stage in LDS
+    constexpr int CHUNKS = STAGE_BYTES / 16 / 256;        // 16-byte chunks per thread per stage
+    constexpr int ROWB = 128 + 16;                        // epilogue patch: bytes per token row (padded)
+    constexpr int PATCHES = (EPI == EPI_I32) ? 2 : 1;     // 32-row patches per wavefront in the epilogue
+    constexpr int EPI_BYTES = 4 * PATCHES * 32 * ROWB;
+    constexpr int LDS_BYTES = 3 * STAGE_BYTES > EPI_BYTES ? 3 * STAGE_BYTES : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) int8_t lds_raw[LDS_BYTES];
+    int8_t (*Bs)[STAGE_BYTES] = reinterpret_cast<int8_t (*)[STAGE_BYTES]>(lds_raw);
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+
+    // ---- which tile: XCD-aware remap of the 1-D grid over the tiles that exist (workgroup i runs on
+    // XCD i % 8; each XCD gets one contiguous eighth of the tile list, in order)
+    const int total = tm.count[0] * n_col_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int slot = (int)(blockIdx.x / 8);
+    const int item = (int)(blockIdx.x % 8) * per_xcd + slot;
+    if (slot >= per_xcd || item >= total) return;
+    const int mt = item / n_col_blocks;
+    const int nt = item % n_col_blocks;
+    const int e = tm.expert[mt];
+    const int64_t row0 = tm.row_begin[mt];
+    int64_t row_end = tm.row_end[mt];
+    if (row_end > a.R) row_end = a.R;
+    if (row0 >= row_end) return;
+
+    const int NB = a.N >> 5, KB = a.K >> 5;
+    const int half_tiles = NB >> 1;
+    // storage tiles of this wavefront
+    int nb0, nb1;
+    if constexpr (EPI == EPI_SWIGLU) {
+        nb0 = nt * 4 + wave;          // gate tile
+        nb1 = nb0 + half_tiles;       // its up tile
+    } else {
+        nb0 = nt * 8 + 2 * wave;
+        nb1 = nb0 + 1;
+    }
+    const bool have = (EPI == EPI_SWIGLU) ? (nb0 < half_tiles) : (nb1 < NB);
+    const int8_t* w0 = a.w + (((int64_t)e * NB + (have ? nb0 : 0)) * KB) * 1024 + lane * 16;
+    const int8_t* w1 = a.w + (((int64_t)e * NB + (have ? nb1 : 0)) * KB) * 1024 + lane * 16;
+
+    const int n_iter = a.K / kBK;
+
+    v4i Areg[3][2][2];   // [stage][tile][k step]
+    v4i Breg[3][CHUNKS];
+
+    // Loads past the last K block or the last row are redirected to valid addresses instead of being
+    // skipped (their results are never used): the loop body stays free of branches, so the compiler can
+    // keep several stages of loads in flight with partial s_waitcnt counts.
+    const int last_it = n_iter - 1;
+    auto load_A = [&](int it, int st) {
+        const int itc = it < last_it ? it : last_it;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            Areg[st][0][s] = *(const v4i*)(w0 + ((int64_t)itc * 2 + s) * 1024);
+            Areg[st][1][s] = *(const v4i*)(w1 + ((int64_t)itc * 2 + s) * 1024);
+        }
+    };
+    const int8_t* xrow[CHUNKS];
+    int lds_off[CHUNKS];
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+        // 16 consecutive lanes take 16 consecutive token rows at the same K chunk: their 16-byte LDS
+        // writes then fall into 16 different bank groups (no conflicts), and a load instruction still
+        // covers 16 rows x 64 contiguous bytes
+        const int row = (tid & 15) + 16 * ((tid >> 6) + 4 * j);
+        const int kc = (tid >> 4) & 3;
+        int64_t r = row0 + row;
+        if (r > row_end - 1) r = row_end - 1;  // rows past the expert's end duplicate its last row
+        xrow[j] = a.x + r * a.K + kc * 16;
+        const int s = kc >> 1, kh = kc & 1;
+        lds_off[j] = (((s * BMT + (row >> 5)) * 64) + kh * 32 + (row & 31)) * 16;
+    }
+    auto load_B = [&](int it, int st) {
+        const int itc = it < last_it ? it : last_it;
+#pragma unroll
+        for (int j = 0; j < CHUNKS; ++j) Breg[st][j] = *(const v4i*)(xrow[j] + (int64_t)itc * kBK);
+    };
+    auto store_B = [&](int st) {
+#pragma unroll
+        for (int j = 0; j < CHUNKS; ++j) *(v4i*)(&Bs[st][lds_off[j]]) = Breg[st][j];
+    };
+
+    v16i acc[2][BMT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int b = 0; b < BMT; ++b) acc[t][b] = (v16i){0};
+
+    // B operands of one K step (BMT fragments of 1 KiB) live in registers; the two K steps of a stage
+    // are double-buffered so that LDS reads of one step run under the MFMAs of the other.
+    v4i bf0[BMT], bf1[BMT];
+    auto read_frags = [&](v4i* dst, int st, int s) {
+#pragma unroll
+        for (int b = 0; b < BMT; ++b) dst[b] = *(const v4i*)(&Bs[st][((s * BMT + b) * 64 + lane) * 16]);
+    };
+    auto mma_step = [&](const v4i* frags, int st, int s) {
+#pragma unroll
+        for (int b = 0; b < BMT; ++b) {
+            acc[0][b] = mfma_i8(Areg[st][0][s], frags[b], acc[0][b]);
+            acc[1][b] = mfma_i8(Areg[st][1][s], frags[b], acc[1][b]);
+        }
+    };
+
+    // ---- prologue.  After it the loads still in flight are, oldest first, A(0) B(1) A(1) B(2): the same
+    // order every iteration leaves behind, so the wait counts the compiler derives at the loop head are exact.
+    load_B(0, 0);
+    store_B(0);
+    __syncthreads();
+    load_A(0, 0);
+    load_B(1, 1);
+    load_A(1, 1);
+    load_B(2, 2);
+    read_frags(bf0, 0, 0);
+
+    // One pipeline step on stage U (compile-time ring position) for K block I.
+#define MOE355_STEP(U, I)                                                          \
+    {                                                                              \
+        store_B(((U) + 1) % 3);             /* B(I+1): registers -> LDS */         \
+        read_frags(bf1, (U), 1);            /* second K step of this stage */      \
+        __builtin_amdgcn_sched_barrier(0);                                         \
+        mma_step(bf0, (U), 0);                                                     \
+        __syncthreads();                    /* B(I+1) visible to all wavefronts */ \
+        load_A((I) + 2, ((U) + 2) % 3);                                            \
+        load_B((I) + 3, (U));                                                      \
+        read_frags(bf0, ((U) + 1) % 3, 0);  /* first K step of the next stage */   \
+        __builtin_amdgcn_sched_barrier(0);                                         \
+        mma_step(bf1, (U), 1);                                                     \
+    }
+    // whole triples run without any condition inside (exact wait counts); the remainder is peeled
+    const int n_full = (n_iter / 3) * 3;
+    for (int i0 = 0; i0 < n_full; i0 += 3) {
+        MOE355_STEP(0, i0)
+        MOE355_STEP(1, i0 + 1)
+        MOE355_STEP(2, i0 + 2)
+    }
+    if (n_iter - n_full >= 1) MOE355_STEP(0, n_full)
+    if (n_iter - n_full >= 2) MOE355_STEP(1, n_full + 1)
+#undef MOE355_STEP
+
+    // ---- epilogue.  In the accumulators a lane owns one token and scattered runs of four channels;
+    // written like that every store would touch 64 different cache lines.  Each wavefront instead
+    // turns one 32-token block at a time through a private LDS patch (token-major, 128 data bytes per
+    // token and tile) and stores whole 128-byte row segments: 8 lanes per token row.
+    __syncthreads();  // all wavefronts are done reading the token stages; LDS is reused below
+    if (!have) return;
+    int8_t* patch = lds_raw + wave * (PATCHES * 32 * ROWB);
+    const int tok = lane & 31;
+    const int hi = lane >> 5;
+    const float* cs = a.ch_scale ? a.ch_scale + (int64_t)e * a.N : nullptr;
+    v4f s0[4], s1[4];
+    if constexpr (EPI != EPI_I32) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            s0[q] = *(const v4f*)(cs + nb0 * 32 + 8 * q + 4 * hi);
+            s1[q] = *(const v4f*)(cs + nb1 * 32 + 8 * q + 4 * hi);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BMT; ++b) {
+        const int64_t row = row0 + b * 32 + tok;
+        const bool valid = row < row_end;
+        float rs = 0.0f;
+        if constexpr (EPI != EPI_I32) rs = valid ? a.row_scale[row] : 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int ch = 8 * q + 4 * hi;  // first of this lane's four channels inside the tile
+            if constexpr (EPI == EPI_I32) {
+                *(v4i*)(patch + tok * ROWB + ch * 4) =
+                    (v4i){acc[0][b][4 * q], acc[0][b][4 * q + 1], acc[0][b][4 * q + 2], acc[0][b][4 * q + 3]};
+                *(v4i*)(patch + 32 * ROWB + tok * ROWB + ch * 4) =
+                    (v4i){acc[1][b][4 * q], acc[1][b][4 * q + 1], acc[1][b][4 * q + 2], acc[1][b][4 * q + 3]};
+            } else if constexpr (EPI == EPI_DEQUANT) {
+                v4u16 o0, o1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    o0[j] = f32_to_bf16(((float)acc[0][b][4 * q + j] * rs) * s0[q][j]);
+                    o1[j] = f32_to_bf16(((float)acc[1][b][4 * q + j] * rs) * s1[q][j]);
+                }
+                // both tiles are adjacent in the output row: 64 bf16 = 128 bytes per token
+                *(v4u16*)(patch + tok * ROWB + ch * 2) = o0;
+                *(v4u16*)(patch + tok * ROWB + 64 + ch * 2) = o1;
+            } else {
+                v4f yv;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float gg = ((float)acc[0][b][4 * q + j] * rs) * s0[q][j];
+                    float uu = ((float)acc[1][b][4 * q + j] * rs) * s1[q][j];
+                    if (a.limit > 0.0f) {
+                        gg = gg > a.limit ? a.limit : gg;
+                        uu = uu > a.limit ? a.limit : uu;
+                        uu = uu < -a.limit ? -a.limit : uu;
+                    }
+                    yv[j] = m_silu(gg) * uu;
+                }
+                *(v4f*)(patch + tok * ROWB + ch * 4) = yv;
+            }
+        }
+        // read back row-major: lane -> (row r8 + 8*p, 16-byte column c16)
+        const int c16 = lane & 7, r8 = lane >> 3;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int r = r8 + 8 * p;
+            const int64_t orow = row0 + b * 32 + r;
+            if (orow < row_end) {
+                if constexpr (EPI == EPI_I32) {
+                    *(v4i*)(a.acc + orow * a.N + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                    *(v4i*)(a.acc + orow * a.N + nb1 * 32 + c16 * 4) =
+                        *(const v4i*)(patch + 32 * ROWB + r * ROWB + c16 * 16);
+                } else if constexpr (EPI == EPI_DEQUANT) {
+                    *(v4i*)(a.out + orow * a.N + nb0 * 32 + c16 * 8) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                } else {
+                    *(v4i*)(a.y + orow * (a.N >> 1) + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                }
+            }
+        }
+    }
+}
+
+
+
+// ------------------------------------------------------------------ host side
+size_t tiled_workspace_bytes(int64_t rows, int E, int BM)
+{
+    const int64_t max_tiles = rows / BM + E;
+    return 256 + (size_t)(((max_tiles * 4 + 255) / 256) * 256) * 3;
+}
+
+template <int EPI, int BMT>
+static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
+{
+    constexpr int BM = 32 * BMT;
+    const int max_tiles = (int)(a.R / BM + a.E);
+    const size_t arr = (size_t)(((size_t)max_tiles * 4 + 255) / 256) * 256;
+    TileMap tm;
+    tm.count = (int32_t*)workspace;
+    tm.expert = (int32_t*)((char*)workspace + 256);
+    tm.row_begin = (int32_t*)((char*)workspace + 256 + arr);
+    tm.row_end = (int32_t*)((char*)workspace + 256 + 2 * arr);
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm);
+    const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
+    const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
+    const int n_col_blocks = (channels + per_block - 1) / per_block;
+    const int total = max_tiles * n_col_blocks;
+    const int grid = ((total + 7) / 8) * 8;
+    if (ev0 && ev1)
+        hipExtLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT>), dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm,
+                              max_tiles, n_col_blocks);
+    else
+        hipLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT>), dim3(grid), dim3(256), 0, st, a, tm, max_tiles,
+                           n_col_blocks);
+}
+
+void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
+                      hipEvent_t ev1)
+{
+#define MOE355_TILED(E_, B_) launch_tiled<E_, B_>(a, workspace, st, ev0, ev1)
+    if (bm == 256) {
+        if (epi == EPI_I32) MOE355_TILED(EPI_I32, 8);
+        else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 8);
+        else MOE355_TILED(EPI_DEQUANT, 8);
+    } else if (bm == 128) {
+        if (epi == EPI_I32) MOE355_TILED(EPI_I32, 4);
+        else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 4);
+        else MOE355_TILED(EPI_DEQUANT, 4);
+    } else {
+        if (epi == EPI_I32) MOE355_TILED(EPI_I32, 2);
+        else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 2);
+        else MOE355_TILED(EPI_DEQUANT, 2);
+    }
+#undef MOE355_TILED
+}
+
+}  // namespace moe355

@@ -26,14 +26,13 @@ __device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uin
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
-// fp32 -> bf16, round to nearest even, NaN stays quiet NaN.
+// fp32 -> bf16, round to nearest even (gfx950 has the conversion in hardware: v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    uint32_t lsb = (u >> 16) & 1u;
-    u += 0x7fffu + lsb;
-    return (uint16_t)(u >> 16);
+    __bf16 b = (__bf16)f;
+    uint16_t h;
+    __builtin_memcpy(&h, &b, 2);
+    return h;
 }
 
 __device__ __forceinline__ float f16_to_f32(uint16_t h)
@@ -51,13 +50,12 @@ __device__ __forceinline__ uint16_t f32_to_f16(float f)
     return h;
 }
 
-// exp(x): n = rint(x*log2e), two-part ln2 reduction, degree-5 polynomial,
-// result scaled by 2^n in two exact steps.  Mul/add only, no contraction.
+// exp(x): argument clamped to [-87, 88.72283] (result always normal or +inf; NaN counts as -87),
+// n = rint(x*log2e), two-part ln2 reduction, degree-5 polynomial, exact scaling by 2^n.
+// Mul/add only, no contraction.
 __device__ __forceinline__ float m_expf(float x)
 {
-    if (x != x) return x;
-    if (x > 88.72283f) return __builtin_inff();
-    if (x < -87.33654f) return 0.0f;
+    x = __builtin_fminf(__builtin_fmaxf(x, -87.0f), 88.72283f);
     float n = __builtin_rintf(x * 1.44269504088896341f);
     float r = x - n * 0.693359375f;
     r = r - n * -2.12194440e-4f;
@@ -70,12 +68,7 @@ __device__ __forceinline__ float m_expf(float x)
     float r2 = r * r;
     float y = p * r2 + r;
     y = y + 1.0f;
-    int ni = (int)n;
-    int n1 = ni / 2;
-    int n2 = ni - n1;
-    float s1 = __uint_as_float((uint32_t)(n1 + 127) << 23);
-    float s2 = __uint_as_float((uint32_t)(n2 + 127) << 23);
-    return (y * s1) * s2;
+    return __builtin_ldexpf(y, (int)n);
 }
 
 __device__ __forceinline__ float m_silu(float g) { return g / (1.0f + m_expf(-g)); }

@@ -164,7 +164,7 @@ def gmm_i32(x, weight_nz, group_list, group_list_type, n, k):
     rows = x.shape[0]
     E = weight_nz.shape[0]
     acc = torch.zeros((rows, n), dtype=torch.int32, device=x.device)
-    ws = _workspace(256, x.device)
+    ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm_i32(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_gl(group_list)),
                              _gl_type(group_list_type), rows, k, n, E, _ptr(acc), _ptr(ws), ws.numel(), _stream(x)),
           "moe355_gmm_i32")
