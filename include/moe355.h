@@ -115,6 +115,16 @@ int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t 
 int moe355_format_cast_nz(const int8_t *w, int layout, int64_t num_experts, int64_t n, int64_t k, int8_t *out,
                           void *stream);
 
+/* int4 weights (W4A8): two 4-bit two's-complement values per byte.
+ * source 0: w is int8 [E, N, K] holding one int4 value (-8..7) per byte (checkpoint order);
+ * source 1: w is packed [E, K, N/2] bytes, low nibble = even channel, the packing of
+ *           vllm_ascend/quantization/methods/w4a8.py:327-336.
+ * out: tiled int4 storage, E*N*K/2 bytes: [E][N/32][K/64][64][16]; inside a 1 KiB tile, byte b of
+ * entry `lane` holds w[e, 32*nb + lane%32, 64*kb + 16*(lane/32) + b] in its low nibble and the
+ * value 32 further along K in its high nibble.  N % 32 == 0, K % 64 == 0. */
+int moe355_format_cast_nz_int4(const uint8_t *w, int source, int64_t num_experts, int64_t n, int64_t k, uint8_t *out,
+                               void *stream);
+
 /* ---------------------------------------------------------------------------
  * gate_up grouped GEMM (int8 x int8 -> int32) + dequant + SwiGLU + per-row int8
  * re-quantisation.
@@ -138,6 +148,21 @@ int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const flo
                              int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
                              float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
 
+/* W4A8 variant: int4 weights (moe355_format_cast_nz_int4 storage), fp32 scales per group of
+ * `group_size` values along K: weight_scale [E, K/group_size, N] (group_size == K: per channel).
+ *   f = (sum_g float(acc_g) * weight_scale[e, g, col] (g ascending) + bias[e, col]) * x_scale[row]
+ * then SwiGLU and re-quantisation as above.  bias [E, N] fp32 or NULL.
+ * Stands in for the int4 form of torch.ops._C_ascend.grouped_matmul_swiglu_quant /
+ * grouped_matmul_swiglu_quant_v2 (csrc/torch_binding.cpp:2025-2053; kernel
+ * csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant_a8w4_msd_*.h; golden
+ * tests/e2e/nightly/single_node/ops/singlecard_ops/test_grouped_matmul_swiglu_quant.py:22-109).
+ * Workspace: rows * (n/2) * 4 bytes.  Limits: N % 64 == 0, K % 64 == 0, group_size % 64 == 0. */
+int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *weight_scale,
+                                int64_t group_size, const float *bias, const float *x_scale,
+                                const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
+                                int num_experts, float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
+                                size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------------------
  * down grouped GEMM (int8 x int8 -> int32) + dequant to bf16.
  * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,
@@ -150,6 +175,14 @@ int moe355_gmm2_dequant(const int8_t *x, const int8_t *weight_nz, const float *s
                         const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
                         int num_experts, void *out, int out_dtype, void *workspace, size_t workspace_bytes,
                         void *stream);
+
+/* W4A8 down projection:
+ *   out[row, col] = bf16( (sum_g float(acc_g) * scale[e, g, col] + bias[e, col]) * per_token_scale[row] )
+ * (the int4 form of torch_npu.npu_grouped_matmul as called from vllm_ascend/ops/fused_moe/moe_mlp.py:552-569). */
+int moe355_gmm2_dequant_w4(const int8_t *x, const uint8_t *weight_nz4, const float *scale, int64_t group_size,
+                           const float *bias, const float *per_token_scale, const int64_t *group_list,
+                           int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, void *out,
+                           int out_dtype, void *stream);
 
 /* Raw int32 accumulators of the same grouped product (no epilogue):
  * acc [R, N] int32.  The integer stage of both ops above, exposed so a caller

@@ -219,6 +219,30 @@ def scale_rows(f, sx):
     return f
 
 
+def w4_rows_to_bf16(f, s1):
+    f = np.ascontiguousarray(f, dtype=np.float32)
+    s1 = np.ascontiguousarray(s1, dtype=np.float32)
+    o = np.zeros(f.shape, dtype=np.uint16)
+    lib().orc_w4_rows_to_bf16(_p(f), _p(s1), _i64(f.shape[0]), _i64(f.shape[1]), _p(o))
+    return o
+
+
+def w4a8_experts_forward(x_bf16, topk_w_bf16, topk_ids, w13_i4, sg13, w2_i4, sg2, group_size) -> LayerTrace:
+    """W4A8 twin of experts_forward: int4 weight values (one per int8) [E,N,K], group scales [E,K/g,N]."""
+    E = w13_i4.shape[0]
+    tr = LayerTrace(topk_weights=topk_w_bf16, topk_ids=topk_ids)
+    tr.xs, tr.expanded_row_idx, tr.expert_tokens, tr.sx = init_routing(x_bf16, topk_ids, E)
+    cum = np.cumsum(tr.expert_tokens)
+    g1 = group_size if group_size > 0 else w13_i4.shape[2]
+    g2 = group_size if group_size > 0 else w2_i4.shape[2]
+    f = scale_rows(gmm_w4_grouped(tr.xs, w13_i4, sg13, cum, g1), tr.sx)
+    tr.q1, tr.s1 = swiglu_quant(f)
+    f2 = gmm_w4_grouped(tr.q1, w2_i4, sg2, cum, g2)
+    tr.o = w4_rows_to_bf16(f2, tr.s1)
+    tr.out = unpermute(tr.o, tr.expanded_row_idx, topk_w_bf16)
+    return tr
+
+
 def swiglu_quant(f, swiglu_limit=0.0, want_y=False):
     f = np.ascontiguousarray(f, dtype=np.float32)
     rows, N = f.shape

@@ -23,6 +23,8 @@ class LayerCfg:
     routed_scaling_factor: float = 1.0
     bias: bool = False
     shared: bool = False
+    w4_group: int = -1  # >= 0: W4A8 (int4 weights); 0 = per-channel scales, g > 0 = groups of g along K
+    zipf: float = 0.0  # > 0: router logits biased so that expert popularity follows Zipf(s)
 
 
 CONFIGS = {
@@ -32,6 +34,11 @@ CONFIGS = {
     "c3_qwen3_prefill": LayerCfg("c3_qwen3_prefill", 8192, 2048, 128, 8, 768),
     "c4_dsv3_prefill": LayerCfg("c4_dsv3_prefill", 4096, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8,
                                 topk_group=4, routed_scaling_factor=2.5, bias=True, shared=True),
+    "c5_w4a8_zipf": LayerCfg("c5_w4a8_zipf", 512, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8, topk_group=4,
+                             routed_scaling_factor=2.5, bias=True, w4_group=256, zipf=1.1),
+    "c5_small": LayerCfg("c5_small", 80, 512, 32, 4, 256, scoring="sigmoid", n_group=4, topk_group=2,
+                         routed_scaling_factor=2.5, bias=True, w4_group=128, zipf=1.1),
+    "c5_small_perchannel": LayerCfg("c5_small_perchannel", 40, 256, 16, 2, 128, w4_group=0),
     # reduced shapes with the same structure
     "c2_small": LayerCfg("c2_small", 48, 512, 32, 4, 256),
     "c3_small": LayerCfg("c3_small", 640, 512, 16, 4, 256),
@@ -47,10 +54,26 @@ def make_layer(cfg: LayerCfg, seed: int = 0, device: str = "cpu"):
     d = {}
     d["x"] = torch.randn(cfg.T, cfg.H, generator=g, dtype=torch.float32).to(torch.bfloat16)
     d["logits"] = torch.randn(cfg.T, cfg.E, generator=g, dtype=torch.float32)
-    d["w13"] = torch.randint(-127, 128, (cfg.E, 2 * cfg.I, cfg.H), generator=g, dtype=torch.int8)
-    d["w2"] = torch.randint(-127, 128, (cfg.E, cfg.H, cfg.I), generator=g, dtype=torch.int8)
-    d["s13"] = torch.rand(cfg.E, 2 * cfg.I, generator=g, dtype=torch.float32) * 0.009 + 0.001
-    d["s2"] = torch.rand(cfg.E, cfg.H, generator=g, dtype=torch.float32) * 0.009 + 0.001
+    if cfg.zipf > 0:
+        # popularity ~ rank^-s over a fixed random ordering of the experts, added as log-prior to the logits
+        order = torch.randperm(cfg.E, generator=g)
+        pmf = torch.arange(1, cfg.E + 1, dtype=torch.float64) ** (-cfg.zipf)
+        prior = torch.empty(cfg.E, dtype=torch.float64)
+        prior[order] = torch.log(pmf / pmf.sum())
+        d["logits"] = (d["logits"].double() + prior).float()
+    if cfg.w4_group >= 0:
+        # int4 values, one per int8 (checkpoint form [E, N, K]); scales [E, N, K/g] (g = K when per channel)
+        d["w13"] = torch.randint(-8, 8, (cfg.E, 2 * cfg.I, cfg.H), generator=g, dtype=torch.int8)
+        d["w2"] = torch.randint(-8, 8, (cfg.E, cfg.H, cfg.I), generator=g, dtype=torch.int8)
+        g13 = cfg.H // cfg.w4_group if cfg.w4_group else 1
+        g2 = cfg.I // cfg.w4_group if cfg.w4_group else 1
+        d["s13"] = torch.rand(cfg.E, 2 * cfg.I, g13, generator=g, dtype=torch.float32) * 0.09 + 0.01
+        d["s2"] = torch.rand(cfg.E, cfg.H, g2, generator=g, dtype=torch.float32) * 0.09 + 0.01
+    else:
+        d["w13"] = torch.randint(-127, 128, (cfg.E, 2 * cfg.I, cfg.H), generator=g, dtype=torch.int8)
+        d["w2"] = torch.randint(-127, 128, (cfg.E, cfg.H, cfg.I), generator=g, dtype=torch.int8)
+        d["s13"] = torch.rand(cfg.E, 2 * cfg.I, generator=g, dtype=torch.float32) * 0.009 + 0.001
+        d["s2"] = torch.rand(cfg.E, cfg.H, generator=g, dtype=torch.float32) * 0.009 + 0.001
     if cfg.bias:
         d["bias"] = torch.randn(cfg.E, generator=g, dtype=torch.float32) * 0.01
     if cfg.shared:

@@ -21,6 +21,12 @@ def build_layer(cfg: LayerCfg, d: dict, device="cuda:0"):
         topk_group=cfg.topk_group if cfg.n_group > 1 else None, scoring_func=cfg.scoring,
         routed_scaling_factor=cfg.routed_scaling_factor,
         e_score_correction_bias=d["bias"].to(device) if cfg.bias else None)
+    if cfg.w4_group >= 0:
+        scheme = get_scheme_class("W4A8_DYNAMIC", "moe")(group_size=cfg.w4_group)
+        layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device)
+        layer.load_weights({"w13_weight": d["w13"].to(device), "w2_weight": d["w2"].to(device),
+                            "w13_weight_scale": d["s13"].to(device), "w2_weight_scale": d["s2"].to(device)})
+        return layer
     scheme = get_scheme_class("W8A8_DYNAMIC", "moe")()
     layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device)
     layer.load_weights({
@@ -36,6 +42,16 @@ def oracle_layer(cfg: LayerCfg, d: dict, keep_acc=True, shared=False):
     from oracle import oracle as orc
 
     kw = gating_kwargs(cfg)
+    if cfg.w4_group >= 0:
+        y, ids, _ = orc.gating_top_k(d["logits"].numpy(), cfg.k, bias=d["bias"].numpy() if cfg.bias else None,
+                                     k_group=kw["k_group"], group_count=kw["group_count"], group_select_mode=1,
+                                     renorm=kw["renorm"], norm_type=kw["norm_type"],
+                                     routed_scaling_factor=kw["routed_scaling_factor"], x_dtype="f32")
+        # scales travel as [E, N, G] in the checkpoint; the checker takes [E, G, N]
+        sg13 = np.ascontiguousarray(d["s13"].numpy().transpose(0, 2, 1))
+        sg2 = np.ascontiguousarray(d["s2"].numpy().transpose(0, 2, 1))
+        return orc.w4a8_experts_forward(bits(d["x"]), orc.f32_to_bf16(y), ids, d["w13"].numpy(), sg13,
+                                        d["w2"].numpy(), sg2, cfg.w4_group)
     sh = None
     if shared and cfg.shared:
         sh = (d["sw13"].numpy(), d["ss13"].numpy(), d["sw2"].numpy(), d["ss2"].numpy())

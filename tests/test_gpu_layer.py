@@ -80,3 +80,34 @@ def test_cpu_tensors_are_refused():
 
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         K.dynamic_quant(torch.zeros(2, 8, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("name", ["c5_small", "c5_small_perchannel"])
+def test_w4a8_layer_bit_exact(name):
+    """W4A8 variant (int4 weights, per-group or per-channel scales, Zipf-skewed routing)."""
+    cfg = CONFIGS[name]
+    print(f"w4a8 layer {name}", flush=True)
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV)
+    res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
+    torch.cuda.synchronize()
+    tr = oracle_layer(cfg, d)
+    assert np.array_equal(res.expert_tokens.cpu().numpy(), tr.expert_tokens)
+    assert np.array_equal(bits(res.routed_out), tr.out)
+
+
+def test_w4a8_packed_source_gives_the_same_tiles():
+    """The reference's packing (two int4 per byte along N, low nibble = even channel;
+    vllm_ascend/quantization/methods/w4a8.py:327-336) and the one-value-per-int8 checkpoint form
+    must cast to identical tiled storage."""
+    from vllm_ascend_amd import kernels as K
+
+    g = torch.Generator().manual_seed(1)
+    E, N, Kd = 3, 64, 128
+    w = torch.randint(-8, 8, (E, N, Kd), generator=g, dtype=torch.int8)
+    wkn = w.transpose(1, 2).contiguous()  # [E, K, N]
+    pairs = wkn.reshape(E, Kd, N // 2, 2)
+    packed = ((pairs[..., 1] << 4) | (pairs[..., 0] & 0x0F)).to(torch.int8).contiguous()  # [E, K, N/2]
+    a = K.format_cast_nz_int4(w.to(DEV), 0, N, Kd)
+    b = K.format_cast_nz_int4(packed.to(DEV), 1, N, Kd)
+    assert torch.equal(a, b)

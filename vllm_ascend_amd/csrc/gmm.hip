@@ -194,6 +194,13 @@ __global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __rest
     }
 }
 
+void launch_swiglu_requant(const float* y, const int64_t* gl, int gl_type, int E, int64_t R, int I, int8_t* q,
+                           float* qs, hipStream_t st)
+{
+    hipLaunchKernelGGL(swiglu_requant_kernel, dim3((unsigned)((R + 3) / 4)), dim3(256), 0, st, y, gl, gl_type, E, R, I,
+                       q, qs);
+}
+
 static int check_gmm(const void* x, const void* w, const int64_t* gl, int gl_type, int64_t rows, int64_t k, int64_t n,
                      int E)
 {
@@ -356,8 +363,7 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
     void* tile_ws = (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
     rc = launch_gemm_auto<EPI_SWIGLU>(a, tile_ws, st);
     if (rc != MOE355_OK) return rc;
-    hipLaunchKernelGGL(swiglu_requant_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, y, group_list,
-                       group_list_type, num_experts, rows, I, out, out_scale);
+    launch_swiglu_requant(y, group_list, group_list_type, num_experts, rows, I, out, out_scale, st);
     return launch_status();
 }
 

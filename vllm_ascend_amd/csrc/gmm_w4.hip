@@ -1,0 +1,326 @@
+// W4A8 grouped GEMM: int4 weights (two per byte), int8 activations, fp32 scales per K group.
+//
+// Weight-streaming kernel (the W4A8 shapes are HBM-bound: half the weight bytes of W8A8).
+// Storage tile = 32 channels x 64 K in 1 KiB: lane l (channel l%32, K half l/32) holds 16 bytes;
+// byte j carries, in its low nibble, w[k = 64*kb + 16*(l/32) + j] (first 32-wide K step) and in its
+// high nibble w[k + 32] (second K step).  One 16-byte load therefore feeds two MFMAs.  A nibble is
+// moved into the top half of its byte ((v << 4) & 0xF0..., v & 0xF0...), which is the signed int8
+// value 16*w: the int32 accumulator is exactly 16x the true sum and is shifted back before use.
+// Every `group` K values the accumulator is folded into fp32, f += float(acc) * scale[e, g, n], in
+// ascending group order (one wavefront owns the whole K range of its channels, so the order is the
+// sequential one), then f (+ bias) * token_scale goes through the shared epilogues.
+#include "gmm_common.h"
+
+namespace moe355 {
+
+// ------------------------------------------------------------------ format cast
+// SRC 0: int8 [E, N, K] holding one int4 value (-8..7) each (checkpoint order).
+// SRC 1: packed [E, K, N/2] bytes, low nibble = even channel (the reference's packing,
+//        vllm_ascend/quantization/methods/w4a8.py:327-336).
+template <int SRC>
+__global__ __launch_bounds__(256) void format_cast_nz_int4_kernel(const uint8_t* __restrict__ w, int64_t E, int64_t N,
+                                                                  int64_t K, uint8_t* __restrict__ out)
+{
+    const int64_t total = E * N * K / 32;  // 16-byte chunks (32 nibbles each)
+    const int64_t KB = K / 64, NB = N / 32;
+    for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+        const int lane = (int)(id & 63);
+        const int64_t tile = id >> 6;
+        const int64_t kb = tile % KB;
+        const int64_t nb = (tile / KB) % NB;
+        const int64_t e = tile / (KB * NB);
+        const int64_t n = nb * 32 + (lane & 31);
+        const int64_t k0 = kb * 64 + (lane >> 5) * 16;
+        uint32_t p[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            uint32_t lo, hi;
+            if constexpr (SRC == 0) {
+                lo = w[(e * N + n) * K + k0 + j] & 0xFu;
+                hi = w[(e * N + n) * K + k0 + 32 + j] & 0xFu;
+            } else {
+                const uint8_t b0 = w[(e * K + k0 + j) * (N / 2) + (n >> 1)];
+                const uint8_t b1 = w[(e * K + k0 + 32 + j) * (N / 2) + (n >> 1)];
+                lo = (n & 1) ? (b0 >> 4) : (b0 & 0xFu);
+                hi = (n & 1) ? (b1 >> 4) : (b1 & 0xFu);
+            }
+            p[j >> 2] |= (lo | (hi << 4)) << (8 * (j & 3));
+        }
+        *(v4i*)(out + id * 16) = (v4i){(int)p[0], (int)p[1], (int)p[2], (int)p[3]};
+    }
+}
+
+struct W4Args {
+    GmmArgs g;            // x, gl, R, K, N, E, row_scale, limit, outputs; g.w unused
+    const uint8_t* w4;    // tiled int4 storage
+    const float* gscale;  // [E, K/group, N]
+    const float* bias;    // [E, N] or null, added before the token scale
+    int group;            // K values per scale group (multiple of 64)
+};
+
+__device__ __forceinline__ v4i nib_lo(v4i v)
+{
+    return (v4i){(int)(((unsigned)v[0] << 4) & 0xF0F0F0F0u), (int)(((unsigned)v[1] << 4) & 0xF0F0F0F0u),
+                 (int)(((unsigned)v[2] << 4) & 0xF0F0F0F0u), (int)(((unsigned)v[3] << 4) & 0xF0F0F0F0u)};
+}
+__device__ __forceinline__ v4i nib_hi(v4i v)
+{
+    return (v4i){(int)((unsigned)v[0] & 0xF0F0F0F0u), (int)((unsigned)v[1] & 0xF0F0F0F0u),
+                 (int)((unsigned)v[2] & 0xF0F0F0F0u), (int)((unsigned)v[3] & 0xF0F0F0F0u)};
+}
+
+// Float twin of epilogue_run: g/u already hold sum_g float(acc_g)*scale_g (+ bias); the token scale is
+// applied here, last.
+template <int EPI>
+__device__ __forceinline__ void epilogue_run_w4(const GmmArgs& a, int64_t row, bool valid, int c0, int c1,
+                                                const float* g, const float* u)
+{
+    if (!valid) return;
+    const float rs = a.row_scale[row];
+    if constexpr (EPI == EPI_DEQUANT) {
+        v4u16 o0, o1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o0[j] = f32_to_bf16(g[j] * rs);
+            o1[j] = f32_to_bf16(u[j] * rs);
+        }
+        *(v4u16*)(a.out + row * a.N + c0) = o0;
+        *(v4u16*)(a.out + row * a.N + c1) = o1;
+    } else {
+        const int I = a.N >> 1;
+        v4f yv;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float gg = g[j] * rs;
+            float uu = u[j] * rs;
+            if (a.limit > 0.0f) {
+                gg = gg > a.limit ? a.limit : gg;
+                uu = uu > a.limit ? a.limit : uu;
+                uu = uu < -a.limit ? -a.limit : uu;
+            }
+            yv[j] = m_silu(gg) * uu;
+        }
+        *(v4f*)(a.y + row * I + c0) = yv;
+    }
+}
+
+// One wavefront per unit (expert, pair of 32-channel tiles), whole K range.
+template <int EPI, int UN>
+__global__ __launch_bounds__(256, 3) void gmm_w4_stream_kernel(W4Args p)
+{
+    const GmmArgs& a = p.g;
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int NB = a.N >> 5, KB64 = a.K >> 6;
+    const int upe = NB >> 1;
+    const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
+    if (unit >= (int64_t)a.E * upe) return;
+    const int e = (int)(unit / upe);
+    const int pi = (int)(unit % upe);
+    const int nb0 = (EPI == EPI_SWIGLU) ? pi : 2 * pi;
+    const int nb1 = (EPI == EPI_SWIGLU) ? pi + upe : 2 * pi + 1;
+
+    const uint8_t* w0 = p.w4 + (((int64_t)e * NB + nb0) * KB64) * 1024 + lane * 16;
+    const uint8_t* w1 = p.w4 + (((int64_t)e * NB + nb1) * KB64) * 1024 + lane * 16;
+    v4i a0[UN], a1[UN];
+    auto load_weights = [&](int kb) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int k = kb + u;
+            if (k < KB64) {
+                a0[u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
+                a1[u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
+            } else {
+                a0[u] = (v4i){0, 0, 0, 0};
+                a1[u] = (v4i){0, 0, 0, 0};
+            }
+        }
+    };
+    load_weights(0);
+
+    int64_t row0, row1;
+    expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
+    if (row1 > a.R) row1 = a.R;
+    if (row1 <= row0) return;
+
+    const int tok = lane & 31;
+    const int hi = lane >> 5;
+    const int steps_per_group = p.group >> 6;  // 64-wide K blocks per scale group
+    const int n_groups = a.K / p.group;
+    const float* gs = p.gscale + (int64_t)e * n_groups * a.N;
+
+    for (int64_t r0 = row0; r0 < row1; r0 += 32) {
+        const int64_t row = r0 + tok;
+        const bool valid = row < row1;
+        const int8_t* xr = a.x + row * a.K + hi * 16;
+        v16i c0 = {0}, c1 = {0};
+        float f0[16], f1[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            f0[v] = 0.0f;
+            f1[v] = 0.0f;
+        }
+        if (r0 != row0) load_weights(0);
+        int in_group = 0, grp = 0;
+        for (int kb = 0; kb < KB64; kb += UN) {
+            v4i b0[UN], b1[UN];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const bool ok = valid && (kb + u < KB64);
+                b0[u] = ok ? *(const v4i*)(xr + (kb + u) * 64) : (v4i){0, 0, 0, 0};
+                b1[u] = ok ? *(const v4i*)(xr + (kb + u) * 64 + 32) : (v4i){0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                if (kb + u < KB64) {
+                    c0 = mfma_i8(nib_lo(a0[u]), b0[u], c0);
+                    c0 = mfma_i8(nib_hi(a0[u]), b1[u], c0);
+                    c1 = mfma_i8(nib_lo(a1[u]), b0[u], c1);
+                    c1 = mfma_i8(nib_hi(a1[u]), b1[u], c1);
+                    if (++in_group == steps_per_group) {
+                        // fold this K group: f += float(acc / 16) * scale[e, grp, channel]
+                        const float* s = gs + (int64_t)grp * a.N;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int ch = 8 * q + 4 * hi;
+                            const v4f s0 = *(const v4f*)(s + nb0 * 32 + ch);
+                            const v4f s1 = *(const v4f*)(s + nb1 * 32 + ch);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                f0[4 * q + j] = f0[4 * q + j] + (float)(c0[4 * q + j] >> 4) * s0[j];
+                                f1[4 * q + j] = f1[4 * q + j] + (float)(c1[4 * q + j] >> 4) * s1[j];
+                            }
+                        }
+                        c0 = (v16i){0};
+                        c1 = (v16i){0};
+                        in_group = 0;
+                        ++grp;
+                    }
+                }
+            }
+            if (kb + UN < KB64) load_weights(kb + UN);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int ch = 8 * q + 4 * hi;
+            float g[4], u[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                g[j] = f0[4 * q + j];
+                u[j] = f1[4 * q + j];
+            }
+            if (p.bias) {
+                const v4f bg = *(const v4f*)(p.bias + (int64_t)e * a.N + nb0 * 32 + ch);
+                const v4f bu = *(const v4f*)(p.bias + (int64_t)e * a.N + nb1 * 32 + ch);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    g[j] = g[j] + bg[j];
+                    u[j] = u[j] + bu[j];
+                }
+            }
+            epilogue_run_w4<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u);
+        }
+    }
+}
+
+static int check_w4(const void* x, const void* w, const float* scale, const int64_t* gl, int gl_type, int64_t rows,
+                    int64_t k, int64_t n, int E, int64_t group)
+{
+    if (rows < 0 || k <= 0 || n <= 0 || E <= 0 || group <= 0) return MOE355_E_ARG;
+    if (gl_type != MOE355_GL_CUMSUM && gl_type != MOE355_GL_COUNT) return MOE355_E_ARG;
+    if (n % 64 != 0 || k % 64 != 0 || group % 64 != 0 || k % group != 0) return MOE355_E_SHAPE;
+    if (rows >= 0x7fffffffLL || n >= 0x7fffffffLL || k >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (rows > 0 && (!x || !w || !scale || !gl)) return MOE355_E_ARG;
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)scale & 15)) return MOE355_E_SHAPE;
+    return MOE355_OK;
+}
+
+}  // namespace moe355
+
+using namespace moe355;
+
+extern "C" int moe355_format_cast_nz_int4(const uint8_t* w, int source, int64_t num_experts, int64_t n, int64_t k,
+                                          uint8_t* out, void* stream)
+{
+    if (num_experts <= 0 || n <= 0 || k <= 0 || !w || !out) return MOE355_E_ARG;
+    if (source != 0 && source != 1) return MOE355_E_ARG;
+    if (n % 32 != 0 || k % 64 != 0) return MOE355_E_SHAPE;
+    if ((uintptr_t)out & 15) return MOE355_E_SHAPE;
+    const int64_t total = num_experts * n * k / 32;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipStream_t st = (hipStream_t)stream;
+    if (source == 0)
+        hipLaunchKernelGGL(format_cast_nz_int4_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, st, w, num_experts, n, k,
+                           out);
+    else
+        hipLaunchKernelGGL(format_cast_nz_int4_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, w, num_experts, n, k,
+                           out);
+    return launch_status();
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weight_nz4, const float* weight_scale,
+                                           int64_t group_size, const float* bias, const float* x_scale,
+                                           const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
+                                           int64_t n, int num_experts, float swiglu_limit, int8_t* out,
+                                           float* out_scale, void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_w4(x, weight_nz4, weight_scale, group_list, group_list_type, rows, k, n, num_experts, group_size);
+    if (rc != MOE355_OK) return rc;
+    if (rows == 0) return MOE355_OK;
+    if (!x_scale || !out || !out_scale) return MOE355_E_ARG;
+    if (((uintptr_t)bias & 15) || ((uintptr_t)out & 3)) return MOE355_E_SHAPE;
+    const size_t ybytes = ((size_t)rows * (size_t)(n / 2) * 4 + 255) & ~(size_t)255;
+    if (!workspace || ((uintptr_t)workspace & 255) || workspace_bytes < ybytes) return MOE355_E_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    W4Args p = {};
+    p.g.x = x;
+    p.g.gl = group_list;
+    p.g.gl_type = group_list_type;
+    p.g.R = rows;
+    p.g.K = (int)k;
+    p.g.N = (int)n;
+    p.g.E = num_experts;
+    p.g.row_scale = x_scale;
+    p.g.limit = swiglu_limit;
+    p.g.y = (float*)workspace;
+    p.w4 = weight_nz4;
+    p.gscale = weight_scale;
+    p.bias = bias;
+    p.group = (int)group_size;
+    const int64_t units = (int64_t)num_experts * (n / 64);
+    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU, 4>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
+    launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
+    return launch_status();
+}
+
+extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4, const float* scale,
+                                      int64_t group_size, const float* bias, const float* per_token_scale,
+                                      const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
+                                      int64_t n, int num_experts, void* out, int out_dtype, void* stream)
+{
+    int rc = check_w4(x, weight_nz4, scale, group_list, group_list_type, rows, k, n, num_experts, group_size);
+    if (rc != MOE355_OK) return rc;
+    if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (rows == 0) return MOE355_OK;
+    if (!per_token_scale || !out) return MOE355_E_ARG;
+    if (((uintptr_t)bias & 15) || ((uintptr_t)out & 7)) return MOE355_E_SHAPE;
+    W4Args p = {};
+    p.g.x = x;
+    p.g.gl = group_list;
+    p.g.gl_type = group_list_type;
+    p.g.R = rows;
+    p.g.K = (int)k;
+    p.g.N = (int)n;
+    p.g.E = num_experts;
+    p.g.row_scale = per_token_scale;
+    p.g.out = (uint16_t*)out;
+    p.w4 = weight_nz4;
+    p.gscale = scale;
+    p.bias = bias;
+    p.group = (int)group_size;
+    const int64_t units = (int64_t)num_experts * (n / 64);
+    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT, 4>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)stream, p);
+    return launch_status();
+}

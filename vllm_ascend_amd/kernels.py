@@ -206,3 +206,48 @@ def token_unpermute(permuted, sorted_indices, probs, residual=None):
                                      _ptr(probs), T, k, H, R, _ptr(residual), _ptr(out), _stream(permuted)),
           "moe355_token_unpermute")
     return out
+
+
+# ------------------------------------------------------------------ W4A8 (int4 weights)
+def format_cast_nz_int4(w: torch.Tensor, source: int, n: int, k: int) -> torch.Tensor:
+    """source 0: int8 [E, N, K] with one int4 value per byte; source 1: packed bytes [E, K, N/2]
+    (low nibble = even channel).  Returns the tiled int4 storage as uint8 [E, N*K/2]."""
+    w = _dev(w, "weight")
+    lib = _lib.load()
+    E = w.shape[0]
+    out = torch.empty((E, n * k // 2), dtype=torch.uint8, device=w.device)
+    check(lib.moe355_format_cast_nz_int4(_ptr(w), source, E, n, k, _ptr(out), _stream(w)),
+          "moe355_format_cast_nz_int4")
+    return out
+
+
+def gmm1_swiglu_quant_w4(x, weight_nz4, weight_scale, group_size, x_scale, group_list, group_list_type, n, k,
+                         bias=None, swiglu_limit=0.0):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows = x.shape[0]
+    E = weight_nz4.shape[0]
+    dev = x.device
+    out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
+    out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    ws = _workspace(rows * (n // 2) * 4 + 256, dev)
+    check(lib.moe355_gmm1_swiglu_quant_w4(_ptr(x), _ptr(_dev(weight_nz4, "weight")),
+                                          _ptr(_dev(weight_scale, "weight_scale")), group_size,
+                                          _ptr(bias), _ptr(_dev(x_scale, "x_scale")), _ptr(_gl(group_list)),
+                                          _gl_type(group_list_type), rows, k, n, E, float(swiglu_limit), _ptr(out),
+                                          _ptr(out_scale), _ptr(ws), ws.numel(), _stream(x)),
+          "moe355_gmm1_swiglu_quant_w4")
+    return out, out_scale
+
+
+def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_list, group_list_type, n, k, bias=None):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    rows = x.shape[0]
+    E = weight_nz4.shape[0]
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
+    check(lib.moe355_gmm2_dequant_w4(_ptr(x), _ptr(_dev(weight_nz4, "weight")), _ptr(_dev(scale, "scale")),
+                                     group_size, _ptr(bias), _ptr(_dev(per_token_scale, "per_token_scale")),
+                                     _ptr(_gl(group_list)), _gl_type(group_list_type), rows, k, n, E, _ptr(out),
+                                     DT_BF16, _stream(x)), "moe355_gmm2_dequant_w4")
+    return out
