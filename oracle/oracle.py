@@ -339,6 +339,20 @@ def experts_forward(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2, *, keep_acc
     return tr
 
 
+def shared_expert_forward(x_bf16, w13, s13, w2, s2) -> np.ndarray:
+    """Dense W8A8 MLP every token goes through, op for op as the reference's shared expert
+    (vllm_ascend/ops/fused_moe/shared_experts.py:254-301): dynamic quant -> int32 matmul ->
+    dequant_swiglu_quant (weight scale first, then activation scale) -> matmul with per-token
+    scale -> bf16.  w13 [2I,H], s13 [2I], w2 [H,I], s2 [H]."""
+    T = x_bf16.shape[0]
+    one = np.array([T], dtype=np.int64)
+    xq, sx = dynamic_quant(x_bf16)
+    acc1 = gmm_i32(xq, w13[None], one)
+    q1, s1 = dequant_swiglu_quant(acc1, s13, sx, activate_left=True)
+    acc2 = gmm_i32(q1, w2[None], one)
+    return gmm2_dequant(acc2, s1, s2[None], one)
+
+
 def moe_layer(x_bf16, logits_f32, w13, s13, w2, s2, *, top_k, bias=None, k_group=1, group_count=1, renorm=1,
               norm_type=0, routed_scaling_factor=1.0, keep_acc=True, shared=None) -> LayerTrace:
     """router logits -> final bf16, all stages.  ``shared`` = (w13s[1,2I,H], s13s[1,2I], w2s[1,H,I], s2s[1,H]):
@@ -351,11 +365,8 @@ def moe_layer(x_bf16, logits_f32, w13, s13, w2, s2, *, top_k, bias=None, k_group
     extra = {}
     if shared is not None:
         sw13, ss13, sw2, ss2 = shared
-        T = x_bf16.shape[0]
-        ones = f32_to_bf16(np.ones((T, 1), dtype=np.float32))
-        st = experts_forward(x_bf16, ones, np.zeros((T, 1), dtype=np.int32), sw13, ss13, sw2, ss2, keep_acc=False)
-        add = st.out
-        extra["shared_out"] = st.out
+        add = shared_expert_forward(x_bf16, sw13[0], ss13[0], sw2[0], ss2[0])
+        extra["shared_out"] = add
     tr = experts_forward(x_bf16, w_bf16, ids, w13, s13, w2, s2, keep_acc=keep_acc, add_bf16=add)
     tr.extra.update(extra)
     return tr

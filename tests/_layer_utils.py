@@ -7,7 +7,7 @@ import torch
 from _inputs import LayerCfg, bits, gating_kwargs
 
 
-def build_layer(cfg: LayerCfg, d: dict, device="cuda:0"):
+def build_layer(cfg: LayerCfg, d: dict, device="cuda:0", shared=False, overlap=False):
     from vllm_ascend_amd.fused_moe.contracts import FusedMoEConfig
     from vllm_ascend_amd.fused_moe.layer import AscendRoutedExperts
     from vllm_ascend_amd.fused_moe.router import AscendFusedTopKRouter
@@ -21,6 +21,12 @@ def build_layer(cfg: LayerCfg, d: dict, device="cuda:0"):
         topk_group=cfg.topk_group if cfg.n_group > 1 else None, scoring_func=cfg.scoring,
         routed_scaling_factor=cfg.routed_scaling_factor,
         e_score_correction_bias=d["bias"].to(device) if cfg.bias else None)
+    shared_experts = None
+    if shared and cfg.shared:
+        from vllm_ascend_amd.fused_moe.shared_experts import AscendSharedExperts
+
+        shared_experts = AscendSharedExperts(d["sw13"][0].to(device), d["ss13"][0].to(device), d["sw2"][0].to(device),
+                                             d["ss2"][0].to(device), multistream_overlap=overlap)
     if cfg.w4_group >= 0:
         scheme = get_scheme_class("W4A8_DYNAMIC", "moe")(group_size=cfg.w4_group)
         layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device)
@@ -28,7 +34,8 @@ def build_layer(cfg: LayerCfg, d: dict, device="cuda:0"):
                             "w13_weight_scale": d["s13"].to(device), "w2_weight_scale": d["s2"].to(device)})
         return layer
     scheme = get_scheme_class("W8A8_DYNAMIC", "moe")()
-    layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device)
+    layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device,
+                                shared_experts=shared_experts)
     layer.load_weights({
         "w13_weight": d["w13"].to(device), "w2_weight": d["w2"].to(device),
         "w13_weight_scale": d["s13"].to(device), "w2_weight_scale": d["s2"].to(device),

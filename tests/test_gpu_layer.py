@@ -111,3 +111,19 @@ def test_w4a8_packed_source_gives_the_same_tiles():
     a = K.format_cast_nz_int4(w.to(DEV), 0, N, Kd)
     b = K.format_cast_nz_int4(packed.to(DEV), 1, N, Kd)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_layer_with_shared_expert(overlap):
+    """DeepSeek-V3-shaped structure (sigmoid, groups, bias, scaling factor) plus the shared expert, whose
+    output is added inside the combine; with and without the second stream."""
+    cfg = CONFIGS["c4_small"]
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV, shared=True, overlap=overlap)
+    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+    for _ in range(3):  # repeated calls: the side-stream fences must hold every time
+        res = layer.forward_impl(x, logits)
+    torch.cuda.synchronize()
+    tr = oracle_layer(cfg, d, shared=True)
+    assert np.array_equal(bits(res.shared_out), tr.extra["shared_out"])
+    assert np.array_equal(bits(res.routed_out), tr.out)

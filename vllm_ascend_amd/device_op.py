@@ -97,10 +97,10 @@ class MI355XDeviceAdaptor:
             output_dtype=fallback_output_dtype)[0]
 
     @staticmethod
-    def npu_moe_token_unpermute(permuted_tokens, sorted_indices, probs):
+    def npu_moe_token_unpermute(permuted_tokens, sorted_indices, probs, residual=None):
         # the kernel takes |index| itself (the reference passes torch.abs(sorted_indices))
         return npu_ops.npu_moe_token_unpermute(permuted_tokens=permuted_tokens, sorted_indices=sorted_indices,
-                                               probs=probs)
+                                               probs=probs, residual=residual)
 
 
 DeviceOperator = MI355XDeviceAdaptor

@@ -99,6 +99,10 @@ class MoEFusedExpertsInput:
     need_trans: bool = False
     dynamic_eplb: bool = False
     lora_context: Any = None
+    # not in the reference: output of the shared expert, added in fp32 inside the combine kernel
+    # (the reference returns both tensors and upstream vLLM adds them)
+    shared_out: torch.Tensor | None = None
+    shared_experts: Any = None
 
 
 @dataclass(frozen=True)
@@ -159,6 +163,8 @@ class FusedExpertsResult:
     before_combine_evt: Any = None
     group_list_type: int = 1
     expert_tokens: torch.Tensor | None = None
+    # set when a shared expert ran with the layer: its output is already added into routed_out
+    shared_out: torch.Tensor | None = None
 
 
 def build_fused_experts_input(*, hidden_states, topk_weights, topk_ids, w1, w2, quant_type: QuantType,
@@ -167,7 +173,8 @@ def build_fused_experts_input(*, hidden_states, topk_weights, topk_ids, w1, w2, 
                               activation="silu", need_trans: bool = False, w1_bias=None, w2_bias=None,
                               comm_quant_mode=None, is_per_channel_weight: bool = False, w4_group_size: int = 0,
                               w1_scale=None, w2_scale=None, w1_scale_bias=None, w2_scale_bias=None, w1_offset=None,
-                              w2_offset=None, lora_context=None) -> MoEFusedExpertsInput:
+                              w2_offset=None, lora_context=None, shared_out=None,
+                              shared_experts=None) -> MoEFusedExpertsInput:
     return MoEFusedExpertsInput(
         hidden_states=hidden_states,
         topk_weights=topk_weights,
@@ -184,6 +191,8 @@ def build_fused_experts_input(*, hidden_states, topk_weights, topk_ids, w1, w2, 
         need_trans=need_trans,
         dynamic_eplb=dynamic_eplb,
         lora_context=lora_context,
+        shared_out=shared_out,
+        shared_experts=shared_experts,
     )
 
 

@@ -15,8 +15,9 @@ from .router import AscendFusedTopKRouter
 
 class AscendRoutedExperts(torch.nn.Module):
     def __init__(self, moe_config: FusedMoEConfig, quant_method: AscendMoEScheme, router: AscendFusedTopKRouter,
-                 params_dtype: torch.dtype = torch.bfloat16, device="cuda"):
+                 params_dtype: torch.dtype = torch.bfloat16, device="cuda", shared_experts=None):
         super().__init__()
+        self.shared_experts = shared_experts
         self.moe_config = moe_config
         self.quant_method = quant_method
         self.router = router
@@ -46,7 +47,7 @@ class AscendRoutedExperts(torch.nn.Module):
     def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
         hidden_states, router_logits, _, _ = self.moe_comm_method.prepare(hidden_states, router_logits)
         topk_weights, topk_ids = self.router.select_experts(hidden_states, router_logits)
-        result = self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, None, None)
+        result = self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
         result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
         return result
 

@@ -63,8 +63,13 @@ class AllGatherCommImpl:
         mlp_out, before_gmm2_evt = unified_apply_mlp(mlp_compute_input=build_mlp_compute_input(
             fused_experts_input=f, token_dispatch_output=dispatched, moe_config=self.moe_config))
         before_combine_evt = stream.record_event() if stream else None
+        shared_out = f.shared_out
+        if f.shared_experts is not None and shared_out is not None:
+            f.shared_experts.wait()  # side-stream MLP must be done before its output is added
         routed_out = self.token_dispatcher.token_combine(hidden_states=mlp_out,
-                                                         combine_metadata=dispatched.combine_metadata)
+                                                         combine_metadata=dispatched.combine_metadata,
+                                                         residual=shared_out)
         return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
                                   before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
-                                  group_list_type=dispatched.group_list_type, expert_tokens=dispatched.group_list)
+                                  group_list_type=dispatched.group_list_type, expert_tokens=dispatched.group_list,
+                                  shared_out=shared_out)

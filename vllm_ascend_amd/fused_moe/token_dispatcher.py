@@ -65,11 +65,13 @@ class TokenDispatcherWithAllGather:
                                                          restore_shape=restore_shape),
         )
 
-    def token_combine(self, hidden_states, combine_metadata: MoEAllGatherCombineMetadata, bias=None):
+    def token_combine(self, hidden_states, combine_metadata: MoEAllGatherCombineMetadata, bias=None, residual=None):
+        """``residual`` (not in the reference): a [T, H] tensor added in fp32 before the bf16 rounding --
+        the shared-expert output, which upstream vLLM would add afterwards."""
         assert bias is None, "bias is not supported by the combine"
         out = DeviceOperator.npu_moe_token_unpermute(permuted_tokens=hidden_states,
                                                      sorted_indices=combine_metadata.expanded_row_idx,
-                                                     probs=combine_metadata.topk_weights)
+                                                     probs=combine_metadata.topk_weights, residual=residual)
         if len(combine_metadata.restore_shape) == 3:
             out = out.view(combine_metadata.restore_shape)
         return out

@@ -88,7 +88,48 @@ def npu_grouped_matmul(x, weight, *, bias=None, scale=None, offset=None, antiqua
     return [out]
 
 
-def npu_moe_token_unpermute(permuted_tokens, sorted_indices, probs=None, padded_mode=False, restore_shape=None):
+def npu_moe_token_unpermute(permuted_tokens, sorted_indices, probs=None, padded_mode=False, restore_shape=None,
+                            residual=None):
+    """``residual`` (extension): [T, H] tensor added in fp32 before the output is rounded."""
     if padded_mode:
         raise NotImplementedError("npu_moe_token_unpermute: padded_mode is not supported")
-    return kernels.token_unpermute(permuted_tokens, sorted_indices, probs)
+    return kernels.token_unpermute(permuted_tokens, sorted_indices, probs, residual)
+
+
+_ONE_GROUP: dict = {}
+
+
+def _single_group_list(rows: int, device) -> torch.Tensor:
+    key = (rows, str(device))
+    t = _ONE_GROUP.get(key)
+    if t is None:
+        t = torch.tensor([rows], dtype=torch.int64, device=device)
+        _ONE_GROUP[key] = t
+    return t
+
+
+def npu_quant_matmul(x1, x2, scale, *, offset=None, pertoken_scale=None, bias=None, output_dtype=None):
+    """Dense int8 x int8 matmul as the shared expert uses it
+    (``vllm_ascend/ops/fused_moe/shared_experts.py:262-301``): ``x1`` int8 ``[M, K]``, ``x2`` int8
+    ``[K, N]`` in the tiled storage of :func:`npu_format_cast`, ``scale`` ``[N]``.
+    ``output_dtype=torch.int32``: the raw accumulators (scales ignored, as in the reference call);
+    ``output_dtype=torch.bfloat16``: ``bf16((acc * pertoken_scale[m]) * scale[n])``.
+    One expert that owns every row: the grouped kernels with E = 1."""
+    if offset is not None or bias is not None:
+        raise NotImplementedError("npu_quant_matmul: offset / bias are not supported")
+    if x1.dtype != torch.int8 or x2.dtype != torch.int8 or x2.dim() != 2:
+        raise NotImplementedError("npu_quant_matmul: int8 [M, K] x int8 [K, N] only")
+    lead = x1.shape[:-1]
+    a = x1.reshape(-1, x1.shape[-1])
+    k, n = x2.shape
+    gl = _single_group_list(a.shape[0], a.device)
+    w = x2.unsqueeze(0)
+    if output_dtype == torch.int32:
+        out = kernels.gmm_i32(a, w, gl, 0, n, k)
+    elif output_dtype in (None, torch.bfloat16):
+        if pertoken_scale is None:
+            raise NotImplementedError("npu_quant_matmul: bf16 output needs pertoken_scale")
+        out = kernels.gmm2_dequant(a, w, scale.to(torch.float32).reshape(1, n), pertoken_scale.reshape(-1), gl, 0, n, k)
+    else:
+        raise NotImplementedError(f"npu_quant_matmul: output_dtype {output_dtype} is not supported")
+    return out.reshape(lead + (n,))

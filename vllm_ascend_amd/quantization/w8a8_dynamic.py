@@ -72,6 +72,10 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         moe_comm_method = _EXTRA_CTX.moe_comm_method
         if moe_comm_method is None:
             raise RuntimeError("no MoE communication method is set up (call setup_moe_comm_method first)")
+        shared_out = None
+        if shared_experts is not None:
+            # the shared expert sees the same hidden states unless the caller hands over others
+            shared_out = shared_experts(x if shared_experts_input is None else shared_experts_input)
         return moe_comm_method.fused_experts(
             fused_experts_input=build_fused_experts_input(
                 hidden_states=x,
@@ -87,6 +91,8 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 apply_router_weight_on_input=getattr(layer, "apply_router_weight_on_input", False),
                 pertoken_scale=getattr(layer, "ascend_pertoken_scale", None),
                 activation=getattr(layer, "activation", "silu"),
+                shared_out=shared_out,
+                shared_experts=shared_experts,
                 w1_scale=[layer.w13_weight_scale_fp32],
                 w2_scale=[layer.w2_weight_scale_fp32],
             ))
