@@ -148,6 +148,16 @@ int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const flo
                              int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
                              float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Per-expert tensors: weight_nz_list / weight_scale_list are DEVICE arrays of num_experts pointers,
+ * entry e pointing at expert e's tiled [N, K] weights / its [N] fp32 scales (experts that can be
+ * swapped one by one, as dynamic expert load balancing does).  Stands in for
+ * torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz_tensor_list (csrc/torch_binding.cpp:2039-2045). */
+int moe355_gmm1_swiglu_quant_list(const int8_t *x, const int8_t *const *weight_nz_list,
+                                  const float *const *weight_scale_list, const float *x_scale,
+                                  const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
+                                  int num_experts, float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
 /* W4A8 variant: int4 weights (moe355_format_cast_nz_int4 storage), fp32 scales per group of
  * `group_size` values along K: weight_scale [E, K/group_size, N] (group_size == K: per channel).
  *   f = (sum_g float(acc_g) * weight_scale[e, g, col] (g ascending) + bias[e, col]) * x_scale[row]
@@ -175,6 +185,13 @@ int moe355_gmm2_dequant(const int8_t *x, const int8_t *weight_nz, const float *s
                         const int64_t *group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
                         int num_experts, void *out, int out_dtype, void *workspace, size_t workspace_bytes,
                         void *stream);
+
+/* Per-expert tensor form of the down projection (weight list of torch_npu.npu_grouped_matmul,
+ * vllm_ascend/device/device_op.py:280-291 with `weight` a list of E tensors). */
+int moe355_gmm2_dequant_list(const int8_t *x, const int8_t *const *weight_nz_list, const float *const *scale_list,
+                             const float *per_token_scale, const int64_t *group_list, int group_list_type,
+                             int64_t rows, int64_t k, int64_t n, int num_experts, void *out, int out_dtype,
+                             void *workspace, size_t workspace_bytes, void *stream);
 
 /* W4A8 down projection:
  *   out[row, col] = bf16( (sum_g float(acc_g) * scale[e, g, col] + bias[e, col]) * per_token_scale[row] )

@@ -127,3 +127,28 @@ def test_layer_with_shared_expert(overlap):
     tr = oracle_layer(cfg, d, shared=True)
     assert np.array_equal(bits(res.shared_out), tr.extra["shared_out"])
     assert np.array_equal(bits(res.routed_out), tr.out)
+
+
+def test_layer_with_per_expert_weight_lists():
+    """dynamic-EPLB form: every expert's weights and scales are separate tensors; swapping two experts'
+    tensors in place must swap what they compute."""
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV, dynamic_eplb=True)
+    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+    res = layer.forward_impl(x, logits)
+    torch.cuda.synchronize()
+    tr = oracle_layer(cfg, d)
+    assert np.array_equal(bits(res.routed_out), tr.out)
+    # swap experts 0 and 1 in the lists AND in the checker's inputs
+    views = layer.quant_method.get_eplb_weight_views(layer)
+    for lst in views:
+        lst[0], lst[1] = lst[1], lst[0]
+    for name in ("w13", "w2", "s13", "s2"):
+        t = d[name].clone()
+        t[0], t[1] = d[name][1], d[name][0]
+        d[name] = t
+    res2 = layer.forward_impl(x, logits)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(res2.routed_out), oracle_layer(cfg, d).out)
+    assert not torch.equal(res.routed_out, res2.routed_out)

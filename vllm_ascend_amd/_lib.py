@@ -39,6 +39,11 @@ PROTOTYPES = {
     "moe355_gmm1_swiglu_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "moe355_gmm1_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
                                          c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "moe355_gmm1_swiglu_quant_list": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                                              c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p, c_size_t,
+                                              c_void_p]),
+    "moe355_gmm2_dequant_list": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                                         c_int64, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "moe355_gmm2_dequant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "moe355_gmm2_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64,
                                     c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),

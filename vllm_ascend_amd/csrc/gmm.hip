@@ -68,8 +68,9 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     const int kb_begin = (KB * ks) / KSPLIT;
     const int kb_end = (KB * (ks + 1)) / KSPLIT;
 
-    const int8_t* w0 = a.w + (((int64_t)e * NB + nb0) * KB) * 1024 + lane * 16;
-    const int8_t* w1 = a.w + (((int64_t)e * NB + nb1) * KB) * 1024 + lane * 16;
+    const int8_t* we = expert_weights(a, e);
+    const int8_t* w0 = we + ((int64_t)nb0 * KB) * 1024 + lane * 16;
+    const int8_t* w1 = we + ((int64_t)nb1 * KB) * 1024 + lane * 16;
 
     // The weight addresses depend only on the unit, so the first batch of weight tiles is requested
     // before the expert's row range is known: the group-list lookup hides behind the HBM latency.
@@ -330,16 +331,17 @@ extern "C" size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, in
     return (((size_t)rows * (size_t)(n / 2) * 4 + 255) & ~(size_t)255) + tiled_ws_max(rows, num_experts);
 }
 
-extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz, const float* weight_scale,
-                                        const float* x_scale, const int64_t* group_list, int group_list_type,
-                                        int64_t rows, int64_t k, int64_t n, int num_experts, float swiglu_limit,
-                                        int8_t* out, float* out_scale, void* workspace, size_t workspace_bytes,
-                                        void* stream)
+static int gmm1_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* const* weight_list,
+                     const float* weight_scale, const float* const* scale_list, const float* x_scale,
+                     const int64_t* group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
+                     int num_experts, float swiglu_limit, int8_t* out, float* out_scale, void* workspace,
+                     size_t workspace_bytes, void* stream)
 {
-    int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
+    const void* wany = weight_list ? (const void*)weight_list : (const void*)weight_nz;
+    int rc = check_gmm(x, wany, group_list, group_list_type, rows, k, n, num_experts);
     if (rc != MOE355_OK) return rc;
     if (rows == 0) return MOE355_OK;
-    if (!weight_scale || !x_scale || !out || !out_scale) return MOE355_E_ARG;
+    if ((!weight_scale && !scale_list) || !x_scale || !out || !out_scale) return MOE355_E_ARG;
     if (((uintptr_t)weight_scale & 15) || ((uintptr_t)out & 3)) return MOE355_E_SHAPE;
     if (!workspace || ((uintptr_t)workspace & 255) ||
         workspace_bytes < moe355_gmm1_swiglu_quant_workspace(rows, n, k, num_experts))
@@ -350,6 +352,7 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
     GmmArgs a = {};
     a.x = x;
     a.w = weight_nz;
+    a.w_list = weight_list;
     a.gl = group_list;
     a.gl_type = group_list_type;
     a.R = rows;
@@ -358,6 +361,7 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
     a.E = num_experts;
     a.row_scale = x_scale;
     a.ch_scale = weight_scale;
+    a.s_list = scale_list;
     a.limit = swiglu_limit;
     a.y = y;
     void* tile_ws = (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
@@ -365,6 +369,27 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
     if (rc != MOE355_OK) return rc;
     launch_swiglu_requant(y, group_list, group_list_type, num_experts, rows, I, out, out_scale, st);
     return launch_status();
+}
+
+extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz, const float* weight_scale,
+                                        const float* x_scale, const int64_t* group_list, int group_list_type,
+                                        int64_t rows, int64_t k, int64_t n, int num_experts, float swiglu_limit,
+                                        int8_t* out, float* out_scale, void* workspace, size_t workspace_bytes,
+                                        void* stream)
+{
+    return gmm1_impl(x, weight_nz, nullptr, weight_scale, nullptr, x_scale, group_list, group_list_type, rows, k, n,
+                     num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_list(const int8_t* x, const int8_t* const* weight_nz_list,
+                                             const float* const* weight_scale_list, const float* x_scale,
+                                             const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
+                                             int64_t n, int num_experts, float swiglu_limit, int8_t* out,
+                                             float* out_scale, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!weight_nz_list || !weight_scale_list) return MOE355_E_ARG;
+    return gmm1_impl(x, nullptr, weight_nz_list, nullptr, weight_scale_list, x_scale, group_list, group_list_type,
+                     rows, k, n, num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream);
 }
 
 extern "C" size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
@@ -375,23 +400,25 @@ extern "C" size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t
     return tiled_ws_max(rows, num_experts);
 }
 
-extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, const float* scale,
-                                   const float* per_token_scale, const int64_t* group_list, int group_list_type,
-                                   int64_t rows, int64_t k, int64_t n, int num_experts, void* out, int out_dtype,
-                                   void* workspace, size_t workspace_bytes, void* stream)
+static int gmm2_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* const* weight_list, const float* scale,
+                     const float* const* scale_list, const float* per_token_scale, const int64_t* group_list,
+                     int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts, void* out,
+                     int out_dtype, void* workspace, size_t workspace_bytes, void* stream)
 {
-    int rc = check_gmm(x, weight_nz, group_list, group_list_type, rows, k, n, num_experts);
+    const void* wany = weight_list ? (const void*)weight_list : (const void*)weight_nz;
+    int rc = check_gmm(x, wany, group_list, group_list_type, rows, k, n, num_experts);
     if (rc != MOE355_OK) return rc;
     if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
     if (rows > 0 && (!workspace || ((uintptr_t)workspace & 255) ||
                      workspace_bytes < moe355_gmm2_dequant_workspace(rows, n, k, num_experts)))
         return MOE355_E_WORKSPACE;
     if (rows == 0) return MOE355_OK;
-    if (!scale || !per_token_scale || !out) return MOE355_E_ARG;
-    if (((uintptr_t)scale & 15) || ((uintptr_t)out & 7)) return MOE355_E_SHAPE;
+    if ((!scale && !scale_list) || !per_token_scale || !out) return MOE355_E_ARG;
+    if (((uintptr_t)scale & 15) || ((uintptr_t)out & 15)) return MOE355_E_SHAPE;
     GmmArgs a = {};
     a.x = x;
     a.w = weight_nz;
+    a.w_list = weight_list;
     a.gl = group_list;
     a.gl_type = group_list_type;
     a.R = rows;
@@ -400,6 +427,27 @@ extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, con
     a.E = num_experts;
     a.row_scale = per_token_scale;
     a.ch_scale = scale;
+    a.s_list = scale_list;
     a.out = (uint16_t*)out;
     return launch_gemm_auto<EPI_DEQUANT>(a, workspace, (hipStream_t)stream);
+}
+
+extern "C" int moe355_gmm2_dequant(const int8_t* x, const int8_t* weight_nz, const float* scale,
+                                   const float* per_token_scale, const int64_t* group_list, int group_list_type,
+                                   int64_t rows, int64_t k, int64_t n, int num_experts, void* out, int out_dtype,
+                                   void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gmm2_impl(x, weight_nz, nullptr, scale, nullptr, per_token_scale, group_list, group_list_type, rows, k, n,
+                     num_experts, out, out_dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int moe355_gmm2_dequant_list(const int8_t* x, const int8_t* const* weight_nz_list,
+                                        const float* const* scale_list, const float* per_token_scale,
+                                        const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
+                                        int64_t n, int num_experts, void* out, int out_dtype, void* workspace,
+                                        size_t workspace_bytes, void* stream)
+{
+    if (!weight_nz_list || !scale_list) return MOE355_E_ARG;
+    return gmm2_impl(x, nullptr, weight_nz_list, nullptr, scale_list, per_token_scale, group_list, group_list_type,
+                     rows, k, n, num_experts, out, out_dtype, workspace, workspace_bytes, stream);
 }

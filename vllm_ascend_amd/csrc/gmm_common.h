@@ -25,12 +25,26 @@ struct GmmArgs {
     int K, N, E;
     const float* row_scale; // [R]     token scale
     const float* ch_scale;  // [E, N]  channel scale
+    // per-expert tensors (weights that can be swapped expert by expert): device arrays of E pointers;
+    // when set they replace w / ch_scale
+    const int8_t* const* w_list;
+    const float* const* s_list;
     float limit;            // swiglu clamp
     // outputs
     int32_t* acc;           // EPI_I32   [R, N]
     float* y;               // EPI_SWIGLU [R, N/2] fp32 SwiGLU values
     uint16_t* out;          // EPI_DEQUANT [R, N] bf16
 };
+
+// tiled weights / channel scales of expert e
+__device__ __forceinline__ const int8_t* expert_weights(const GmmArgs& a, int e)
+{
+    return a.w_list ? a.w_list[e] : a.w + (int64_t)e * a.N * a.K;
+}
+__device__ __forceinline__ const float* expert_scales(const GmmArgs& a, int e)
+{
+    return a.s_list ? a.s_list[e] : a.ch_scale + (int64_t)e * a.N;
+}
 
 __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c)
 {
@@ -60,7 +74,7 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
     } else if constexpr (EPI == EPI_DEQUANT) {
         if (!valid) return;
         const float rs = a.row_scale[row];
-        const float* cs = a.ch_scale + (int64_t)e * a.N;
+        const float* cs = expert_scales(a, e);
         const v4f s0 = *(const v4f*)(cs + n0 + ch);
         const v4f s1 = *(const v4f*)(cs + n1 + ch);
         v4u16 o0, o1;
@@ -76,7 +90,7 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
         if (!valid) return;
         const int I = a.N >> 1;
         const float rs = a.row_scale[row];
-        const float* cs = a.ch_scale + (int64_t)e * a.N;
+        const float* cs = expert_scales(a, e);
         const v4f sg = *(const v4f*)(cs + n0 + ch);
         const v4f su = *(const v4f*)(cs + n1 + ch);
         v4f yv;

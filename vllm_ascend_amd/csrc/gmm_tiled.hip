@@ -119,8 +119,9 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
         nb1 = nb0 + 1;
     }
     const bool have = (EPI == EPI_SWIGLU) ? (nb0 < half_tiles) : (nb1 < NB);
-    const int8_t* w0 = a.w + (((int64_t)e * NB + (have ? nb0 : 0)) * KB) * 1024 + lane * 16;
-    const int8_t* w1 = a.w + (((int64_t)e * NB + (have ? nb1 : 0)) * KB) * 1024 + lane * 16;
+    const int8_t* we = expert_weights(a, e);
+    const int8_t* w0 = we + ((int64_t)(have ? nb0 : 0) * KB) * 1024 + lane * 16;
+    const int8_t* w1 = we + ((int64_t)(have ? nb1 : 0) * KB) * 1024 + lane * 16;
 
     const int n_iter = a.K / kBK;
 
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
     int8_t* patch = lds_raw + wave * (PATCHES * 32 * ROWB);
     const int tok = lane & 31;
     const int hi = lane >> 5;
-    const float* cs = a.ch_scale ? a.ch_scale + (int64_t)e * a.N : nullptr;
+    const float* cs = (a.ch_scale || a.s_list) ? expert_scales(a, e) : nullptr;
     v4f s0[4], s1[4];
     if constexpr (EPI != EPI_I32) {
 #pragma unroll

@@ -107,25 +107,19 @@ def _gmm_swiglu_quant_nz_meta(x, weight, weight_scale, x_scale, group_list, *, b
             x.new_empty((), dtype=torch.float32))
 
 
-def _stack_list(tensors):
-    """Per-expert tensors -> one [E, ...] tensor (no copy when they are consecutive views of one buffer)."""
-    first = tensors[0]
-    step = first.numel() * first.element_size()
-    base = first.data_ptr()
-    if all(t.is_contiguous() and t.data_ptr() == base + i * step and t.shape == first.shape
-           for i, t in enumerate(tensors)):
-        storage_view = torch.empty(0, dtype=first.dtype, device=first.device)
-        storage_view.set_(first.untyped_storage(), first.storage_offset(), (len(tensors),) + tuple(first.shape))
-        return storage_view
-    return torch.stack(list(tensors))
-
-
 def _gmm_swiglu_quant_nz_tensor_list(x, weight, weight_scale, x_scale, group_list, *, bias=None, offset=None,
                                      swiglu_limit=0.0):
+    """Per-expert weight / scale tensors (each [K, N] tiled / [N]); the kernels follow a device table of
+    their addresses, nothing is stacked or copied."""
     _reject_unsupported(bias, offset)
-    w = _stack_list(weight)
-    s = _stack_list(weight_scale)
-    out, out_scale, _ = _gmm_swiglu_quant_nz(x, w, s, x_scale, group_list, swiglu_limit=swiglu_limit)
+    if len(weight) != len(weight_scale) or len(weight) == 0:
+        raise RuntimeError("weight and weight_scale must be lists of the same non-zero length")
+    if len(weight) == 1 and weight[0].dim() == 3:
+        out, out_scale, _ = _gmm_swiglu_quant_nz(x, weight[0], weight_scale[0], x_scale, group_list,
+                                                  swiglu_limit=swiglu_limit)
+    else:
+        scales = [s if s.dtype == torch.float32 else s.to(torch.float32) for s in weight_scale]
+        out, out_scale = kernels.gmm1_swiglu_quant_list(x, list(weight), scales, x_scale, group_list, 0, swiglu_limit)
     return out, out_scale, x.new_empty((x.shape[0],), dtype=torch.float32)
 
 

@@ -67,8 +67,17 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
     else:
         pertoken_scale = dynamic_scale
 
-    if dynamic_eplb or isinstance(w2, (list, tuple)) and len(w2) != 1:
-        raise NotImplementedError("per-expert weight lists (dynamic EPLB) are not built yet")
+    if dynamic_eplb or (isinstance(w1, (list, tuple)) and len(w1) > 1):
+        # per-expert weight lists (the form dynamic expert load balancing swaps in place)
+        hidden_states, swiglu_out_scale, _ = torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz_tensor_list(
+            x=hidden_states, weight=list(w1), weight_scale=list(w1_scale), x_scale=pertoken_scale,
+            group_list=cumsum_group_list(group_list, group_list_type, 0), bias=None, swiglu_limit=swiglu_limit)
+        before_gmm2_evt = torch.cuda.current_stream().record_event() if hidden_states.is_cuda else None
+        out = DeviceOperator.npu_grouped_matmul_gmm2(
+            hidden_states=hidden_states, weight=list(w2), weight_scale=list(w2_scale),
+            per_token_scale=swiglu_out_scale, group_list=group_list, group_list_type=group_list_type,
+            input_dtype=input_dtype if input_dtype != torch.int8 else torch.bfloat16)
+        return out, before_gmm2_evt
     # gmm1: gate_up_proj + dequant + SwiGLU + dynamic re-quant in one op
     hidden_states, swiglu_out_scale, _ = DeviceOperator.npu_grouped_matmul_swiglu_quant(
         x=hidden_states, weight=_single(w1, "w1"),

@@ -251,3 +251,60 @@ def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_lis
                                      _ptr(_gl(group_list)), _gl_type(group_list_type), rows, k, n, E, _ptr(out),
                                      DT_BF16, _stream(x)), "moe355_gmm2_dequant_w4")
     return out
+
+
+# ------------------------------------------------------------------ per-expert tensor lists
+_PTR_TABLES: dict = {}
+
+
+def _ptr_table(tensors) -> torch.Tensor:
+    """Device array with the data pointers of ``tensors`` (cached per exact list of pointers)."""
+    key = tuple(t.data_ptr() for t in tensors)
+    tab = _PTR_TABLES.get(key)
+    if tab is None:
+        if len(_PTR_TABLES) > 64:
+            _PTR_TABLES.clear()
+        tab = torch.tensor(key, dtype=torch.int64, device=tensors[0].device)
+        _PTR_TABLES[key] = tab
+    return tab
+
+
+def _check_list(tensors, name, dtype):
+    for t in tensors:
+        if not t.is_cuda or not t.is_contiguous() or t.dtype != dtype or t.shape != tensors[0].shape:
+            raise RuntimeError(f"{name}: every per-expert tensor must be a contiguous {dtype} GPU tensor of one shape")
+
+
+def gmm1_swiglu_quant_list(x, weight_list, scale_list, x_scale, group_list, group_list_type, swiglu_limit=0.0):
+    """weight_list: E tiled int8 tensors of logical shape [K, N]; scale_list: E fp32 tensors [N]."""
+    x = _dev(x, "x")
+    lib = _lib.load()
+    _check_list(weight_list, "weight", torch.int8)
+    _check_list(scale_list, "weight_scale", torch.float32)
+    k, n = weight_list[0].shape
+    rows, E, dev = x.shape[0], len(weight_list), x.device
+    out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
+    out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.moe355_gmm1_swiglu_quant_workspace(rows, n, k, E), dev)
+    check(lib.moe355_gmm1_swiglu_quant_list(_ptr(x), _ptr(_ptr_table(weight_list)), _ptr(_ptr_table(scale_list)),
+                                            _ptr(_dev(x_scale, "x_scale")), _ptr(_gl(group_list)),
+                                            _gl_type(group_list_type), rows, k, n, E, float(swiglu_limit), _ptr(out),
+                                            _ptr(out_scale), _ptr(ws), ws.numel(), _stream(x)),
+          "moe355_gmm1_swiglu_quant_list")
+    return out, out_scale
+
+
+def gmm2_dequant_list(x, weight_list, scale_list, per_token_scale, group_list, group_list_type):
+    x = _dev(x, "x")
+    lib = _lib.load()
+    _check_list(weight_list, "weight", torch.int8)
+    _check_list(scale_list, "scale", torch.float32)
+    k, n = weight_list[0].shape
+    rows, E = x.shape[0], len(weight_list)
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
+    ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
+    check(lib.moe355_gmm2_dequant_list(_ptr(x), _ptr(_ptr_table(weight_list)), _ptr(_ptr_table(scale_list)),
+                                       _ptr(_dev(per_token_scale, "per_token_scale")), _ptr(_gl(group_list)),
+                                       _gl_type(group_list_type), rows, k, n, E, _ptr(out), DT_BF16, _ptr(ws),
+                                       ws.numel(), _stream(x)), "moe355_gmm2_dequant_list")
+    return out

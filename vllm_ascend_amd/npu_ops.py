@@ -76,6 +76,12 @@ def npu_grouped_matmul(x, weight, *, bias=None, scale=None, offset=None, antiqua
     ws = weight if isinstance(weight, (list, tuple)) else [weight]
     ss = scale if isinstance(scale, (list, tuple)) else [scale]
     ps = per_token_scale if isinstance(per_token_scale, (list, tuple)) else [per_token_scale]
+    if len(xs) == 1 and len(ps) == 1 and len(ws) > 1 and len(ws) == len(ss):
+        # one tiled [K, N] weight and one [N] scale per expert
+        if output_dtype not in (None, torch.bfloat16):
+            raise NotImplementedError(f"npu_grouped_matmul: output_dtype {output_dtype} is not supported")
+        scales = [s_ if s_.dtype == torch.float32 else s_.to(torch.float32) for s_ in ss]
+        return [kernels.gmm2_dequant_list(xs[0], list(ws), scales, ps[0], group_list, group_list_type)]
     if len(xs) != 1 or len(ws) != 1 or len(ss) != 1 or len(ps) != 1 or ss[0] is None or ps[0] is None:
         raise NotImplementedError("npu_grouped_matmul: expects exactly one x, weight, scale and per_token_scale")
     a, w, s, p = xs[0], ws[0], ss[0], ps[0]

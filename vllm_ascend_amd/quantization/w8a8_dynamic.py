@@ -24,11 +24,10 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
     def __init__(self, in_dtype: torch.dtype = torch.bfloat16, dynamic_eplb: bool = False):
         # The reference reads these from the vLLM / Ascend configs (w8a8_dynamic.py:173-196);
         # there is no vLLM here, so they are constructor arguments with the 1-GPU defaults.
-        if dynamic_eplb:
-            raise NotImplementedError("dynamic EPLB (per-expert weight lists) is not built yet")
         self.in_dtype = in_dtype
-        self.dynamic_eplb = False
-        self.use_expert_weight_list = False
+        self.dynamic_eplb = dynamic_eplb
+        # per-expert tensors that can be swapped one by one (w8a8_dynamic.py:180-183, 365-389)
+        self.use_expert_weight_list = dynamic_eplb
         self.use_aclgraph = False
         self.moe_all_to_all_group_name = ""  # no MC2 group on one device
 
@@ -63,6 +62,13 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 p.data = p.data.view(p.data.shape[0], -1)
         layer.w13_weight_scale_fp32 = layer.w13_weight_scale.data.to(torch.float32)
         layer.w2_weight_scale_fp32 = layer.w2_weight_scale.data.to(torch.float32)
+        if self.use_expert_weight_list:
+            layer.w13_weight_list = [w.clone() for w in layer.w13_weight.data.unbind(dim=0)]
+            layer.w2_weight_list = [w.clone() for w in layer.w2_weight.data.unbind(dim=0)]
+            layer.w13_weight_scale_fp32_list = [s.clone() for s in layer.w13_weight_scale_fp32.unbind(dim=0)]
+            layer.w2_weight_scale_list = [s.clone() for s in layer.w2_weight_scale_fp32.unbind(dim=0)]
+            del layer.w13_weight, layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale
+            del layer.w13_weight_scale_fp32, layer.w2_weight_scale_fp32
 
     def apply(self, layer, x: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
               shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
@@ -81,8 +87,8 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 hidden_states=x,
                 topk_weights=topk_weights,
                 topk_ids=topk_ids,
-                w1=[layer.w13_weight],
-                w2=[layer.w2_weight],
+                w1=layer.w13_weight_list if self.use_expert_weight_list else [layer.w13_weight],
+                w2=layer.w2_weight_list if self.use_expert_weight_list else [layer.w2_weight],
                 quant_type=self.quant_type,
                 dynamic_eplb=self.use_expert_weight_list,
                 expert_map=getattr(layer, "ascend_expert_map", None),
@@ -93,10 +99,14 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 activation=getattr(layer, "activation", "silu"),
                 shared_out=shared_out,
                 shared_experts=shared_experts,
-                w1_scale=[layer.w13_weight_scale_fp32],
-                w2_scale=[layer.w2_weight_scale_fp32],
+                w1_scale=(layer.w13_weight_scale_fp32_list if self.use_expert_weight_list
+                          else [layer.w13_weight_scale_fp32]),
+                w2_scale=layer.w2_weight_scale_list if self.use_expert_weight_list else [layer.w2_weight_scale_fp32],
             ))
 
     @staticmethod
     def get_eplb_weight_views(layer) -> list:
+        if hasattr(layer, "w13_weight_list"):
+            return [layer.w13_weight_list, layer.w2_weight_list, layer.w13_weight_scale_fp32_list,
+                    layer.w2_weight_scale_list]
         return [layer.w13_weight, layer.w2_weight, layer.w13_weight_scale_fp32, layer.w2_weight_scale_fp32]
