@@ -173,6 +173,13 @@ int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, cons
                                 int num_experts, float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
                                 size_t workspace_bytes, void *stream);
 
+/* corr[e, col] = 8 * sum_g float(sum_{k in g} w[e, col, k]) * weight_scale[e, g, col]  (fp32 [E, N]).
+ * The reference's int4 op computes (x - 8) . W and expects the caller to pass this term back in as
+ * `bias` / `weight_assist_matrix` (vllm_ascend/quantization/methods/w4a8.py:385-394); a caller of
+ * moe355_gmm1_swiglu_quant_w4, which computes x . W, passes `bias - corr` instead. */
+int moe355_w4_offset_correction(const uint8_t *weight_nz4, const float *weight_scale, int64_t group_size,
+                                int num_experts, int64_t n, int64_t k, float *corr, void *stream);
+
 /* ---------------------------------------------------------------------------
  * down grouped GEMM (int8 x int8 -> int32) + dequant to bf16.
  * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,

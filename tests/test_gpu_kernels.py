@@ -233,3 +233,49 @@ def test_dequant_swiglu_quant(K, orc, rows, n, left):
     yo, so = orc.dequant_swiglu_quant(x.numpy(), ws.numpy(), a.numpy(), left, 0.0)
     assert np.array_equal(y.cpu().numpy(), yo)
     assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+def test_grouped_matmul_swiglu_quant_v2_against_the_reference_golden(orc):
+    """A8W4 operator with per-group scales and an arbitrary assist matrix, against a numpy rendering of
+    gmm_swiglu_quant_golden_a8_w4 (tests/e2e/nightly/single_node/ops/singlecard_ops/
+    test_grouped_matmul_swiglu_quant.py:58-109) in fp32: out = ((x - 8) . W . scale + bias) * per_token,
+    SwiGLU, dynamic int8.  Tolerance of the reference test: int8 +-1, scale rtol 5e-3."""
+    from vllm_ascend_amd import npu_ops
+    from vllm_ascend_amd.custom_ops import enable_custom_op
+
+    enable_custom_op()
+    g = torch.Generator().manual_seed(0)
+    E, M, Kd, N, grp = 4, 96, 512, 256, 256
+    x = torch.randint(-5, 5, (M, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-5, 5, (E, Kd, N), generator=g, dtype=torch.int8)  # [E, K, N] int4 values
+    scale = torch.randn(E, Kd // grp, N, generator=g)
+    per_token = torch.randn(M, generator=g)
+    bias = torch.rand(E, N, generator=g) * 10 - 5
+    cum = torch.tensor([20, 20, 70, 90], dtype=torch.int64)  # rows 90..95 belong to no expert
+    pairs = w.reshape(E, Kd, N // 2, 2)
+    packed = ((pairs[..., 1] << 4) | (pairs[..., 0] & 0x0F)).to(torch.int8).contiguous().view(torch.int32)
+    w_nz = npu_ops.npu_format_cast_int4(packed.to(DEV))
+    scale_i64 = torch.from_numpy(scale.numpy().view(np.uint32).astype(np.int64))
+    out, out_scale = torch.ops._C_ascend.grouped_matmul_swiglu_quant_v2(
+        x=x.to(DEV), weight=[w_nz], weight_scale=[scale_i64.to(DEV)], x_scale=per_token.to(DEV),
+        group_list=cum.to(DEV), weight_assist_matrix=[bias.to(DEV)], dequant_mode=0, group_list_type=0)
+    # the older entry point of the same kernel takes the assist matrix as `bias`
+    out_b, scale_b, _ = torch.ops._C_ascend.grouped_matmul_swiglu_quant(
+        x=x.to(DEV), weight=w_nz, bias=bias.to(DEV), group_list=cum.to(DEV), weight_scale=scale_i64.to(DEV),
+        x_scale=per_token.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(out_b[:90], out[:90]) and torch.equal(scale_b[:90], out_scale[:90])
+    lo = 0
+    for e, hi in enumerate(cum.tolist()):
+        if hi > lo:
+            xe = (x[lo:hi].to(torch.float64) - 8).reshape(hi - lo, Kd // grp, grp)
+            we = w[e].to(torch.float64).reshape(Kd // grp, grp, N)
+            mm = torch.einsum("mgk,gkn->gmn", xe, we) * scale[e].to(torch.float64)[:, None, :]
+            f = (mm.sum(0) + bias[e].to(torch.float64)) * per_token[lo:hi, None].to(torch.float64)
+            a, gate = f.chunk(2, dim=-1)
+            y = a * torch.sigmoid(a) * gate
+            mx = y.abs().max(dim=-1).values
+            q_ref = torch.round(y * (127 / mx)[:, None]).to(torch.int8)
+            assert (out[lo:hi].cpu().to(torch.int32) - q_ref.to(torch.int32)).abs().max() <= 1
+            torch.testing.assert_close(out_scale[lo:hi].cpu().double(), mx / 127, rtol=5e-3, atol=1e-6)
+        lo = hi

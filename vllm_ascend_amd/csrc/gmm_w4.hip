@@ -50,6 +50,39 @@ __global__ __launch_bounds__(256) void format_cast_nz_int4_kernel(const uint8_t*
     }
 }
 
+// corr[e, n] = 8 * sum_g float(sum_{k in g} w[e, n, k]) * scale[e, g, n]  (g ascending, fp32):
+// the term the Ascend kernel's unsigned-nibble trick adds (x = (x - 8) + 8), which callers of the
+// int4 op pass in as `bias` / `weight_assist_matrix`.  One wavefront per (expert, 32-channel tile).
+__global__ __launch_bounds__(256) void w4_offset_correction_kernel(const uint8_t* __restrict__ w4,
+                                                                   const float* __restrict__ gscale, int E, int N,
+                                                                   int K, int group, float* __restrict__ corr)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t tile_row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int NB = N >> 5, KB64 = K >> 6;
+    if (tile_row >= (int64_t)E * NB) return;
+    const int e = (int)(tile_row / NB), nb = (int)(tile_row % NB);
+    const uint8_t* wp = w4 + (tile_row * KB64) * 1024 + lane * 16;
+    const int steps_per_group = group >> 6;
+    const int n_groups = K / group;
+    const int ch = nb * 32 + (lane & 31);
+    float total = 0.0f;
+    for (int g = 0; g < n_groups; ++g) {
+        int sum = 0;
+        for (int t = 0; t < steps_per_group; ++t) {
+            const v4i v = *(const v4i*)(wp + (int64_t)(g * steps_per_group + t) * 1024);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                for (int b = 0; b < 8; ++b) sum += ((int)((unsigned)v[d] << (28 - 4 * b))) >> 28;  // signed nibble b
+            }
+        }
+        sum += __shfl_xor(sum, 32, 64);  // the two K halves of the tile
+        total = total + (float)sum * gscale[((int64_t)e * n_groups + g) * N + ch];
+    }
+    if (lane < 32) corr[(int64_t)e * N + ch] = 8.0f * total;
+}
+
 struct W4Args {
     GmmArgs g;            // x, gl, R, K, N, E, row_scale, limit, outputs; g.w unused
     const uint8_t* w4;    // tiled int4 storage
@@ -256,6 +289,20 @@ extern "C" int moe355_format_cast_nz_int4(const uint8_t* w, int source, int64_t 
     else
         hipLaunchKernelGGL(format_cast_nz_int4_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, w, num_experts, n, k,
                            out);
+    return launch_status();
+}
+
+extern "C" int moe355_w4_offset_correction(const uint8_t* weight_nz4, const float* weight_scale, int64_t group_size,
+                                           int num_experts, int64_t n, int64_t k, float* corr, void* stream)
+{
+    if (num_experts <= 0 || n <= 0 || k <= 0 || group_size <= 0 || !weight_nz4 || !weight_scale || !corr)
+        return MOE355_E_ARG;
+    if (n % 32 != 0 || k % 64 != 0 || group_size % 64 != 0 || k % group_size != 0) return MOE355_E_SHAPE;
+    if ((uintptr_t)weight_nz4 & 15) return MOE355_E_SHAPE;
+    const int64_t tiles = (int64_t)num_experts * (n / 32);
+    hipLaunchKernelGGL(w4_offset_correction_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)stream, weight_nz4, weight_scale, num_experts, (int)n, (int)k, (int)group_size,
+                       corr);
     return launch_status();
 }
 

@@ -83,10 +83,18 @@ def _reject_unsupported(bias, offset):
 
 
 def _gmm_swiglu_quant_nz(x, weight, weight_scale, x_scale, group_list, *, bias=None, offset=None, swiglu_limit=0.0):
+    if weight.dtype == torch.int32:
+        # A8W4 form of the same op (eight int4 values per int32; is_a8w4 in
+        # csrc/gmm/grouped_matmul_swiglu_quant_weight_nz_tensor_list/grouped_matmul_swiglu_quant_torch_adpt.h:27-31):
+        # `bias` is the assist matrix of the int4 kernel
+        if offset is not None and offset.numel() > 0:
+            raise NotImplementedError("grouped_matmul_swiglu_quant: `offset` is not supported")
+        out, out_scale = _gmm_swiglu_quant_v2(x, [weight], [weight_scale], x_scale, group_list,
+                                              weight_assist_matrix=None if bias is None else [bias],
+                                              group_list_type=0, swiglu_limit=swiglu_limit)
+        return out, out_scale, x.new_empty((), dtype=torch.float32)
     if weight.dtype != torch.int8:
-        raise NotImplementedError(
-            f"grouped_matmul_swiglu_quant: weight dtype {weight.dtype}; int4 weights go through "
-            "grouped_matmul_swiglu_quant_v2")
+        raise NotImplementedError(f"grouped_matmul_swiglu_quant: weight dtype {weight.dtype} is not supported")
     _reject_unsupported(bias, offset)
     if x.dtype != torch.int8 or x.dim() != 2 or weight.dim() != 3:
         raise RuntimeError("grouped_matmul_swiglu_quant expects x int8 [M, K] and weight int8 [E, K, N]")
@@ -130,10 +138,50 @@ def _gmm_swiglu_quant_nz_tensor_list_meta(x, weight, weight_scale, x_scale, grou
             x.new_empty((m,), dtype=torch.float32))
 
 
+_W4_CORR: dict = {}
+
+
+def _decode_scale(scale: torch.Tensor) -> torch.Tensor:
+    """The reference widens fp32 scale bits into int64 (w4a8.py:320-325); undo that."""
+    if scale.dtype == torch.int64:
+        return scale.to(torch.int32).view(torch.float32)
+    return scale.to(torch.float32)
+
+
 def _gmm_swiglu_quant_v2(x, weight, weight_scale, x_scale, group_list, smooth_scale=None, weight_assist_matrix=None,
                          bias=None, dequant_mode=0, dequant_dtype=0, quant_mode=0, quant_dtype=0,
                          transpose_weight=False, group_list_type=0, tuning_config=(), swiglu_limit=0.0):
-    raise NotImplementedError("grouped_matmul_swiglu_quant_v2 (int4 weights) is not built yet")
+    """A8W4 form: ``x`` int8 [M, K]; ``weight`` = [tiled int4 storage from ``npu_format_cast_int4``, logical
+    [E, K, N]]; ``weight_scale`` = [[E, N] per channel or [E, K/g, N] per group, fp32 or int64-encoded fp32];
+    ``weight_assist_matrix`` = [[E, N] fp32]: the reference kernel computes (x - 8) . W . scale and adds this
+    matrix, so the result here is x . W . scale + (assist - 8 * sum_k W * scale)."""
+    if smooth_scale is not None or bias is not None or transpose_weight:
+        raise NotImplementedError("grouped_matmul_swiglu_quant_v2: smooth_scale / bias / transpose_weight")
+    if (dequant_mode or 0) != 0 or (quant_mode or 0) != 0 or (quant_dtype or 0) != 0:
+        raise NotImplementedError("grouped_matmul_swiglu_quant_v2: only dequant_mode=0, quant_mode=0 (int8 out)")
+    if len(weight) != 1 or len(weight_scale) != 1 or x.dtype != torch.int8:
+        raise NotImplementedError("grouped_matmul_swiglu_quant_v2: one stacked int4 weight and one scale tensor")
+    w, s = weight[0], _decode_scale(weight_scale[0])
+    k = x.shape[1]
+    n = s.shape[-1]
+    e = w.shape[0]
+    s = s.reshape(e, -1, n).contiguous()
+    group = k // s.shape[1]
+    w_bytes = w.contiguous().view(torch.uint8).reshape(e, -1)
+    if w_bytes.shape[1] * 2 != n * k:
+        raise RuntimeError("grouped_matmul_swiglu_quant_v2: weight holds a different number of int4 values than K*N")
+    eff_bias = None
+    if weight_assist_matrix is not None:
+        key = (w.data_ptr(), s.data_ptr(), group)
+        corr = _W4_CORR.get(key)
+        if corr is None:
+            if len(_W4_CORR) > 16:
+                _W4_CORR.clear()
+            corr = kernels.w4_offset_correction(w_bytes, s, group, n, k)
+            _W4_CORR[key] = corr
+        eff_bias = (weight_assist_matrix[0].to(torch.float32).reshape(e, n) - corr).contiguous()
+    return kernels.gmm1_swiglu_quant_w4(x, w_bytes, s, group, x_scale, group_list, group_list_type, n, k,
+                                        bias=eff_bias, swiglu_limit=swiglu_limit)
 
 
 def _gmm_swiglu_quant_v2_meta(x, weight, weight_scale, x_scale, group_list, smooth_scale=None,

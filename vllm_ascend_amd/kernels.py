@@ -308,3 +308,14 @@ def gmm2_dequant_list(x, weight_list, scale_list, per_token_scale, group_list, g
                                        _gl_type(group_list_type), rows, k, n, E, _ptr(out), DT_BF16, _ptr(ws),
                                        ws.numel(), _stream(x)), "moe355_gmm2_dequant_list")
     return out
+
+
+def w4_offset_correction(weight_nz4, weight_scale, group_size, n, k):
+    """fp32 [E, N]: 8 * sum_k w * scale, the correction term of the reference's int4 op."""
+    lib = _lib.load()
+    w = _dev(weight_nz4, "weight")
+    E = w.shape[0]
+    corr = torch.empty((E, n), dtype=torch.float32, device=w.device)
+    check(lib.moe355_w4_offset_correction(_ptr(w), _ptr(_dev(weight_scale, "weight_scale")), group_size, E, n, k,
+                                          _ptr(corr), _stream(w)), "moe355_w4_offset_correction")
+    return corr

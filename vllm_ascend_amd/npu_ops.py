@@ -139,3 +139,16 @@ def npu_quant_matmul(x1, x2, scale, *, offset=None, pertoken_scale=None, bias=No
     else:
         raise NotImplementedError(f"npu_quant_matmul: output_dtype {output_dtype} is not supported")
     return out.reshape(lead + (n,))
+
+
+def npu_format_cast_int4(packed: torch.Tensor) -> torch.Tensor:
+    """int4 weights packed two per byte along N (low nibble = even channel), logical ``[E, K, N]`` held as
+    int8 ``[E, K, N/2]`` or its int32 view ``[E, K, N/8]`` (``vllm_ascend/quantization/methods/w4a8.py:313-336``)
+    -> same shape and dtype, tiled int4 storage for the W4A8 grouped-matmul operators."""
+    if packed.dim() != 3 or packed.dtype not in (torch.int8, torch.uint8, torch.int32):
+        raise TypeError("npu_format_cast_int4 expects a packed 3-D int8 / int32 weight")
+    per = 8 if packed.dtype == torch.int32 else 2
+    e, k, n = packed.shape[0], packed.shape[1], packed.shape[2] * per
+    raw = packed.contiguous().view(torch.uint8).reshape(e, k, n // 2)
+    tiled = kernels.format_cast_nz_int4(raw, 1, n, k)
+    return tiled.view(packed.dtype).reshape(packed.shape)
