@@ -262,7 +262,13 @@ static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
         return launch_status();
     }
     const int64_t units = (int64_t)a.E * (a.N / 64);
-    launch_gemm(gmm_stream_kernel<EPI, 4, 4, 4>, dim3((unsigned)units), st, a);
+    // Occupancy 3 keeps the SwiGLU epilogue out of scratch memory (131 registers).  With enough units to
+    // fill the chip four times over, the down GEMM lets every wavefront stream a whole unit by itself (no
+    // K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K.
+    if (EPI != EPI_SWIGLU && units >= 2048)
+        launch_gemm(gmm_stream_kernel<EPI, 1, 4, 2>, dim3((unsigned)((units + 3) / 4)), st, a);
+    else
+        launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units), st, a);
     return launch_status();
 }
 
