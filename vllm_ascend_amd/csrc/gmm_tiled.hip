@@ -75,37 +75,34 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
 constexpr int kBN = 256;  // channels per workgroup (4 wavefronts x 2 storage tiles)
 constexpr int kBK = 64;   // K per pipeline stage (2 MFMA K steps)
 
-template <int EPI, int BMT>  // BMT = token blocks of 32 per workgroup tile (BM = 32 * BMT)
-__global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+// LDS of one workgroup: RING token stages of the tallest tile, reused by the epilogue patches
+template <int EPI, int BMT, int RING>
+struct TiledLds {
+    static constexpr int BM = 32 * BMT;
+    static constexpr int STAGE_BYTES = BM * kBK;               // tokens of one stage in LDS
+    static constexpr int ROWB = 128 + 16;                      // epilogue patch: bytes per token row (padded)
+    static constexpr int PATCHES = (EPI == EPI_I32) ? 2 : 1;   // 32-row patches per wavefront in the epilogue
+    static constexpr int EPI_BYTES = 4 * PATCHES * 32 * ROWB;
+    static constexpr int BYTES = RING * STAGE_BYTES > EPI_BYTES ? RING * STAGE_BYTES : EPI_BYTES;
+};
+
+// One tile of BMT token blocks: rows [row0, row_end) of expert e (at most 32 * BMT of them are computed),
+// column block nt.
+// RING = depth of the operand ring in registers: weights are requested RING - 1 K blocks ahead, tokens RING.
+template <int EPI, int BMT, int RING>  // BMT = token blocks of 32 per tile (BM = 32 * BMT)
+__device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
+                                           int8_t* lds_raw)
 {
-    constexpr int BM = 32 * BMT;
-    constexpr int STAGE_BYTES = BM * kBK;                 // tokens of one stage in LDS
+    constexpr int STAGE_BYTES = TiledLds<EPI, BMT, RING>::STAGE_BYTES;
     constexpr int CHUNKS = STAGE_BYTES / 16 / 256;        // 16-byte chunks per thread per stage
-    constexpr int ROWB = 128 + 16;                        // epilogue patch: bytes per token row (padded)
-    constexpr int PATCHES = (EPI == EPI_I32) ? 2 : 1;     // 32-row patches per wavefront in the epilogue
-    constexpr int EPI_BYTES = 4 * PATCHES * 32 * ROWB;
-    constexpr int LDS_BYTES = 3 * STAGE_BYTES > EPI_BYTES ? 3 * STAGE_BYTES : EPI_BYTES;
-    __shared__ __attribute__((aligned(16))) int8_t lds_raw[LDS_BYTES];
+    constexpr int ROWB = TiledLds<EPI, BMT, RING>::ROWB;
+    constexpr int PATCHES = TiledLds<EPI, BMT, RING>::PATCHES;
+    static_assert(CHUNKS >= 1, "a stage is at least one 16-byte chunk per thread");
     int8_t (*Bs)[STAGE_BYTES] = reinterpret_cast<int8_t (*)[STAGE_BYTES]>(lds_raw);
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-
-    // ---- which tile: XCD-aware remap of the 1-D grid over the tiles that exist (workgroup i runs on
-    // XCD i % 8; each XCD gets one contiguous eighth of the tile list, in order)
-    const int total = tm.count[0] * n_col_blocks;
-    const int per_xcd = (total + 7) / 8;
-    const int slot = (int)(blockIdx.x / 8);
-    const int item = (int)(blockIdx.x % 8) * per_xcd + slot;
-    if (slot >= per_xcd || item >= total) return;
-    const int mt = item / n_col_blocks;
-    const int nt = item % n_col_blocks;
-    const int e = tm.expert[mt];
-    const int64_t row0 = tm.row_begin[mt];
-    int64_t row_end = tm.row_end[mt];
-    if (row_end > a.R) row_end = a.R;
-    if (row0 >= row_end) return;
 
     const int NB = a.N >> 5, KB = a.K >> 5;
     const int half_tiles = NB >> 1;
@@ -125,8 +122,8 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
 
     const int n_iter = a.K / kBK;
 
-    v4i Areg[3][2][2];   // [stage][tile][k step]
-    v4i Breg[3][CHUNKS];
+    v4i Areg[RING][2][2];   // [stage][tile][k step]
+    v4i Breg[RING][CHUNKS];
 
     // Loads past the last K block or the last row are redirected to valid addresses instead of being
     // skipped (their results are never used): the loop body stays free of branches, so the compiler can
@@ -186,40 +183,45 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
         }
     };
 
-    // ---- prologue.  After it the loads still in flight are, oldest first, A(0) B(1) A(1) B(2): the same
+    // ---- prologue.  After it the loads still in flight are, oldest first, A(0) B(1) A(1) B(2) ...: the same
     // order every iteration leaves behind, so the wait counts the compiler derives at the loop head are exact.
     load_B(0, 0);
     store_B(0);
     __syncthreads();
-    load_A(0, 0);
-    load_B(1, 1);
-    load_A(1, 1);
-    load_B(2, 2);
+#pragma unroll
+    for (int r = 0; r + 1 < RING; ++r) {
+        load_A(r, r);
+        load_B(r + 1, r + 1);
+    }
     read_frags(bf0, 0, 0);
 
     // One pipeline step on stage U (compile-time ring position) for K block I.
 #define MOE355_STEP(U, I)                                                          \
     {                                                                              \
-        store_B(((U) + 1) % 3);             /* B(I+1): registers -> LDS */         \
+        store_B(((U) + 1) % RING);          /* B(I+1): registers -> LDS */         \
         read_frags(bf1, (U), 1);            /* second K step of this stage */      \
         __builtin_amdgcn_sched_barrier(0);                                         \
         mma_step(bf0, (U), 0);                                                     \
         __syncthreads();                    /* B(I+1) visible to all wavefronts */ \
-        load_A((I) + 2, ((U) + 2) % 3);                                            \
-        load_B((I) + 3, (U));                                                      \
-        read_frags(bf0, ((U) + 1) % 3, 0);  /* first K step of the next stage */   \
+        load_A((I) + RING - 1, ((U) + RING - 1) % RING);                           \
+        load_B((I) + RING, (U));                                                   \
+        read_frags(bf0, ((U) + 1) % RING, 0);  /* first K step of the next stage */ \
         __builtin_amdgcn_sched_barrier(0);                                         \
         mma_step(bf1, (U), 1);                                                     \
     }
-    // whole triples run without any condition inside (exact wait counts); the remainder is peeled
-    const int n_full = (n_iter / 3) * 3;
-    for (int i0 = 0; i0 < n_full; i0 += 3) {
+    // whole passes through the ring run without any condition inside (exact wait counts); the remainder is peeled
+    const int n_full = (n_iter / RING) * RING;
+    for (int i0 = 0; i0 < n_full; i0 += RING) {
         MOE355_STEP(0, i0)
         MOE355_STEP(1, i0 + 1)
         MOE355_STEP(2, i0 + 2)
+        if constexpr (RING > 3) MOE355_STEP(3, i0 + 3)
     }
     if (n_iter - n_full >= 1) MOE355_STEP(0, n_full)
     if (n_iter - n_full >= 2) MOE355_STEP(1, n_full + 1)
+    if constexpr (RING > 3) {
+        if (n_iter - n_full >= 3) MOE355_STEP(2, n_full + 2)
+    }
 #undef MOE355_STEP
 
     // ---- epilogue.  In the accumulators a lane owns one token and scattered runs of four channels;
@@ -301,7 +303,41 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
     }
 }
 
-
+// The last tile of an expert is usually short.  Tiles of at most 64 rows run the two-block body (half the
+// MFMAs and half the token traffic of a full tile) inside the same launch, next to the full tiles of their
+// expert, so that they still find the expert's weights in the L2 of their XCD.
+template <int EPI, int BMT, int RING>
+__global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+{
+    __shared__ __attribute__((aligned(16))) int8_t lds_raw[TiledLds<EPI, BMT, RING>::BYTES];
+    // ---- which tile: XCD-aware remap of the 1-D grid over the tiles that exist (workgroup i runs on
+    // XCD i % 8; each XCD gets one contiguous eighth of the tile list, in order)
+    const int total = tm.count[0] * n_col_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int slot = (int)(blockIdx.x / 8);
+    const int item = (int)(blockIdx.x % 8) * per_xcd + slot;
+    if (slot >= per_xcd || item >= total) return;
+    const int mt = item / n_col_blocks;
+    const int nt = item % n_col_blocks;
+    const int e = tm.expert[mt];
+    const int64_t row0 = tm.row_begin[mt];
+    int64_t row_end = tm.row_end[mt];
+    if (row_end > a.R) row_end = a.R;
+    if (row0 >= row_end) return;
+    if constexpr (BMT > 2) {
+        if (row_end - row0 <= 64) {
+            tiled_body<EPI, 2, RING>(a, e, row0, row_end, nt, lds_raw);
+            return;
+        }
+    }
+    if constexpr (BMT > 4) {
+        if (row_end - row0 <= 128) {
+            tiled_body<EPI, 4, RING>(a, e, row0, row_end, nt, lds_raw);
+            return;
+        }
+    }
+    tiled_body<EPI, BMT, RING>(a, e, row0, row_end, nt, lds_raw);
+}
 
 // ------------------------------------------------------------------ host side
 size_t tiled_workspace_bytes(int64_t rows, int E, int BM)
@@ -310,7 +346,7 @@ size_t tiled_workspace_bytes(int64_t rows, int E, int BM)
     return 256 + (size_t)(((max_tiles * 4 + 255) / 256) * 256) * 3;
 }
 
-template <int EPI, int BMT>
+template <int EPI, int BMT, int RING>
 static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
 {
     constexpr int BM = 32 * BMT;
@@ -328,17 +364,17 @@ static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipE
     const int total = max_tiles * n_col_blocks;
     const int grid = ((total + 7) / 8) * 8;
     if (ev0 && ev1)
-        hipExtLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT>), dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm,
+        hipExtLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT, RING>), dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm,
                               max_tiles, n_col_blocks);
     else
-        hipLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT>), dim3(grid), dim3(256), 0, st, a, tm, max_tiles,
+        hipLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT, RING>), dim3(grid), dim3(256), 0, st, a, tm, max_tiles,
                            n_col_blocks);
 }
 
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
                       hipEvent_t ev1)
 {
-#define MOE355_TILED(E_, B_) launch_tiled<E_, B_>(a, workspace, st, ev0, ev1)
+#define MOE355_TILED(E_, B_) launch_tiled<E_, B_, ((B_) > 4 ? 4 : 3)>(a, workspace, st, ev0, ev1)
     if (bm == 256) {
         if (epi == EPI_I32) MOE355_TILED(EPI_I32, 8);
         else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 8);
