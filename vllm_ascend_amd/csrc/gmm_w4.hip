@@ -137,44 +137,95 @@ __device__ __forceinline__ void epilogue_run_w4(const GmmArgs& a, int64_t row, b
     }
 }
 
-// One wavefront per unit (expert, pair of 32-channel tiles), whole K range.
-template <int EPI, int UN>
-__global__ __launch_bounds__(256, 3) void gmm_w4_stream_kernel(W4Args p)
+// Chunk c of the list "rows of expert 0 in pieces of CHUNK rows, then expert 1, ...": which expert, which
+// rows.  Every lane returns the same answer; false past the last chunk.  Lane l owns experts
+// [l*seg, (l+1)*seg): local counts, a wavefront scan, then a short walk inside the owning lane's segment.
+__device__ __forceinline__ bool find_chunk(const int64_t* gl, int gl_type, int E, int c, int CHUNK, int lane, int& e,
+                                           int64_t& row0, int64_t& row1)
 {
+    auto rows_of = [&](int i) -> int {
+        const int64_t m = (gl_type == MOE355_GL_COUNT) ? gl[i] : gl[i] - (i > 0 ? gl[i - 1] : 0);
+        return m < 0 ? 0 : (int)m;
+    };
+    const int seg = (E + 63) >> 6;
+    const int e0 = lane * seg;
+    int rows = 0, chunks = 0;
+    for (int j = 0; j < seg; ++j) {
+        if (e0 + j < E) {
+            const int m = rows_of(e0 + j);
+            rows += m;
+            chunks += (m + CHUNK - 1) / CHUNK;
+        }
+    }
+    int inc_rows = rows, inc_chunks = chunks;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int r = __shfl_up(inc_rows, off, 64), k = __shfl_up(inc_chunks, off, 64);
+        if (lane >= off) {
+            inc_rows += r;
+            inc_chunks += k;
+        }
+    }
+    if (c >= __shfl(inc_chunks, 63, 64)) return false;
+    const uint64_t owns = __ballot(c < inc_chunks);  // lanes at or after the owner
+    const int owner = __builtin_ctzll(owns);
+    int cc = __shfl(inc_chunks - chunks, owner, 64);
+    int64_t rr = __shfl(inc_rows - rows, owner, 64);
+    const int oe0 = owner * seg;
+    for (int j = 0; j < seg; ++j) {
+        const int i = oe0 + j;
+        if (i >= E) break;
+        const int m = rows_of(i);
+        const int nc = (m + CHUNK - 1) / CHUNK;
+        if (c - cc < nc) {
+            e = i;
+            row0 = rr + (int64_t)(c - cc) * CHUNK;
+            row1 = rr + m;
+            return true;
+        }
+        cc += nc;
+        rr += m;
+    }
+    return false;
+}
+
+// One wavefront per unit (chunk of up to 64 rows of one expert, pair of 32-channel tiles), whole K range in
+// ascending order (the fp32 sum over scale groups has one fixed order).  An expert with many rows becomes
+// many units that run side by side on different CUs and find the expert's weights in L2 / Infinity Cache,
+// instead of one wavefront streaming the same weights once per 32 rows.
+constexpr int kW4Chunk = 64;
+template <int EPI>
+__global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
+{
+    constexpr int UN = 2;  // 64-wide K blocks per batch of loads
     const GmmArgs& a = p.g;
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int NB = a.N >> 5, KB64 = a.K >> 6;
     const int upe = NB >> 1;
     const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
-    if (unit >= (int64_t)a.E * upe) return;
-    const int e = (int)(unit / upe);
+    const int chunk = (int)(unit / upe);
     const int pi = (int)(unit % upe);
+    int e = 0;
+    int64_t row0 = 0, row1 = 0;
+    if (!find_chunk(a.gl, a.gl_type, a.E, chunk, kW4Chunk, lane, e, row0, row1)) return;
+    if (row1 > a.R) row1 = a.R;
+    if (row1 <= row0) return;
     const int nb0 = (EPI == EPI_SWIGLU) ? pi : 2 * pi;
     const int nb1 = (EPI == EPI_SWIGLU) ? pi + upe : 2 * pi + 1;
 
     const uint8_t* w0 = p.w4 + (((int64_t)e * NB + nb0) * KB64) * 1024 + lane * 16;
     const uint8_t* w1 = p.w4 + (((int64_t)e * NB + nb1) * KB64) * 1024 + lane * 16;
-    v4i a0[UN], a1[UN];
-    auto load_weights = [&](int kb) {
+    v4i a0[2][UN], a1[2][UN];  // double-buffered weight batches
+    auto load_weights = [&](int buf, int kb) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int k = kb + u;
-            if (k < KB64) {
-                a0[u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
-                a1[u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
-            } else {
-                a0[u] = (v4i){0, 0, 0, 0};
-                a1[u] = (v4i){0, 0, 0, 0};
-            }
+            const int k = kb + u < KB64 ? kb + u : KB64 - 1;
+            a0[buf][u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
+            a1[buf][u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
         }
     };
-    load_weights(0);
-
-    int64_t row0, row1;
-    expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
-    if (row1 > a.R) row1 = a.R;
-    if (row1 <= row0) return;
+    load_weights(0, 0);
 
     const int tok = lane & 31;
     const int hi = lane >> 5;
@@ -182,65 +233,100 @@ __global__ __launch_bounds__(256, 3) void gmm_w4_stream_kernel(W4Args p)
     const int n_groups = a.K / p.group;
     const float* gs = p.gscale + (int64_t)e * n_groups * a.N;
 
-    for (int64_t r0 = row0; r0 < row1; r0 += 32) {
-        const int64_t row = r0 + tok;
-        const bool valid = row < row1;
-        const int8_t* xr = a.x + row * a.K + hi * 16;
-        v16i c0 = {0}, c1 = {0};
-        float f0[16], f1[16];
+    int64_t row[2];
+    bool valid[2];
+    const int8_t* xr[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        row[b] = row0 + 32 * b + tok;
+        valid[b] = row[b] < row1;
+        xr[b] = a.x + (valid[b] ? row[b] : row0) * a.K + hi * 16;
+    }
+    const bool two = row0 + 32 < row1;  // the second token block holds rows (wavefront-uniform)
+
+    v16i c0[2], c1[2];
+    float f0[2][16], f1[2][16];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        c0[b] = (v16i){0};
+        c1[b] = (v16i){0};
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            f0[v] = 0.0f;
-            f1[v] = 0.0f;
+            f0[b][v] = 0.0f;
+            f1[b][v] = 0.0f;
         }
-        if (r0 != row0) load_weights(0);
-        int in_group = 0, grp = 0;
-        for (int kb = 0; kb < KB64; kb += UN) {
-            v4i b0[UN], b1[UN];
+    }
+    int in_group = 0, grp = 0;
+    auto fold = [&]() {  // f += float(acc / 16) * scale[e, grp, channel]
+        const float* s = gs + (int64_t)grp * a.N;
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const bool ok = valid && (kb + u < KB64);
-                b0[u] = ok ? *(const v4i*)(xr + (kb + u) * 64) : (v4i){0, 0, 0, 0};
-                b1[u] = ok ? *(const v4i*)(xr + (kb + u) * 64 + 32) : (v4i){0, 0, 0, 0};
-            }
+        for (int q = 0; q < 4; ++q) {
+            const int ch = 8 * q + 4 * hi;
+            const v4f s0 = *(const v4f*)(s + nb0 * 32 + ch);
+            const v4f s1 = *(const v4f*)(s + nb1 * 32 + ch);
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                if (kb + u < KB64) {
-                    c0 = mfma_i8(nib_lo(a0[u]), b0[u], c0);
-                    c0 = mfma_i8(nib_hi(a0[u]), b1[u], c0);
-                    c1 = mfma_i8(nib_lo(a1[u]), b0[u], c1);
-                    c1 = mfma_i8(nib_hi(a1[u]), b1[u], c1);
-                    if (++in_group == steps_per_group) {
-                        // fold this K group: f += float(acc / 16) * scale[e, grp, channel]
-                        const float* s = gs + (int64_t)grp * a.N;
+            for (int b = 0; b < 2; ++b)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int ch = 8 * q + 4 * hi;
-                            const v4f s0 = *(const v4f*)(s + nb0 * 32 + ch);
-                            const v4f s1 = *(const v4f*)(s + nb1 * 32 + ch);
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                f0[4 * q + j] = f0[4 * q + j] + (float)(c0[4 * q + j] >> 4) * s0[j];
-                                f1[4 * q + j] = f1[4 * q + j] + (float)(c1[4 * q + j] >> 4) * s1[j];
-                            }
-                        }
-                        c0 = (v16i){0};
-                        c1 = (v16i){0};
-                        in_group = 0;
-                        ++grp;
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    f0[b][4 * q + j] = f0[b][4 * q + j] + (float)(c0[b][4 * q + j] >> 4) * s0[j];
+                    f1[b][4 * q + j] = f1[b][4 * q + j] + (float)(c1[b][4 * q + j] >> 4) * s1[j];
                 }
-            }
-            if (kb + UN < KB64) load_weights(kb + UN);
         }
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            c0[b] = (v16i){0};
+            c1[b] = (v16i){0};
+        }
+        in_group = 0;
+        ++grp;
+    };
+    auto batch = [&](int buf, int kb) {
+        v4i bl[UN][2], bh[UN][2];  // [K block][token block]: K 0..31 / 32..63 of the block
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int k = kb + u < KB64 ? kb + u : KB64 - 1;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const bool ok = valid[b] && (b == 0 || two);
+                bl[u][b] = ok ? *(const v4i*)(xr[b] + k * 64) : (v4i){0, 0, 0, 0};
+                bh[u][b] = ok ? *(const v4i*)(xr[b] + k * 64 + 32) : (v4i){0, 0, 0, 0};
+            }
+        }
+        if (kb + UN < KB64) load_weights(buf ^ 1, kb + UN);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (kb + u < KB64) {
+                const v4i l0 = nib_lo(a0[buf][u]), h0 = nib_hi(a0[buf][u]);
+                const v4i l1 = nib_lo(a1[buf][u]), h1 = nib_hi(a1[buf][u]);
+                c0[0] = mfma_i8(l0, bl[u][0], c0[0]);
+                c0[0] = mfma_i8(h0, bh[u][0], c0[0]);
+                c1[0] = mfma_i8(l1, bl[u][0], c1[0]);
+                c1[0] = mfma_i8(h1, bh[u][0], c1[0]);
+                if (two) {
+                    c0[1] = mfma_i8(l0, bl[u][1], c0[1]);
+                    c0[1] = mfma_i8(h0, bh[u][1], c0[1]);
+                    c1[1] = mfma_i8(l1, bl[u][1], c1[1]);
+                    c1[1] = mfma_i8(h1, bh[u][1], c1[1]);
+                }
+                if (++in_group == steps_per_group) fold();
+            }
+        }
+    };
+    for (int kb = 0; kb < KB64; kb += 2 * UN) {
+        batch(0, kb);
+        if (kb + UN < KB64) batch(1, kb + UN);
+    }
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        if (b == 1 && !two) break;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int ch = 8 * q + 4 * hi;
             float g[4], u[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                g[j] = f0[4 * q + j];
-                u[j] = f1[4 * q + j];
+                g[j] = f0[b][4 * q + j];
+                u[j] = f1[b][4 * q + j];
             }
             if (p.bias) {
                 const v4f bg = *(const v4f*)(p.bias + (int64_t)e * a.N + nb0 * 32 + ch);
@@ -251,9 +337,15 @@ __global__ __launch_bounds__(256, 3) void gmm_w4_stream_kernel(W4Args p)
                     u[j] = u[j] + bu[j];
                 }
             }
-            epilogue_run_w4<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u);
+            epilogue_run_w4<EPI>(a, row[b], valid[b], nb0 * 32 + ch, nb1 * 32 + ch, g, u);
         }
     }
+}
+
+// upper bound of the number of 64-row chunks: known on the host without reading the group list
+static int64_t w4_units(int64_t rows, int num_experts, int64_t n)
+{
+    return (rows / kW4Chunk + num_experts) * (n / 64);
 }
 
 static int check_w4(const void* x, const void* w, const float* scale, const int64_t* gl, int gl_type, int64_t rows,
@@ -335,8 +427,8 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     p.gscale = weight_scale;
     p.bias = bias;
     p.group = (int)group_size;
-    const int64_t units = (int64_t)num_experts * (n / 64);
-    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU, 4>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
+    const int64_t units = w4_units(rows, num_experts, n);
+    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
     launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
     return launch_status();
 }
@@ -366,8 +458,8 @@ extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4
     p.gscale = scale;
     p.bias = bias;
     p.group = (int)group_size;
-    const int64_t units = (int64_t)num_experts * (n / 64);
-    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT, 4>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+    const int64_t units = w4_units(rows, num_experts, n);
+    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
                        (hipStream_t)stream, p);
     return launch_status();
 }
