@@ -279,3 +279,76 @@ def test_grouped_matmul_swiglu_quant_v2_against_the_reference_golden(orc):
             assert (out[lo:hi].cpu().to(torch.int32) - q_ref.to(torch.int32)).abs().max() <= 1
             torch.testing.assert_close(out_scale[lo:hi].cpu().double(), mx / 127, rtol=5e-3, atol=1e-6)
         lo = hi
+
+
+# ------------------------------------------------------------------ W4A8 grouped GEMMs, chunk boundaries
+# rows per expert chosen around the 64-row unit of the int4 kernel (and its 32-row token blocks)
+W4_COUNTS = [0, 1, 31, 32, 33, 63, 64, 65, 0, 130, 200, 7]
+
+
+@pytest.mark.parametrize("Kd,N,group", [(256, 128, 128), (512, 192, 256), (128, 64, 128), (256, 128, 0)])
+@pytest.mark.parametrize("gl_type", [0, 1])
+def test_w4_gemms_at_chunk_boundaries(K, orc, Kd, N, group, gl_type):
+    print(f"w4 gemms K={Kd} N={N} group={group} gl_type={gl_type}", flush=True)
+    g = torch.Generator().manual_seed(Kd + N + group)
+    cnt = torch.tensor(W4_COUNTS, dtype=torch.int64)
+    E, R = len(W4_COUNTS), int(cnt.sum())
+    cum = torch.cumsum(cnt, 0)
+    gsz = group if group else Kd
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-8, 8, (E, N, Kd), generator=g, dtype=torch.int8)
+    sg = torch.rand(E, Kd // gsz, N, generator=g) * 0.09 + 0.01
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    bias = torch.randn(E, N, generator=g)
+    gl = (cum if gl_type == 0 else cnt).to(DEV)
+    w4 = K.format_cast_nz_int4(w.to(DEV), 0, N, Kd)
+    # down-GEMM form: f = sum_g float(acc_g) * s_g (+ bias), then the token scale, bf16
+    f = orc.gmm_w4_grouped(x.numpy(), w.numpy(), sg.numpy(), cum.numpy(), gsz)
+    want = orc.w4_rows_to_bf16(f, sx.numpy())
+    got = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), gsz, sx.to(DEV), gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got.cpu()), want)
+    # gate_up form: token scale, SwiGLU, per-row re-quantisation
+    q_want, s_want = orc.swiglu_quant(orc.scale_rows(f, sx.numpy()))
+    q, s = K.gmm1_swiglu_quant_w4(x.to(DEV), w4, sg.to(DEV), gsz, sx.to(DEV), gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+    # with the bias of the offset-corrected A8W4 form (added before the token scale)
+    fb = f + np.repeat(bias.numpy(), W4_COUNTS, axis=0)
+    got_b = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), gsz, sx.to(DEV), gl, gl_type, N, Kd, bias=bias.to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got_b.cpu()), orc.w4_rows_to_bf16(fb, sx.numpy()))
+
+
+# rows per expert around the 128-row tile of the LDS-tiled kernel and its 64-row short-tile path
+TILE_COUNTS = [128, 64, 65, 129, 192, 193, 1, 0, 256, 63, 127, 320]
+
+
+@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320)])
+def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
+    print(f"tiled gemms at tile boundaries K={Kd} N={N}", flush=True)
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(Kd * 3 + N)
+    cnt = torch.tensor(TILE_COUNTS, dtype=torch.int64)
+    E, R = len(TILE_COUNTS), int(cnt.sum())
+    cum = torch.cumsum(cnt, 0)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    acc = K.gmm_i32(x.to(DEV), wnz, cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    want = orc.gmm2_dequant(ref, sx.numpy(), sw.numpy(), cum.numpy())
+    got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt.to(DEV), 1, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got.cpu()), want)
+    q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw.numpy(), cum.numpy()))
+    q, s = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
