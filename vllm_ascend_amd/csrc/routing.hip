@@ -2,13 +2,13 @@
 // permutation of the flattened (token, slot) pairs, and the token gather with
 // fused per-row int8 quantisation.
 //
-// The flat index space [0, R) is cut into chunks of 1024.  Stability needs
+// The flat index space [0, R) is cut into chunks of 256.  Stability needs
 //   dst[f] = off[e] + #{f' < f : ids[f'] == e},
 // which is built in three launches:
 //   1. per-chunk expert histograms (LDS atomics; counts are order independent);
 //   2. one workgroup turns them into per-(chunk, expert) start rows and the
 //      per-expert offsets (exclusive scans);
-//   3. one wavefront per chunk walks its 1024 indices in order, 64 at a time:
+//   3. one wavefront per chunk walks its 256 indices in order, 64 at a time:
 //      lanes with equal expert ids find each other with ballots, rank
 //      themselves by lane number, and the lowest lane advances the running
 //      per-expert cursor kept in LDS.
@@ -18,7 +18,7 @@
 
 namespace moe355 {
 
-constexpr int kChunk = 1024;
+constexpr int kChunk = 256;
 
 struct RouteWs {
     int32_t* chunk_hist;  // [nchunks][E]   histogram, then start row of (chunk, expert)
@@ -54,12 +54,18 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ c
     extern __shared__ int32_t cnt[];  // [E] counts, then [256] partials
     int32_t* partial = cnt + E;
     // column scan over chunks: chunk_hist[c][e] <- number of rows of expert e in chunks before c
+    // (32 chunks at a time: the loads of a batch are independent, so their latencies overlap)
     for (int e = threadIdx.x; e < E; e += 256) {
         int32_t run = 0;
-        for (int c = 0; c < nchunks; ++c) {
-            int32_t v = chunk_hist[(int64_t)c * E + e];
-            chunk_hist[(int64_t)c * E + e] = run;
-            run += v;
+        for (int c0 = 0; c0 < nchunks; c0 += 32) {
+            int32_t v[32];
+#pragma unroll
+            for (int j = 0; j < 32; ++j) v[j] = (c0 + j < nchunks) ? chunk_hist[(int64_t)(c0 + j) * E + e] : 0;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                if (c0 + j < nchunks) chunk_hist[(int64_t)(c0 + j) * E + e] = run;
+                run += v[j];
+            }
         }
         cnt[e] = run;
     }
