@@ -33,7 +33,7 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 # scaled by a copy kernel of known size); filled in from the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/moe_layer_qwen3_decode_hbm_traffic.md: 194221.0 KiB x 2.00 fetched + 4260.2 KiB x 1.00 written
-    "c2_qwen3_decode": 402_200_000,
+    "c2_qwen3_decode": 399_300_000,
 }
 
 
