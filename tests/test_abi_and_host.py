@@ -186,3 +186,44 @@ def test_bench_refuses_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "ONE GPU" in r.stderr
+
+
+def test_w4a8_scheme_specs_and_argument_checks():
+    """Parameter names of vllm_ascend/quantization/methods/w4a8.py:146-196 (one int4 value per int8) with the
+    group dimension of the scales last; group sizes the kernels cannot take are refused at construction."""
+    from vllm_ascend_amd.quant_type import QuantType
+    from vllm_ascend_amd.quantization import get_scheme_class
+
+    cls = get_scheme_class("W4A8_DYNAMIC", "moe")
+    scheme = cls(group_size=256)
+    assert scheme.quant_type == QuantType.W4A8
+    w = scheme.get_weight(4, 512, 1024, torch.bfloat16)
+    assert w["w13_weight"].shape == (4, 1024, 1024) and w["w13_weight"].dtype == torch.int8
+    assert w["w2_weight"].shape == (4, 1024, 512)
+    q = scheme.get_dynamic_quant_param(4, 512, 1024, torch.bfloat16)
+    assert q["w13_weight_scale"].shape == (4, 1024, 4) and q["w2_weight_scale"].shape == (4, 1024, 2)
+    q0 = cls(group_size=0).get_dynamic_quant_param(4, 512, 1024, torch.bfloat16)
+    assert q0["w13_weight_scale"].shape == (4, 1024, 1) and q0["w2_weight_scale"].shape == (4, 1024, 1)
+    for bad in (-64, 32, 100):
+        with pytest.raises(ValueError, match="group_size"):
+            cls(group_size=bad)
+
+
+def test_dense_quant_matmul_argument_checks():
+    """npu_quant_matmul stands in for the call in vllm_ascend/ops/fused_moe/shared_experts.py:262-301: what it
+    cannot do is refused by name before any kernel is launched."""
+    from vllm_ascend_amd import npu_ops
+
+    x = torch.zeros(2, 64, dtype=torch.int8)
+    w = torch.zeros(64, 128, dtype=torch.int8)
+    s = torch.ones(128)
+    with pytest.raises(NotImplementedError, match="offset / bias"):
+        npu_ops.npu_quant_matmul(x, w, s, bias=torch.zeros(128))
+    with pytest.raises(NotImplementedError, match="int8"):
+        npu_ops.npu_quant_matmul(x.to(torch.bfloat16), w, s)
+    with pytest.raises(NotImplementedError, match="pertoken_scale"):
+        npu_ops.npu_quant_matmul(x, w, s, output_dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="output_dtype"):
+        npu_ops.npu_quant_matmul(x, w, s, pertoken_scale=torch.ones(2), output_dtype=torch.float16)
+    with pytest.raises(RuntimeError):   # CPU tensors never reach a kernel: there is no host fallback
+        npu_ops.npu_quant_matmul(x, w, s, output_dtype=torch.int32)

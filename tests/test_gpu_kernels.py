@@ -352,3 +352,23 @@ def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     torch.cuda.synchronize()
     assert np.array_equal(q.cpu().numpy(), q_want)
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
+def test_w4_group_sum_order_on_the_gpu(K, orc):
+    """The order-sensitive case of the CPU suite (terms 2^24, 1, 1 over three scale groups) through the kernel."""
+    Kd, g, N = 192, 64, 64
+    x = torch.zeros(1, Kd, dtype=torch.int8)
+    w = torch.zeros(1, N, Kd, dtype=torch.int8)
+    for grp in range(3):
+        x[0, 64 * grp] = 1
+        w[0, :, 64 * grp] = 1
+    w4 = K.format_cast_nz_int4(w.to(DEV), 0, N, Kd)
+    one = torch.tensor([1], dtype=torch.int64, device=DEV)
+    sx = torch.ones(1, device=DEV)
+    for scales, want in (((2.0 ** 24, 1.0, 1.0), 2.0 ** 24), ((1.0, 1.0, 2.0 ** 24), 2.0 ** 24 + 2)):
+        sg = torch.tensor(scales, dtype=torch.float32).reshape(1, 3, 1).expand(1, 3, N).contiguous()
+        ref = orc.gmm_w4_grouped(x.numpy(), w.numpy(), sg.numpy(), np.array([1], dtype=np.int64), g)
+        assert np.all(ref == np.float32(want))
+        got = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), g, sx, one, 0, N, Kd)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(got.cpu()), orc.w4_rows_to_bf16(ref, np.ones(1, dtype=np.float32)))

@@ -297,3 +297,62 @@ def test_layer_matches_the_dense_reference_within_quantisation_noise():
     w2 = orc.f32_to_bf16(orc.bf16_to_f32(tr.topk_weights) * 2)
     out2 = orc.unpermute(tr.o, tr.expanded_row_idx, w2)
     assert np.array_equal(orc.bf16_to_f32(out2), orc.bf16_to_f32(tr.out) * 2)
+
+
+def test_w4_sum_over_groups_runs_in_ascending_group_order():
+    """f = ((0 + t_0) + t_1) + t_2 in fp32.  With t = (2^24, 1, 1) the ascending order loses both ones
+    (2^24 + 1 ties back to 2^24, twice); any order that adds the ones first gives 2^24 + 2.  Pins the order
+    that the int4 kernel must reproduce."""
+    K, g, N = 192, 64, 32
+    x = np.zeros((1, K), dtype=np.int8)
+    w = np.zeros((1, N, K), dtype=np.int8)
+    for grp in range(3):
+        x[0, 64 * grp] = 1
+        w[0, :, 64 * grp] = 1   # every group's integer sum is 1
+    one = np.array([1], dtype=np.int64)
+    sg = np.zeros((1, 3, N), dtype=np.float32)
+    sg[0, :, :] = np.array([2.0 ** 24, 1.0, 1.0], dtype=np.float32)[:, None]
+    assert np.all(orc.gmm_w4_grouped(x, w, sg, one, g) == np.float32(2.0 ** 24))
+    sg[0, :, :] = np.array([1.0, 1.0, 2.0 ** 24], dtype=np.float32)[:, None]
+    assert np.all(orc.gmm_w4_grouped(x, w, sg, one, g) == np.float32(2.0 ** 24 + 2))
+    sg[0, :, :] = np.array([3.0, 0.0, 2.0 ** 24], dtype=np.float32)[:, None]
+    assert np.all(orc.gmm_w4_grouped(x, w, sg, one, g) == np.float32(2.0 ** 24 + 4))  # 2^24 + 3 rounds to even
+
+
+def test_w4_stage_extremes_and_empty_groups():
+    """Largest magnitudes (x = -128, w = -8 everywhere) stay exact integers in the int32 group sums; rows past
+    the last group stay zero; an empty expert changes nothing."""
+    K, g, N = 256, 128, 32
+    x = np.full((3, K), -128, dtype=np.int8)
+    w = np.full((2, N, K), -8, dtype=np.int8)
+    sg = np.ones((2, K // g, N), dtype=np.float32)
+    f = orc.gmm_w4_grouped(x, w, sg, np.array([0, 2], dtype=np.int64), g)   # expert 0 empty, row 2 unowned
+    assert np.all(f[:2] == np.float32(128 * 8 * K)) and np.all(f[2] == 0)
+    o = orc.w4_rows_to_bf16(f, np.array([0.5, 0.0, 1.0], dtype=np.float32))
+    assert np.all(orc.bf16_to_f32(o[0]) == 128 * 8 * K / 2) and np.all(o[1] == 0) and np.all(o[2] == 0)
+
+
+def test_w4_layer_matches_a_dense_float64_rendering():
+    import sys
+
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _inputs import CONFIGS, bits, make_layer
+    from _layer_utils import oracle_layer, rel_err
+
+    cfg = CONFIGS["c5_small"]
+    d = make_layer(cfg, seed=0)
+    tr = oracle_layer(cfg, d)
+    # the same quantised pipeline in float64 from the traced int8 activations: no fp32 or bf16 rounding
+    g = cfg.w4_group
+    sg2 = d["s2"].numpy().transpose(0, 2, 1)   # [E, G, N]
+    cum = np.cumsum(tr.expert_tokens)
+    o = np.zeros((tr.q1.shape[0], cfg.H), dtype=np.float64)
+    lo = 0
+    for e, hi in enumerate(cum):
+        if hi > lo:
+            q = tr.q1[lo:hi].astype(np.float64).reshape(hi - lo, -1, g)
+            w = d["w2"].numpy()[e].astype(np.float64).reshape(cfg.H, -1, g)
+            part = np.einsum("mgk,ngk->gmn", q, w)
+            o[lo:hi] = (part * sg2[e][:, None, :]).sum(axis=0) * tr.s1[lo:hi, None].astype(np.float64)
+        lo = hi
+    assert rel_err(orc.bf16_to_f32(tr.o), o) <= 1e-2
