@@ -165,7 +165,8 @@ def main() -> int:
         hooked = {"i": 0}
         from vllm_ascend_amd import kernels as K
 
-        orig = K.gmm1_swiglu_quant
+        hook_name = "gmm1_swiglu_quant_w4" if cfg.w4_group >= 0 else "gmm1_swiglu_quant"
+        orig = getattr(K, hook_name)
 
         def timed_gmm1(*a, **kw):
             s, e = evs[hooked["i"]]
@@ -176,7 +177,7 @@ def main() -> int:
             lib.moe355_profile_next_gemm(ctypes.c_void_p(s.cuda_event), ctypes.c_void_p(e.cuda_event))
             return orig(*a, **kw)
 
-        K.gmm1_swiglu_quant = timed_gmm1
+        setattr(K, hook_name, timed_gmm1)
         try:
             torch.cuda.synchronize()
             te0 = time.perf_counter()
@@ -186,7 +187,7 @@ def main() -> int:
             torch.cuda.synchronize()
             te1 = time.perf_counter()
         finally:
-            K.gmm1_swiglu_quant = orig
+            setattr(K, hook_name, orig)
         eager_ms = (te1 - te0) * 1e3 / n
         fired = hooked.get("fired", 0) > 0
         durs = sorted(s.elapsed_time(e) for s, e in evs) if fired else [1.0]  # ms
@@ -208,7 +209,8 @@ def main() -> int:
         if roofline is not None:
             roofline.update({
                 "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                "kernel": ("gmm_tiled_kernel<EPI_SWIGLU>" if (R // cfg.E >= 48 and cfg.H % 64 == 0)
+                "kernel": ("gmm_w4_stream_kernel<EPI_SWIGLU>" if cfg.w4_group >= 0 else
+                           "gmm_tiled_kernel<EPI_SWIGLU>" if (R // cfg.E >= 48 and cfg.H % 64 == 0)
                            else "gmm_stream_kernel<EPI_SWIGLU>") + " (gate_up grouped GEMM + dequant + SwiGLU)",
                 "kernel_avg_us": round(avg_ms * 1e3, 2),
                 "kernel_p50_us": round(durs[len(durs) // 2] * 1e3, 2),

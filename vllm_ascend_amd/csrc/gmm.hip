@@ -220,6 +220,14 @@ static int check_gmm(const void* x, const void* w, const int64_t* gl, int gl_typ
 static thread_local hipEvent_t t_ev_start = nullptr;
 static thread_local hipEvent_t t_ev_stop = nullptr;
 
+void take_profile_events(hipEvent_t& start, hipEvent_t& stop)
+{
+    start = t_ev_start;
+    stop = t_ev_stop;
+    t_ev_start = nullptr;
+    t_ev_stop = nullptr;
+}
+
 template <typename KernelT>
 static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs& a)
 {

@@ -122,6 +122,10 @@ __device__ __forceinline__ void epilogue_quad(const GmmArgs& a, int e, int64_t r
     epilogue_run<EPI>(a, e, row, valid, n0 + ch, n1 + ch, g, u);
 }
 
+// Measurement hook (gmm.hip): hands out, once, the events that moe355_profile_next_gemm armed on this thread
+// (both null when nothing is armed); the caller records them around exactly one kernel launch.
+void take_profile_events(hipEvent_t& start, hipEvent_t& stop);
+
 // SwiGLU values y fp32 [R, I] -> per-row absmax -> int8 + scale (defined in gmm.hip).
 void launch_swiglu_requant(const float* y, const int64_t* gl, int gl_type, int E, int64_t R, int I, int8_t* q,
                            float* qs, hipStream_t st);

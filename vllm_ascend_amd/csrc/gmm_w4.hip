@@ -9,6 +9,8 @@
 // Every `group` K values the accumulator is folded into fp32, f += float(acc) * scale[e, g, n], in
 // ascending group order (one wavefront owns the whole K range of its channels, so the order is the
 // sequential one), then f (+ bias) * token_scale goes through the shared epilogues.
+#include <hip/hip_ext.h>
+
 #include "gmm_common.h"
 
 namespace moe355 {
@@ -428,7 +430,13 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     p.bias = bias;
     p.group = (int)group_size;
     const int64_t units = w4_units(rows, num_experts, n);
-    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    take_profile_events(ev0, ev1);
+    if (ev0 && ev1)
+        hipExtLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st,
+                              ev0, ev1, 0, p);
+    else
+        hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
     launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
     return launch_status();
 }
