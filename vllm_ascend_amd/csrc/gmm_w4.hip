@@ -195,19 +195,26 @@ __device__ __forceinline__ bool find_chunk(const int64_t* gl, int gl_type, int E
 // ascending order (the fp32 sum over scale groups has one fixed order).  An expert with many rows becomes
 // many units that run side by side on different CUs and find the expert's weights in L2 / Infinity Cache,
 // instead of one wavefront streaming the same weights once per 32 rows.
+// The four wavefronts of a workgroup work on the same chunk (four neighbouring tile pairs), so the chunk's
+// tokens go through LDS once per workgroup: every thread loads one 16-byte piece of the 64 x 64-byte K block
+// (rows are read in 64-byte runs instead of 16-byte crumbs per lane), writes it in MFMA-operand order, and
+// each wavefront reads its four B operands back with conflict-free 1 KiB sweeps.
 constexpr int kW4Chunk = 64;
 template <int EPI>
 __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 {
-    constexpr int UN = 2;  // 64-wide K blocks per batch of loads
+    constexpr int UN = 4;  // 64-wide K blocks per batch of loads
     const GmmArgs& a = p.g;
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int NB = a.N >> 5, KB64 = a.K >> 6;
     const int upe = NB >> 1;
-    const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
-    const int chunk = (int)(unit / upe);
-    const int pi = (int)(unit % upe);
+    // workgroup = (chunk, four neighbouring tile pairs); a wavefront past the last pair still stages tokens
+    const int quads = (upe + 3) >> 2;
+    const int chunk = (int)(blockIdx.x / quads);
+    const int pi_raw = (int)(blockIdx.x % quads) * 4 + wave;
+    const bool have = pi_raw < upe;
+    const int pi = have ? pi_raw : 0;
     int e = 0;
     int64_t row0 = 0, row1 = 0;
     if (!find_chunk(a.gl, a.gl_type, a.E, chunk, kW4Chunk, lane, e, row0, row1)) return;
@@ -235,15 +242,21 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     const int n_groups = a.K / p.group;
     const float* gs = p.gscale + (int64_t)e * n_groups * a.N;
 
+    __shared__ __attribute__((aligned(16))) int8_t Bs[2][kW4Chunk * 64];  // two stages of 64 rows x 64 K bytes
     int64_t row[2];
     bool valid[2];
-    const int8_t* xr[2];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
         row[b] = row0 + 32 * b + tok;
         valid[b] = row[b] < row1;
-        xr[b] = a.x + (valid[b] ? row[b] : row0) * a.K + hi * 16;
     }
+    // staging: thread t carries row (t % 16) + 16 * (t / 64), 16-byte piece (t / 16) % 4 of the K block
+    const int srow = (threadIdx.x & 15) + 16 * wave;
+    const int skc = (threadIdx.x >> 4) & 3;
+    int64_t sr = row0 + srow;
+    if (sr > row1 - 1) sr = row1 - 1;  // rows past the chunk's end repeat its last row (never stored)
+    const int8_t* xs = a.x + sr * a.K + skc * 16;
+    const int lds_off = ((((skc >> 1) * 2 + (srow >> 5)) * 64) + (skc & 1) * 32 + (srow & 31)) * 16;
     const bool two = row0 + 32 < row1;  // the second token block holds rows (wavefront-uniform)
 
     v16i c0[2], c1[2];
@@ -282,42 +295,51 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         in_group = 0;
         ++grp;
     };
-    auto batch = [&](int buf, int kb) {
-        v4i bl[UN][2], bh[UN][2];  // [K block][token block]: K 0..31 / 32..63 of the block
+    // tokens: K block kb lives in stage kb & 1; breg carries block kb + 1 until it is written behind the
+    // barrier of the step before it is used
+    auto load_tokens = [&](int kb) { return *(const v4i*)(xs + (int64_t)(kb < KB64 ? kb : KB64 - 1) * 64); };
+    v4i breg = load_tokens(0);
+    *(v4i*)(&Bs[0][lds_off]) = breg;
+    breg = load_tokens(1);
+    __syncthreads();
+    auto step = [&](int buf, int u, int kb) {  // one 64-wide K block
+        v4i bl[2], bh[2];  // [token block]: K 0..31 / 32..63 of the block
+        const int8_t* st = Bs[kb & 1];
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int k = kb + u < KB64 ? kb + u : KB64 - 1;
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const bool ok = valid[b] && (b == 0 || two);
-                bl[u][b] = ok ? *(const v4i*)(xr[b] + k * 64) : (v4i){0, 0, 0, 0};
-                bh[u][b] = ok ? *(const v4i*)(xr[b] + k * 64 + 32) : (v4i){0, 0, 0, 0};
-            }
+        for (int b = 0; b < 2; ++b) {
+            bl[b] = *(const v4i*)(st + ((0 * 2 + b) * 64 + lane) * 16);
+            bh[b] = *(const v4i*)(st + ((1 * 2 + b) * 64 + lane) * 16);
         }
-        if (kb + UN < KB64) load_weights(buf ^ 1, kb + UN);
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            if (kb + u < KB64) {
-                const v4i l0 = nib_lo(a0[buf][u]), h0 = nib_hi(a0[buf][u]);
-                const v4i l1 = nib_lo(a1[buf][u]), h1 = nib_hi(a1[buf][u]);
-                c0[0] = mfma_i8(l0, bl[u][0], c0[0]);
-                c0[0] = mfma_i8(h0, bh[u][0], c0[0]);
-                c1[0] = mfma_i8(l1, bl[u][0], c1[0]);
-                c1[0] = mfma_i8(h1, bh[u][0], c1[0]);
-                if (two) {
-                    c0[1] = mfma_i8(l0, bl[u][1], c0[1]);
-                    c0[1] = mfma_i8(h0, bh[u][1], c0[1]);
-                    c1[1] = mfma_i8(l1, bl[u][1], c1[1]);
-                    c1[1] = mfma_i8(h1, bh[u][1], c1[1]);
-                }
-                if (++in_group == steps_per_group) fold();
-            }
+        *(v4i*)(&Bs[(kb + 1) & 1][lds_off]) = breg;  // block kb + 1 (that stage was last read in step kb - 1)
+        breg = load_tokens(kb + 2);
+        const v4i l0 = nib_lo(a0[buf][u]), h0 = nib_hi(a0[buf][u]);
+        const v4i l1 = nib_lo(a1[buf][u]), h1 = nib_hi(a1[buf][u]);
+        c0[0] = mfma_i8(l0, bl[0], c0[0]);
+        c0[0] = mfma_i8(h0, bh[0], c0[0]);
+        c1[0] = mfma_i8(l1, bl[0], c1[0]);
+        c1[0] = mfma_i8(h1, bh[0], c1[0]);
+        if (two) {
+            c0[1] = mfma_i8(l0, bl[1], c0[1]);
+            c0[1] = mfma_i8(h0, bh[1], c0[1]);
+            c1[1] = mfma_i8(l1, bl[1], c1[1]);
+            c1[1] = mfma_i8(h1, bh[1], c1[1]);
         }
+        if (++in_group == steps_per_group) fold();
+        __syncthreads();  // block kb + 1 is visible; nobody still reads block kb
     };
     for (int kb = 0; kb < KB64; kb += 2 * UN) {
-        batch(0, kb);
-        if (kb + UN < KB64) batch(1, kb + UN);
+        if (kb + UN < KB64) load_weights(1, kb + UN);
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (kb + u < KB64) step(0, u, kb + u);
+        if (kb + UN < KB64) {
+            if (kb + 2 * UN < KB64) load_weights(0, kb + 2 * UN);
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
+                if (kb + UN + u < KB64) step(1, u, kb + UN + u);
+        }
     }
+    if (!have) return;  // (after the last barrier)
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
         if (b == 1 && !two) break;
@@ -344,10 +366,11 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     }
 }
 
-// upper bound of the number of 64-row chunks: known on the host without reading the group list
-static int64_t w4_units(int64_t rows, int num_experts, int64_t n)
+// workgroups: an upper bound of the number of 64-row chunks (known on the host without reading the group
+// list) times the groups of four tile pairs
+static int64_t w4_blocks(int64_t rows, int num_experts, int64_t n)
 {
-    return (rows / kW4Chunk + num_experts) * (n / 64);
+    return (rows / kW4Chunk + num_experts) * ((n / 64 + 3) / 4);
 }
 
 static int check_w4(const void* x, const void* w, const float* scale, const int64_t* gl, int gl_type, int64_t rows,
@@ -429,14 +452,14 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     p.gscale = weight_scale;
     p.bias = bias;
     p.group = (int)group_size;
-    const int64_t units = w4_units(rows, num_experts, n);
+    const int64_t blocks = w4_blocks(rows, num_experts, n);
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     take_profile_events(ev0, ev1);
     if (ev0 && ev1)
-        hipExtLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st,
+        hipExtLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)blocks), dim3(256), 0, st,
                               ev0, ev1, 0, p);
     else
-        hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)blocks), dim3(256), 0, st, p);
     launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
     return launch_status();
 }
@@ -466,8 +489,8 @@ extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4
     p.gscale = scale;
     p.bias = bias;
     p.group = (int)group_size;
-    const int64_t units = w4_units(rows, num_experts, n);
-    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+    const int64_t blocks = w4_blocks(rows, num_experts, n);
+    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT>), dim3((unsigned)blocks), dim3(256), 0,
                        (hipStream_t)stream, p);
     return launch_status();
 }
