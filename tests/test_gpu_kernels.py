@@ -372,3 +372,49 @@ def test_w4_group_sum_order_on_the_gpu(K, orc):
         got = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), g, sx, one, 0, N, Kd)
         torch.cuda.synchronize()
         assert np.array_equal(bits(got.cpu()), orc.w4_rows_to_bf16(ref, np.ones(1, dtype=np.float32)))
+
+
+@pytest.mark.parametrize("R,E,Kd,N", [(24, 8, 256, 128), (1538, 12, 256, 256)])  # streaming / LDS-tiled kernel
+def test_gmm1_swiglu_clamp(K, orc, R, E, Kd, N):
+    """swiglu_limit > 0: gate <= L, up in [-L, L] before the activation (the reference's clamp,
+    csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:461-485)."""
+    print(f"gmm1 clamp R={R} E={E} K={Kd} N={N}", flush=True)
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(R + 5)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    cnt = torch.tensor(TILE_COUNTS, dtype=torch.int64) if R == 1538 else _rand_groups(g, E, R)
+    cum = torch.cumsum(cnt, 0)
+    f = orc.dequant_acc(orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy()), sx.numpy(), sw.numpy(), cum.numpy())
+    limit = float(np.percentile(np.abs(f), 60))  # bites on a large share of the values
+    q_want, s_want = orc.swiglu_quant(f, swiglu_limit=limit)
+    q_free, _ = orc.swiglu_quant(f)
+    assert not np.array_equal(q_want, q_free)
+    q, s = K.gmm1_swiglu_quant(x.to(DEV), K.format_cast_nz(w.to(DEV), W_ENK), sw.to(DEV), sx.to(DEV), cum.to(DEV), 0,
+                               N, Kd, swiglu_limit=limit)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
+def test_w4_gmm1_swiglu_clamp(K, orc):
+    Kd, N, gsz = 256, 128, 128
+    g = torch.Generator().manual_seed(77)
+    cnt = torch.tensor(W4_COUNTS, dtype=torch.int64)
+    E, R = len(W4_COUNTS), int(cnt.sum())
+    cum = torch.cumsum(cnt, 0)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-8, 8, (E, N, Kd), generator=g, dtype=torch.int8)
+    sg = torch.rand(E, Kd // gsz, N, generator=g) * 0.09 + 0.01
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    f = orc.scale_rows(orc.gmm_w4_grouped(x.numpy(), w.numpy(), sg.numpy(), cum.numpy(), gsz), sx.numpy())
+    limit = float(np.percentile(np.abs(f), 60))
+    q_want, s_want = orc.swiglu_quant(f, swiglu_limit=limit)
+    q, s = K.gmm1_swiglu_quant_w4(x.to(DEV), K.format_cast_nz_int4(w.to(DEV), 0, N, Kd), sg.to(DEV), gsz, sx.to(DEV),
+                                  cum.to(DEV), 0, N, Kd, swiglu_limit=limit)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
