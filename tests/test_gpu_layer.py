@@ -152,3 +152,25 @@ def test_layer_with_per_expert_weight_lists():
     torch.cuda.synchronize()
     assert np.array_equal(bits(res2.routed_out), oracle_layer(cfg, d).out)
     assert not torch.equal(res.routed_out, res2.routed_out)
+
+
+@pytest.mark.parametrize("name", ["c2_small", "c4_small", "c5_small"])
+def test_empty_and_single_token_batches(name):
+    """T = 0 (a rank with nothing to do in a padded step) returns an empty result without launching anything
+    that faults; T = 1 is bit-exact like any other batch."""
+    print(f"empty / single-token batch {name}", flush=True)
+    import dataclasses
+
+    cfg = CONFIGS[name]
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV, shared=cfg.shared)
+    res = layer.forward_impl(d["x"][:0].to(DEV), d["logits"][:0].to(DEV))
+    torch.cuda.synchronize()
+    assert tuple(res.routed_out.shape) == (0, cfg.H)
+    assert int(res.expert_tokens.sum()) == 0
+    d1 = dict(d)
+    d1["x"], d1["logits"] = d["x"][:1].contiguous(), d["logits"][:1].contiguous()
+    res = layer.forward_impl(d1["x"].to(DEV), d1["logits"].to(DEV))
+    torch.cuda.synchronize()
+    tr = oracle_layer(dataclasses.replace(cfg, T=1), d1, shared=cfg.shared)
+    assert np.array_equal(bits(res.routed_out), tr.out)

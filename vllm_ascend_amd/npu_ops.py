@@ -56,7 +56,7 @@ def npu_moe_init_routing_v2(x, expert_idx, *, scale=None, offset=None, active_nu
         raise NotImplementedError("npu_moe_init_routing_v2: a partial active_expert_range (expert parallelism) "
                                   "is not supported on one GPU")
     x2 = x.reshape(-1, x.shape[-1])
-    xs, row_idx, tokens, dyn = kernels.init_routing(x2, expert_idx.reshape(x2.shape[0], -1), expert_num, quant_mode,
+    xs, row_idx, tokens, dyn = kernels.init_routing(x2, expert_idx.reshape(x2.shape[0], expert_idx.shape[-1]), expert_num, quant_mode,
                                                     expert_tokens_num_type)
     return xs, row_idx, tokens, dyn
 
