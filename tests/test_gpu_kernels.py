@@ -418,3 +418,47 @@ def test_w4_gmm1_swiglu_clamp(K, orc):
     torch.cuda.synchronize()
     assert np.array_equal(q.cpu().numpy(), q_want)
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
+@pytest.mark.parametrize("T,k,E", [(300, 2, 64), (5000, 4, 16), (33, 8, 8)])
+def test_init_routing_maximum_skew(K, orc, T, k, E):
+    """Every token picks the same k experts (the other experts stay empty): the histogram atomics all collide,
+    and the stable order inside an expert is the flat (token, slot) order."""
+    print(f"init_routing skew T={T} k={k} E={E}", flush=True)
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, 64, generator=g).to(torch.bfloat16)
+    hot = torch.randperm(E, generator=g)[:k].to(torch.int32)
+    ids = hot.repeat(T, 1).contiguous()
+    xs, dst, cnt, sx = K.init_routing(x.to(DEV), ids.to(DEV), E, 1, 1)
+    torch.cuda.synchronize()
+    xo, do, co, so = orc.init_routing(bits(x), ids.numpy(), E, quant=True)
+    assert np.array_equal(dst.cpu().numpy(), do) and np.array_equal(cnt.cpu().numpy(), co)
+    assert np.array_equal(bits(xs), xo) and np.array_equal(sx.cpu().numpy().view(np.uint32), so.view(np.uint32))
+    assert sorted(co.tolist())[-k:] == [T] * k and int(co.sum()) == T * k
+
+
+def test_grouped_gemms_with_one_expert_owning_every_row(K, orc):
+    """Maximum skew for the GEMMs: one expert in the middle owns all rows, all others are empty
+    (both the LDS-tiled and, with few rows, the streaming kernel)."""
+    from vllm_ascend_amd._lib import W_ENK
+
+    for R in (20, 900):
+        E, Kd, N = 8, 256, 128
+        g = torch.Generator().manual_seed(R)
+        x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+        w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+        sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+        sx = torch.rand(R, generator=g) * 0.05 + 0.001
+        cnt = torch.zeros(E, dtype=torch.int64)
+        cnt[5] = R
+        cum = torch.cumsum(cnt, 0)
+        wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+        ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+        assert np.array_equal(K.gmm_i32(x.to(DEV), wnz, cnt.to(DEV), 1, N, Kd).cpu().numpy(), ref)
+        got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd)
+        assert np.array_equal(bits(got.cpu()), orc.gmm2_dequant(ref, sx.numpy(), sw.numpy(), cum.numpy()))
+        q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw.numpy(), cum.numpy()))
+        q, s = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt.to(DEV), 1, N, Kd)
+        torch.cuda.synchronize()
+        assert np.array_equal(q.cpu().numpy(), q_want)
+        assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
