@@ -80,8 +80,8 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
         for (int u = 0; u < UN; ++u) {
             const int k = kb + u;
             if (k < kb_end) {
-                a0[u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
-                a1[u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
+                a0[u] = gload16_nt(w0 + (int64_t)k * 1024);
+                a1[u] = gload16_nt(w1 + (int64_t)k * 1024);
             } else {
                 a0[u] = (v4i){0, 0, 0, 0};
                 a1[u] = (v4i){0, 0, 0, 0};

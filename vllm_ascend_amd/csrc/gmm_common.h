@@ -46,6 +46,16 @@ __device__ __forceinline__ const float* expert_scales(const GmmArgs& a, int e)
     return a.s_list ? a.s_list[e] : a.ch_scale + (int64_t)e * a.N;
 }
 
+// Loads through pointers that may come out of a per-expert pointer table.  The compiler cannot prove that
+// such a pointer is global memory and would emit FLAT loads, which count against the LDS counter as well:
+// every s_waitcnt after them becomes a full drain (vmcnt(0) lgkmcnt(0)) and the software pipeline of the
+// GEMM kernels collapses to one batch in flight.  Saying "global" keeps the waits partial.
+typedef const v4i __attribute__((address_space(1))) * gv4i_ptr;
+typedef const v4f __attribute__((address_space(1))) * gv4f_ptr;
+__device__ __forceinline__ v4i gload16(const void* p) { return *(gv4i_ptr)(uintptr_t)p; }
+__device__ __forceinline__ v4i gload16_nt(const void* p) { return __builtin_nontemporal_load((gv4i_ptr)(uintptr_t)p); }
+__device__ __forceinline__ v4f gload4f(const float* p) { return *(gv4f_ptr)(uintptr_t)p; }
+
 __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c)
 {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
@@ -75,8 +85,8 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
         if (!valid) return;
         const float rs = a.row_scale[row];
         const float* cs = expert_scales(a, e);
-        const v4f s0 = *(const v4f*)(cs + n0 + ch);
-        const v4f s1 = *(const v4f*)(cs + n1 + ch);
+        const v4f s0 = gload4f(cs + n0 + ch);
+        const v4f s1 = gload4f(cs + n1 + ch);
         v4u16 o0, o1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -91,8 +101,8 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
         const int I = a.N >> 1;
         const float rs = a.row_scale[row];
         const float* cs = expert_scales(a, e);
-        const v4f sg = *(const v4f*)(cs + n0 + ch);
-        const v4f su = *(const v4f*)(cs + n1 + ch);
+        const v4f sg = gload4f(cs + n0 + ch);
+        const v4f su = gload4f(cs + n1 + ch);
         v4f yv;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {

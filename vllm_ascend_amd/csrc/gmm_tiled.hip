@@ -133,8 +133,8 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
         const int itc = it < last_it ? it : last_it;
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            Areg[st][0][s] = *(const v4i*)(w0 + ((int64_t)itc * 2 + s) * 1024);
-            Areg[st][1][s] = *(const v4i*)(w1 + ((int64_t)itc * 2 + s) * 1024);
+            Areg[st][0][s] = gload16(w0 + ((int64_t)itc * 2 + s) * 1024);
+            Areg[st][1][s] = gload16(w1 + ((int64_t)itc * 2 + s) * 1024);
         }
     };
     const int8_t* xrow[CHUNKS];
@@ -238,8 +238,8 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
     if constexpr (EPI != EPI_I32) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            s0[q] = *(const v4f*)(cs + nb0 * 32 + 8 * q + 4 * hi);
-            s1[q] = *(const v4f*)(cs + nb1 * 32 + 8 * q + 4 * hi);
+            s0[q] = gload4f(cs + nb0 * 32 + 8 * q + 4 * hi);
+            s1[q] = gload4f(cs + nb1 * 32 + 8 * q + 4 * hi);
         }
     }
 #pragma unroll
