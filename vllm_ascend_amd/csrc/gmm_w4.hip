@@ -200,10 +200,11 @@ __device__ __forceinline__ bool find_chunk(const int64_t* gl, int gl_type, int E
 // (rows are read in 64-byte runs instead of 16-byte crumbs per lane), writes it in MFMA-operand order, and
 // each wavefront reads its four B operands back with conflict-free 1 KiB sweeps.
 constexpr int kW4Chunk = 64;
-template <int EPI>
+constexpr int kW4LdsGroups = 32;  // K groups whose scales are kept in LDS (8 KiB per wavefront)
+// LDS_SCALES: the group scales of the wavefront's channels fit LDS (K / group <= kW4LdsGroups)
+template <int EPI, bool LDS_SCALES>
 __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 {
-    constexpr int UN = 4;  // 64-wide K blocks per batch of loads
     const GmmArgs& a = p.g;
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -225,16 +226,16 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 
     const uint8_t* w0 = p.w4 + (((int64_t)e * NB + nb0) * KB64) * 1024 + lane * 16;
     const uint8_t* w1 = p.w4 + (((int64_t)e * NB + nb1) * KB64) * 1024 + lane * 16;
-    v4i a0[2][UN], a1[2][UN];  // double-buffered weight batches
-    auto load_weights = [&](int buf, int kb) {
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int k = kb + u < KB64 ? kb + u : KB64 - 1;
-            a0[buf][u] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
-            a1[buf][u] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
-        }
+    // weights and tokens: rings of RW single K blocks, requested RW - 1 blocks ahead of their MFMAs.  Both
+    // rings have the same depth on purpose: the memory counter retires loads in order, so waiting for a
+    // token block that was requested late would also wait for every weight block requested before it.
+    constexpr int RW = 6;
+    v4i a0[RW], a1[RW];
+    auto load_weights = [&](int slot, int kb) {
+        const int k = kb < KB64 ? kb : KB64 - 1;  // past the end: a valid block that is never used
+        a0[slot] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
+        a1[slot] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
     };
-    load_weights(0, 0);
 
     const int tok = lane & 31;
     const int hi = lane >> 5;
@@ -271,22 +272,35 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
             f1[b][v] = 0.0f;
         }
     }
-    int in_group = 0, grp = 0;
-    auto fold = [&]() {  // f += float(acc / 16) * scale[e, grp, channel]
-        const float* s = gs + (int64_t)grp * a.N;
+    // The scales of this wavefront's 64 channels for every K group sit in LDS (when they fit: up to 32
+    // groups), loaded once up front: the K loop then has no load whose result is needed at once, and its
+    // waits for weights and tokens stay partial.
+    __shared__ float Ss[4][LDS_SCALES ? kW4LdsGroups * 64 : 1];
+    if constexpr (LDS_SCALES) {
+        const int ch = lane < 32 ? nb0 * 32 + lane : nb1 * 32 + (lane - 32);
+        for (int g0 = 0; g0 < n_groups; g0 += 8) {  // eight loads in flight at a time
+            float t[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ch = 8 * q + 4 * hi;
-            const v4f s0 = *(const v4f*)(s + nb0 * 32 + ch);
-            const v4f s1 = *(const v4f*)(s + nb1 * 32 + ch);
+            for (int j = 0; j < 8; ++j) t[j] = gs[(int64_t)(g0 + j < n_groups ? g0 + j : n_groups - 1) * a.N + ch];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (g0 + j < n_groups) Ss[wave][(g0 + j) * 64 + lane] = t[j];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RW - 1; ++i) load_weights(i, i);
+    int in_group = 0, grp = 0;
+    // f += float(acc / 16) * scale[e, grp, channel]
+    auto fold_with = [&](const v4f* s0, const v4f* s1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    f0[b][4 * q + j] = f0[b][4 * q + j] + (float)(c0[b][4 * q + j] >> 4) * s0[j];
-                    f1[b][4 * q + j] = f1[b][4 * q + j] + (float)(c1[b][4 * q + j] >> 4) * s1[j];
+                    f0[b][4 * q + j] = f0[b][4 * q + j] + (float)(c0[b][4 * q + j] >> 4) * s0[q][j];
+                    f1[b][4 * q + j] = f1[b][4 * q + j] + (float)(c1[b][4 * q + j] >> 4) * s1[q][j];
                 }
-        }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             c0[b] = (v16i){0};
@@ -295,14 +309,36 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         in_group = 0;
         ++grp;
     };
-    // tokens: K block kb lives in stage kb & 1; breg carries block kb + 1 until it is written behind the
-    // barrier of the step before it is used
+    auto fold = [&]() {
+        v4f s0[4], s1[4];
+        if constexpr (LDS_SCALES) {
+            const float* sl = &Ss[wave][grp * 64 + 4 * hi];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                s0[q] = *(const v4f*)(sl + 8 * q);
+                s1[q] = *(const v4f*)(sl + 32 + 8 * q);
+            }
+            fold_with(s0, s1);
+        } else {
+            const float* s = gs + (int64_t)grp * a.N + 4 * hi;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                s0[q] = *(const v4f*)(s + nb0 * 32 + 8 * q);
+                s1[q] = *(const v4f*)(s + nb1 * 32 + 8 * q);
+            }
+            fold_with(s0, s1);
+        }
+    };
+    // tokens: K block kb lives in LDS stage kb & 1; treg[(kb) % RW] carries block kb from its load (RW - 1
+    // steps before its MFMAs) until it is written to LDS in the step before it is used
     auto load_tokens = [&](int kb) { return *(const v4i*)(xs + (int64_t)(kb < KB64 ? kb : KB64 - 1) * 64); };
-    v4i breg = load_tokens(0);
-    *(v4i*)(&Bs[0][lds_off]) = breg;
-    breg = load_tokens(1);
+    v4i treg[RW];
+    treg[0] = load_tokens(0);
+    *(v4i*)(&Bs[0][lds_off]) = treg[0];
+#pragma unroll
+    for (int i = 1; i < RW; ++i) treg[i] = load_tokens(i);
     __syncthreads();
-    auto step = [&](int buf, int u, int kb) {  // one 64-wide K block
+    auto step = [&](int slot, int kb) {  // one 64-wide K block; slot = kb % RW (compile time)
         v4i bl[2], bh[2];  // [token block]: K 0..31 / 32..63 of the block
         const int8_t* st = Bs[kb & 1];
 #pragma unroll
@@ -310,10 +346,11 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
             bl[b] = *(const v4i*)(st + ((0 * 2 + b) * 64 + lane) * 16);
             bh[b] = *(const v4i*)(st + ((1 * 2 + b) * 64 + lane) * 16);
         }
-        *(v4i*)(&Bs[(kb + 1) & 1][lds_off]) = breg;  // block kb + 1 (that stage was last read in step kb - 1)
-        breg = load_tokens(kb + 2);
-        const v4i l0 = nib_lo(a0[buf][u]), h0 = nib_hi(a0[buf][u]);
-        const v4i l1 = nib_lo(a1[buf][u]), h1 = nib_hi(a1[buf][u]);
+        *(v4i*)(&Bs[(kb + 1) & 1][lds_off]) = treg[(slot + 1) % RW];  // block kb + 1 (stage last read in step kb - 1)
+        treg[slot] = load_tokens(kb + RW);   // block kb has left its register in the step before
+        const v4i l0 = nib_lo(a0[slot]), h0 = nib_hi(a0[slot]);
+        const v4i l1 = nib_lo(a1[slot]), h1 = nib_hi(a1[slot]);
+        load_weights((slot + RW - 1) % RW, kb + RW - 1);  // the slot block kb - 1 has just left
         c0[0] = mfma_i8(l0, bl[0], c0[0]);
         c0[0] = mfma_i8(h0, bh[0], c0[0]);
         c1[0] = mfma_i8(l1, bl[0], c1[0]);
@@ -327,18 +364,15 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         if (++in_group == steps_per_group) fold();
         __syncthreads();  // block kb + 1 is visible; nobody still reads block kb
     };
-    for (int kb = 0; kb < KB64; kb += 2 * UN) {
-        if (kb + UN < KB64) load_weights(1, kb + UN);
+    // whole passes through the ring without a condition on kb; the remainder is peeled
+    const int kb_full = (KB64 / RW) * RW;
+    for (int kb = 0; kb < kb_full; kb += RW) {
 #pragma unroll
-        for (int u = 0; u < UN; ++u)
-            if (kb + u < KB64) step(0, u, kb + u);
-        if (kb + UN < KB64) {
-            if (kb + 2 * UN < KB64) load_weights(0, kb + 2 * UN);
-#pragma unroll
-            for (int u = 0; u < UN; ++u)
-                if (kb + UN + u < KB64) step(1, u, kb + UN + u);
-        }
+        for (int i = 0; i < RW; ++i) step(i, kb + i);
     }
+#pragma unroll
+    for (int i = 0; i < RW - 1; ++i)
+        if (kb_full + i < KB64) step(i, kb_full + i);
     if (!have) return;  // (after the last barrier)
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
@@ -371,6 +405,17 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 static int64_t w4_blocks(int64_t rows, int num_experts, int64_t n)
 {
     return (rows / kW4Chunk + num_experts) * ((n / 64 + 3) / 4);
+}
+
+template <int EPI>
+static void launch_w4(const W4Args& p, int64_t blocks, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
+{
+    const bool lds_scales = p.g.K / p.group <= kW4LdsGroups;
+    auto kernel = lds_scales ? gmm_w4_stream_kernel<EPI, true> : gmm_w4_stream_kernel<EPI, false>;
+    if (ev0 && ev1)
+        hipExtLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, st, ev0, ev1, 0, p);
+    else
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
 }
 
 static int check_w4(const void* x, const void* w, const float* scale, const int64_t* gl, int gl_type, int64_t rows,
@@ -455,11 +500,7 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     const int64_t blocks = w4_blocks(rows, num_experts, n);
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     take_profile_events(ev0, ev1);
-    if (ev0 && ev1)
-        hipExtLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)blocks), dim3(256), 0, st,
-                              ev0, ev1, 0, p);
-    else
-        hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_SWIGLU>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+    launch_w4<EPI_SWIGLU>(p, blocks, st, ev0, ev1);
     launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
     return launch_status();
 }
@@ -490,7 +531,6 @@ extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4
     p.bias = bias;
     p.group = (int)group_size;
     const int64_t blocks = w4_blocks(rows, num_experts, n);
-    hipLaunchKernelGGL((gmm_w4_stream_kernel<EPI_DEQUANT>), dim3((unsigned)blocks), dim3(256), 0,
-                       (hipStream_t)stream, p);
+    launch_w4<EPI_DEQUANT>(p, blocks, (hipStream_t)stream, nullptr, nullptr);
     return launch_status();
 }
