@@ -242,12 +242,23 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
             s1[q] = gload4f(cs + nb1 * 32 + 8 * q + 4 * hi);
         }
     }
+    // every token scale is requested before the first store: the memory counter retires in order, so a load
+    // behind a block's stores would wait for their acknowledgement, once per token block
+    float rs_all[BMT];
+#pragma unroll
+    for (int b = 0; b < BMT; ++b) {
+        rs_all[b] = 0.0f;
+        if constexpr (EPI != EPI_I32) {
+            const int64_t row = row0 + b * 32 + tok;
+            rs_all[b] = a.row_scale[row < row_end ? row : row_end - 1];
+            if (row >= row_end) rs_all[b] = 0.0f;
+        }
+    }
 #pragma unroll
     for (int b = 0; b < BMT; ++b) {
         const int64_t row = row0 + b * 32 + tok;
         const bool valid = row < row_end;
-        float rs = 0.0f;
-        if constexpr (EPI != EPI_I32) rs = valid ? a.row_scale[row] : 0.0f;
+        const float rs = rs_all[b];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int ch = 8 * q + 4 * hi;  // first of this lane's four channels inside the tile
