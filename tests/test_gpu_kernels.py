@@ -325,7 +325,10 @@ def test_w4_gemms_at_chunk_boundaries(K, orc, Kd, N, group, gl_type):
 TILE_COUNTS = [128, 64, 65, 129, 192, 193, 1, 0, 256, 63, 127, 320]
 
 
-@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320)])
+# K >= 4096 at about 128 rows per expert selects the 256-row weight-streaming tiles (tall and wide ones occur in
+# TILE_COUNTS); the K values leave every remainder of the four- and five-stage rings
+@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320), (4096, 256), (4160, 320), (4224, 128),
+                                  (4288, 256), (4352, 192), (4416, 1152)])
 def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     print(f"tiled gemms at tile boundaries K={Kd} N={N}", flush=True)
     from vllm_ascend_amd._lib import W_ENK
@@ -374,7 +377,8 @@ def test_w4_group_sum_order_on_the_gpu(K, orc):
         assert np.array_equal(bits(got.cpu()), orc.w4_rows_to_bf16(ref, np.ones(1, dtype=np.float32)))
 
 
-@pytest.mark.parametrize("R,E,Kd,N", [(24, 8, 256, 128), (1538, 12, 256, 256)])  # streaming / LDS-tiled kernel
+# streaming / LDS-tiled / 256-row weight-streaming kernel
+@pytest.mark.parametrize("R,E,Kd,N", [(24, 8, 256, 128), (1538, 12, 256, 256), (1538, 12, 4096, 128)])
 def test_gmm1_swiglu_clamp(K, orc, R, E, Kd, N):
     """swiglu_limit > 0: gate <= L, up in [-L, L] before the activation (the reference's clamp,
     csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:461-485)."""

@@ -240,18 +240,22 @@ static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs
     }
 }
 
-// Rows per expert decide the kernel: few rows -> weight streaming; many -> LDS-tiled MFMA kernel.
+// Rows per expert decide the kernel: few rows -> weight streaming over single wavefronts; many -> LDS-tiled
+// MFMA kernel with 128-row tiles; in between, when K is long enough to amortise a tile's fill and epilogue, the
+// 256-row weight-streaming tiles that fetch an expert's weights once.
 static int tiled_bm(const GmmArgs& a)
 {
-    static const char* force = getenv("MOE355_GEMM");  // development knob: 's' stream, 't' tiled 128, 'T' tiled 256
+    // development knob: 's' stream, 't' 128-row tiles, 'T' 256-row weight-streaming tiles, 'u' 64-row tiles
+    static const char* force = getenv("MOE355_GEMM");
     if (a.K % 64 != 0) return 0;
     if (force && force[0] == 's') return 0;
     if (force && force[0] == 't') return 128;
     if (force && force[0] == 'T') return 256;
     if (force && force[0] == 'u') return 64;
     const int64_t avg = a.R / a.E;
-    if (avg >= 48) return 128;
-    return 0;
+    if (avg < 48) return 0;
+    if (avg <= 256 && a.K >= 4096) return 256;
+    return 128;
 }
 
 static size_t tiled_ws_max(int64_t rows, int E)

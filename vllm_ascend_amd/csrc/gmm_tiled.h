@@ -13,10 +13,10 @@ struct TileMap {
     int32_t* row_end;    // [max_tiles] end of the expert's rows
 };
 
-// bytes of scratch for the tile map (BM = rows per tile: 128 or 256)
+// bytes of scratch for the tile map (BM = rows per tile: 64, 128 or 256)
 size_t tiled_workspace_bytes(int64_t rows, int E, int BM);
 
-// epi: EPI_*; bm: 128 or 256.  ev0/ev1: optional events recorded around the GEMM kernel itself.
+// epi: EPI_*; bm: 64 or 128 (LDS-tiled kernel) or 256 (weight-streaming tiles).  ev0/ev1: optional events recorded around the GEMM kernel itself.
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
                       hipEvent_t ev1);
 

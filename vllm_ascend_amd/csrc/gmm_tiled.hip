@@ -86,6 +86,99 @@ struct TiledLds {
     static constexpr int BYTES = RING * STAGE_BYTES > EPI_BYTES ? RING * STAGE_BYTES : EPI_BYTES;
 };
 
+// Epilogue of one wavefront: BMT token blocks x two 32-channel storage tiles (nb0, nb1) out of the MFMA
+// accumulators.  In the accumulators a lane owns one token and scattered runs of four channels;
+// written like that every store would touch 64 different cache lines.  The wavefront instead
+// turns one 32-token block at a time through a private LDS patch (token-major, 128 data bytes per
+// token and tile) and stores whole 128-byte row segments: 8 lanes per token row.
+template <int EPI, int BMT>
+__device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&acc)[2][BMT], int64_t row0,
+                                               int64_t row_end, int nb0, int nb1, int8_t* patch, int lane)
+{
+    constexpr int ROWB = TiledLds<EPI, BMT, 3>::ROWB;
+    const int tok = lane & 31;
+    const int hi = lane >> 5;
+    const float* cs = (a.ch_scale || a.s_list) ? expert_scales(a, e) : nullptr;
+    v4f s0[4], s1[4];
+    if constexpr (EPI != EPI_I32) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            s0[q] = gload4f(cs + nb0 * 32 + 8 * q + 4 * hi);
+            s1[q] = gload4f(cs + nb1 * 32 + 8 * q + 4 * hi);
+        }
+    }
+    // every token scale is requested before the first store: the memory counter retires in order, so a load
+    // behind a block's stores would wait for their acknowledgement, once per token block
+    float rs_all[BMT];
+#pragma unroll
+    for (int b = 0; b < BMT; ++b) {
+        rs_all[b] = 0.0f;
+        if constexpr (EPI != EPI_I32) {
+            const int64_t row = row0 + b * 32 + tok;
+            rs_all[b] = a.row_scale[row < row_end ? row : row_end - 1];
+            if (row >= row_end) rs_all[b] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BMT; ++b) {
+        const int64_t row = row0 + b * 32 + tok;
+        const bool valid = row < row_end;
+        const float rs = rs_all[b];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int ch = 8 * q + 4 * hi;  // first of this lane's four channels inside the tile
+            if constexpr (EPI == EPI_I32) {
+                *(v4i*)(patch + tok * ROWB + ch * 4) =
+                    (v4i){acc[0][b][4 * q], acc[0][b][4 * q + 1], acc[0][b][4 * q + 2], acc[0][b][4 * q + 3]};
+                *(v4i*)(patch + 32 * ROWB + tok * ROWB + ch * 4) =
+                    (v4i){acc[1][b][4 * q], acc[1][b][4 * q + 1], acc[1][b][4 * q + 2], acc[1][b][4 * q + 3]};
+            } else if constexpr (EPI == EPI_DEQUANT) {
+                v4u16 o0, o1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    o0[j] = f32_to_bf16(((float)acc[0][b][4 * q + j] * rs) * s0[q][j]);
+                    o1[j] = f32_to_bf16(((float)acc[1][b][4 * q + j] * rs) * s1[q][j]);
+                }
+                // both tiles are adjacent in the output row: 64 bf16 = 128 bytes per token
+                *(v4u16*)(patch + tok * ROWB + ch * 2) = o0;
+                *(v4u16*)(patch + tok * ROWB + 64 + ch * 2) = o1;
+            } else {
+                v4f yv;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float gg = ((float)acc[0][b][4 * q + j] * rs) * s0[q][j];
+                    float uu = ((float)acc[1][b][4 * q + j] * rs) * s1[q][j];
+                    if (a.limit > 0.0f) {
+                        gg = gg > a.limit ? a.limit : gg;
+                        uu = uu > a.limit ? a.limit : uu;
+                        uu = uu < -a.limit ? -a.limit : uu;
+                    }
+                    yv[j] = m_silu(gg) * uu;
+                }
+                *(v4f*)(patch + tok * ROWB + ch * 4) = yv;
+            }
+        }
+        // read back row-major: lane -> (row r8 + 8*p, 16-byte column c16)
+        const int c16 = lane & 7, r8 = lane >> 3;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int r = r8 + 8 * p;
+            const int64_t orow = row0 + b * 32 + r;
+            if (orow < row_end) {
+                if constexpr (EPI == EPI_I32) {
+                    *(v4i*)(a.acc + orow * a.N + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                    *(v4i*)(a.acc + orow * a.N + nb1 * 32 + c16 * 4) =
+                        *(const v4i*)(patch + 32 * ROWB + r * ROWB + c16 * 16);
+                } else if constexpr (EPI == EPI_DEQUANT) {
+                    *(v4i*)(a.out + orow * a.N + nb0 * 32 + c16 * 8) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                } else {
+                    *(v4i*)(a.y + orow * (a.N >> 1) + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                }
+            }
+        }
+    }
+}
+
 // One tile of BMT token blocks: rows [row0, row_end) of expert e (at most 32 * BMT of them are computed),
 // column block nt.
 // RING = depth of the operand ring in registers: weights are requested RING - 1 K blocks ahead, tokens RING.
@@ -224,101 +317,16 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
     }
 #undef MOE355_STEP
 
-    // ---- epilogue.  In the accumulators a lane owns one token and scattered runs of four channels;
-    // written like that every store would touch 64 different cache lines.  Each wavefront instead
-    // turns one 32-token block at a time through a private LDS patch (token-major, 128 data bytes per
-    // token and tile) and stores whole 128-byte row segments: 8 lanes per token row.
     __syncthreads();  // all wavefronts are done reading the token stages; LDS is reused below
     if (!have) return;
-    int8_t* patch = lds_raw + wave * (PATCHES * 32 * ROWB);
-    const int tok = lane & 31;
-    const int hi = lane >> 5;
-    const float* cs = (a.ch_scale || a.s_list) ? expert_scales(a, e) : nullptr;
-    v4f s0[4], s1[4];
-    if constexpr (EPI != EPI_I32) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            s0[q] = gload4f(cs + nb0 * 32 + 8 * q + 4 * hi);
-            s1[q] = gload4f(cs + nb1 * 32 + 8 * q + 4 * hi);
-        }
-    }
-    // every token scale is requested before the first store: the memory counter retires in order, so a load
-    // behind a block's stores would wait for their acknowledgement, once per token block
-    float rs_all[BMT];
-#pragma unroll
-    for (int b = 0; b < BMT; ++b) {
-        rs_all[b] = 0.0f;
-        if constexpr (EPI != EPI_I32) {
-            const int64_t row = row0 + b * 32 + tok;
-            rs_all[b] = a.row_scale[row < row_end ? row : row_end - 1];
-            if (row >= row_end) rs_all[b] = 0.0f;
-        }
-    }
-#pragma unroll
-    for (int b = 0; b < BMT; ++b) {
-        const int64_t row = row0 + b * 32 + tok;
-        const bool valid = row < row_end;
-        const float rs = rs_all[b];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ch = 8 * q + 4 * hi;  // first of this lane's four channels inside the tile
-            if constexpr (EPI == EPI_I32) {
-                *(v4i*)(patch + tok * ROWB + ch * 4) =
-                    (v4i){acc[0][b][4 * q], acc[0][b][4 * q + 1], acc[0][b][4 * q + 2], acc[0][b][4 * q + 3]};
-                *(v4i*)(patch + 32 * ROWB + tok * ROWB + ch * 4) =
-                    (v4i){acc[1][b][4 * q], acc[1][b][4 * q + 1], acc[1][b][4 * q + 2], acc[1][b][4 * q + 3]};
-            } else if constexpr (EPI == EPI_DEQUANT) {
-                v4u16 o0, o1;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    o0[j] = f32_to_bf16(((float)acc[0][b][4 * q + j] * rs) * s0[q][j]);
-                    o1[j] = f32_to_bf16(((float)acc[1][b][4 * q + j] * rs) * s1[q][j]);
-                }
-                // both tiles are adjacent in the output row: 64 bf16 = 128 bytes per token
-                *(v4u16*)(patch + tok * ROWB + ch * 2) = o0;
-                *(v4u16*)(patch + tok * ROWB + 64 + ch * 2) = o1;
-            } else {
-                v4f yv;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float gg = ((float)acc[0][b][4 * q + j] * rs) * s0[q][j];
-                    float uu = ((float)acc[1][b][4 * q + j] * rs) * s1[q][j];
-                    if (a.limit > 0.0f) {
-                        gg = gg > a.limit ? a.limit : gg;
-                        uu = uu > a.limit ? a.limit : uu;
-                        uu = uu < -a.limit ? -a.limit : uu;
-                    }
-                    yv[j] = m_silu(gg) * uu;
-                }
-                *(v4f*)(patch + tok * ROWB + ch * 4) = yv;
-            }
-        }
-        // read back row-major: lane -> (row r8 + 8*p, 16-byte column c16)
-        const int c16 = lane & 7, r8 = lane >> 3;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const int r = r8 + 8 * p;
-            const int64_t orow = row0 + b * 32 + r;
-            if (orow < row_end) {
-                if constexpr (EPI == EPI_I32) {
-                    *(v4i*)(a.acc + orow * a.N + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
-                    *(v4i*)(a.acc + orow * a.N + nb1 * 32 + c16 * 4) =
-                        *(const v4i*)(patch + 32 * ROWB + r * ROWB + c16 * 16);
-                } else if constexpr (EPI == EPI_DEQUANT) {
-                    *(v4i*)(a.out + orow * a.N + nb0 * 32 + c16 * 8) = *(const v4i*)(patch + r * ROWB + c16 * 16);
-                } else {
-                    *(v4i*)(a.y + orow * (a.N >> 1) + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
-                }
-            }
-        }
-    }
+    tiled_epilogue<EPI, BMT>(a, e, acc, row0, row_end, nb0, nb1, lds_raw + wave * (PATCHES * 32 * ROWB), lane);
 }
 
 // The last tile of an expert is usually short.  Tiles of at most 64 rows run the two-block body (half the
 // MFMAs and half the token traffic of a full tile) inside the same launch, next to the full tiles of their
 // expert, so that they still find the expert's weights in the L2 of their XCD.
 template <int EPI, int BMT, int RING>
-__global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+__global__ __launch_bounds__(256, (BMT <= 2 ? 3 : 2)) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
 {
     __shared__ __attribute__((aligned(16))) int8_t lds_raw[TiledLds<EPI, BMT, RING>::BYTES];
     // ---- which tile: XCD-aware remap of the 1-D grid over the tiles that exist (workgroup i runs on
@@ -341,13 +349,208 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : (BMT <= 4 ? 2 : 1))) void gmm_
             return;
         }
     }
-    if constexpr (BMT > 4) {
-        if (row_end - row0 <= 128) {
-            tiled_body<EPI, 4, RING>(a, e, row0, row_end, nt, lds_raw);
-            return;
-        }
-    }
     tiled_body<EPI, BMT, RING>(a, e, row0, row_end, nt, lds_raw);
+}
+
+// ------------------------------------------------------------------ weight-streaming tiles
+// Tiles for shapes whose grouped GEMM is bound by streaming the weights (a few hundred rows per expert at
+// most).  A workgroup of eight wavefronts works on up to 256 rows of one expert, so that an expert with up to
+// 256 rows fetches its weights from HBM exactly once; every wavefront computes 128 tokens x one channel group
+// (two storage tiles) with the accumulator layout and the epilogue of the 128-row tiles.
+//   tall tile (129..256 rows left): wavefront (h, g) = token half h x channel group g of 4 -> 256 x 256;
+//   wide tile (at most 128 rows left): wavefront g = channel group g of 8 -> 128 x 512, which halves the
+//   token traffic per weight byte (tokens come from L2, and that traffic costs weight bandwidth).
+// Both operands reach LDS by LDS-direct loads (no register staging, so the prefetch depth costs no registers).
+// A stage holds the weights of 64 K values (every storage tile x 2 K steps is a contiguous 1 KiB MFMA operand
+// that is copied as it lies) and the tokens' 64 bytes (row-major, with a rotation of the 16-byte chunks).
+// The compiler does not count LDS-direct loads against the LDS reads that consume them: the wait for a stage
+// is written by hand, before the barrier that publishes the stage.
+constexpr int kWideLdsBytes = 163840;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+#define MOE355_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define MOE355_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+template <int EPI, bool WIDE>
+__device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
+                                                 int8_t* lds)
+{
+    constexpr int GROUPS = WIDE ? 8 : 4;            // channel groups (two storage tiles each) per workgroup
+    constexpr int A_BYTES = GROUPS * 4096;          // weights of a stage
+    constexpr int STAGE = A_BYTES + (WIDE ? 8192 : 16384);
+    constexpr int S = kWideLdsBytes / STAGE;        // 4 wide, 5 tall
+    constexpr int NA = WIDE ? 4 : 2;                // weight loads per wavefront and stage
+    constexpr int ROWB = TiledLds<EPI, 4, 3>::ROWB;
+    constexpr int PATCHES = TiledLds<EPI, 4, 3>::PATCHES;
+    static_assert(8 * PATCHES * 32 * ROWB <= S * STAGE, "epilogue patches fit the stages");
+    static_assert(S * STAGE <= kWideLdsBytes && S >= 3, "stages fit LDS");
+
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int h = WIDE ? 0 : wave >> 2;
+    const int g = WIDE ? wave : wave & 3;
+    const int NB = a.N >> 5, KB = a.K >> 5;
+    const int half_tiles = NB >> 1;
+    auto tiles_of = [&](int cg, int& t0, int& t1) -> bool {
+        if constexpr (EPI == EPI_SWIGLU) {
+            t0 = cg;
+            t1 = cg + half_tiles;
+            return cg < half_tiles;
+        } else {
+            t0 = 2 * cg;
+            t1 = t0 + 1;
+            return t1 < NB;
+        }
+    };
+    // what this wavefront computes
+    int nb0, nb1;
+    const bool have = tiles_of(nt * GROUPS + g, nb0, nb1);
+    const int64_t hrow0 = row0 + 128 * h;
+    const bool active = have && hrow0 < row_end;
+
+    // what this wavefront copies.  Weights: tall -- storage tile wave % 2 of group wave / 2; wide -- both
+    // storage tiles of group wave; always both K steps of the stage (2 KiB contiguous per tile).
+    const int8_t* we = expert_weights(a, e);
+    const int8_t* wsrc[WIDE ? 2 : 1];
+    if constexpr (WIDE) {
+        wsrc[0] = we + (int64_t)(have ? nb0 : 0) * KB * 1024 + lane * 16;
+        wsrc[1] = we + (int64_t)(have ? nb1 : 0) * KB * 1024 + lane * 16;
+    } else {
+        int l0, l1;
+        const bool lhave = tiles_of(nt * GROUPS + (wave >> 1), l0, l1);
+        wsrc[0] = we + (int64_t)(lhave ? ((wave & 1) ? l1 : l0) : 0) * KB * 1024 + lane * 16;
+    }
+    // Tokens: one load covers 16 rows x the 64 K bytes of a stage, four neighbouring lanes on one row (one
+    // 64-byte line per lane quad).  LDS slot of (row r, 16-byte chunk c) inside its 16-row KiB:
+    // 4 * (r % 16) + (c + (r % 16) / 4) % 4 -- the rotation spreads the MFMA operand reads (32 rows at one
+    // chunk, 64 bytes apart) over all banks.  Wavefront w copies rows 32 w .. 32 w + 31 (tall: two loads) or
+    // 16 w .. 16 w + 15 (wide); 16-row blocks that lie past the expert's last row are not loaded at all
+    // (their products are never stored).
+    constexpr int XROWS = WIDE ? 16 : 32;
+    const int xchunk = ((lane & 3) - (lane >> 4)) & 3;
+    const int64_t xfirst = row0 + wave * XROWS;
+    const int n_xloads = xfirst >= row_end ? 0 : ((!WIDE && xfirst + 16 < row_end) ? 2 : 1);
+    int64_t xr0 = xfirst + (lane >> 2), xr1 = xr0 + 16;
+    if (xr0 > row_end - 1) xr0 = row_end - 1;  // rows past the expert's end duplicate its last row
+    if (xr1 > row_end - 1) xr1 = row_end - 1;
+    const int8_t* xsrc0 = a.x + xr0 * a.K + xchunk * 16;
+    const int8_t* xsrc1 = a.x + xr1 * a.K + xchunk * 16;
+    // operand reads of this lane: token l % 32 of a block, K half l / 32, K step s -> chunk 2 s + l / 32
+    const int r16 = lane & 15;
+    const int frag_off = A_BYTES + (h * 8 + ((lane >> 4) & 1)) * 1024 + r16 * 64;
+    const int frag_s0 = frag_off + (((lane >> 5) + (r16 >> 2)) & 3) * 16;
+    const int frag_s1 = frag_off + ((2 + (lane >> 5) + (r16 >> 2)) & 3) * 16;
+    const int a_off = g * 4096 + lane * 16;
+
+    const int n_iter = a.K / kBK;
+    const int last_it = n_iter - 1;
+    // loads past the last K block are redirected to it (never used), so that the number of loads in flight,
+    // which the hand-written waits rely on, is the same in every step
+    auto load_stage = [&](int it, int st) {
+        const int itc = it < last_it ? it : last_it;
+        int8_t* base = lds + st * STAGE;
+        // weights are read once: non-temporal (cache policy bit 1), so they do not push the tokens out of L2
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int8_t* wp = wsrc[t] + (int64_t)itc * 2048;
+                __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp), MOE355_LPTR(base + wave * 4096 + t * 2048), 16, 0,
+                                                 2);
+                __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp + 1024),
+                                                 MOE355_LPTR(base + wave * 4096 + t * 2048 + 1024), 16, 0, 2);
+            }
+        } else {
+            const int8_t* wp = wsrc[0] + (int64_t)itc * 2048;
+            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp), MOE355_LPTR(base + wave * 2048), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp + 1024), MOE355_LPTR(base + wave * 2048 + 1024), 16, 0, 2);
+        }
+        if (n_xloads >= 1)
+            __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc0 + (int64_t)itc * kBK),
+                                             MOE355_LPTR(base + A_BYTES + wave * (XROWS * 64)), 16, 0, 0);
+        if constexpr (!WIDE) {
+            if (n_xloads >= 2)
+                __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc1 + (int64_t)itc * kBK),
+                                                 MOE355_LPTR(base + A_BYTES + wave * 2048 + 1024), 16, 0, 0);
+        }
+    };
+
+    v16i acc[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[t][b] = (v16i){0};
+
+#pragma unroll
+    for (int r = 0; r + 1 < S; ++r) load_stage(r, r);
+
+    // One K block on LDS stage u.  A stage is complete for this wavefront when at most (loads per step) x
+    // (stages - 2) younger loads are in flight; the barrier then covers the other wavefronts and also says that
+    // everybody is done reading the stage that the next loads overwrite.
+    auto step = [&](int u, int it) {
+        if (n_xloads == 2) wait_vmcnt<(NA + 2) * (S - 2)>();
+        else if (n_xloads == 1) wait_vmcnt<(NA + 1) * (S - 2)>();
+        else wait_vmcnt<NA * (S - 2)>();
+        __builtin_amdgcn_s_barrier();
+        load_stage(it + S - 1, (u + S - 1) % S);
+        if (active) {
+            const int8_t* base = lds + u * STAGE;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const v4i a0 = *(const v4i*)(base + a_off + s * 1024);
+                const v4i a1 = *(const v4i*)(base + a_off + 2048 + s * 1024);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const v4i f = *(const v4i*)(base + (s ? frag_s1 : frag_s0) + b * 2048);
+                    acc[0][b] = mfma_i8(a0, f, acc[0][b]);
+                    acc[1][b] = mfma_i8(a1, f, acc[1][b]);
+                }
+            }
+        }
+    };
+    const int n_full = (n_iter / S) * S;
+    for (int i0 = 0; i0 < n_full; i0 += S) {
+#pragma unroll
+        for (int u = 0; u < S; ++u) step(u, i0 + u);
+    }
+#pragma unroll
+    for (int u = 0; u + 1 < S; ++u)
+        if (n_full + u < n_iter) step(u, n_full + u);
+
+    wait_vmcnt<0>();  // the redirected loads past the end still write LDS
+    __builtin_amdgcn_s_barrier();
+    if (!active) return;
+    tiled_epilogue<EPI, 4>(a, e, acc, hrow0, row_end, nb0, nb1, lds + wave * (PATCHES * 32 * ROWB), lane);
+}
+
+template <int EPI>
+__global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) int8_t wide_lds[];
+    // same XCD-aware walk over (256-row tile, column block of 256 channels) as the 128-row kernel
+    const int total = tm.count[0] * n_col_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int slot = (int)(blockIdx.x / 8);
+    const int item = (int)(blockIdx.x % 8) * per_xcd + slot;
+    if (slot >= per_xcd || item >= total) return;
+    const int mt = item / n_col_blocks;
+    const int nt = item % n_col_blocks;
+    const int e = tm.expert[mt];
+    const int64_t row0 = tm.row_begin[mt];
+    int64_t row_end = tm.row_end[mt];
+    if (row_end > a.R) row_end = a.R;
+    if (row0 >= row_end) return;
+    if (row_end - row0 <= 128) {
+        // a wide tile spans two column blocks: the first half of this tile's workgroups does the work
+        if (nt * 2 >= n_col_blocks) return;
+        stream_tile_body<EPI, true>(a, e, row0, row_end, nt, wide_lds);
+    } else {
+        stream_tile_body<EPI, false>(a, e, row0, row_end, nt, wide_lds);
+    }
 }
 
 // ------------------------------------------------------------------ host side
@@ -382,14 +585,43 @@ static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipE
                            n_col_blocks);
 }
 
+template <int EPI>
+static void launch_wide(const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
+{
+    constexpr int BM = 256;
+    constexpr int lds_bytes = kWideLdsBytes;
+    static const hipError_t attr = hipFuncSetAttribute((const void*)gmm_wide_kernel<EPI>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    (void)attr;
+    const int max_tiles = (int)(a.R / BM + a.E);
+    const size_t arr = (size_t)(((size_t)max_tiles * 4 + 255) / 256) * 256;
+    TileMap tm;
+    tm.count = (int32_t*)workspace;
+    tm.expert = (int32_t*)((char*)workspace + 256);
+    tm.row_begin = (int32_t*)((char*)workspace + 256 + arr);
+    tm.row_end = (int32_t*)((char*)workspace + 256 + 2 * arr);
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm);
+    const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
+    const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
+    const int n_col_blocks = (channels + per_block - 1) / per_block;
+    const int total = max_tiles * n_col_blocks;
+    const int grid = ((total + 7) / 8) * 8;
+    if (ev0 && ev1)
+        hipExtLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, ev0, ev1, 0, a, tm,
+                              max_tiles, n_col_blocks);
+    else
+        hipLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, a, tm, max_tiles,
+                           n_col_blocks);
+}
+
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
                       hipEvent_t ev1)
 {
-#define MOE355_TILED(E_, B_) launch_tiled<E_, B_, ((B_) > 4 ? 4 : 3)>(a, workspace, st, ev0, ev1)
+#define MOE355_TILED(E_, B_) launch_tiled<E_, B_, 3>(a, workspace, st, ev0, ev1)
     if (bm == 256) {
-        if (epi == EPI_I32) MOE355_TILED(EPI_I32, 8);
-        else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 8);
-        else MOE355_TILED(EPI_DEQUANT, 8);
+        if (epi == EPI_I32) launch_wide<EPI_I32>(a, workspace, st, ev0, ev1);
+        else if (epi == EPI_SWIGLU) launch_wide<EPI_SWIGLU>(a, workspace, st, ev0, ev1);
+        else launch_wide<EPI_DEQUANT>(a, workspace, st, ev0, ev1);
     } else if (bm == 128) {
         if (epi == EPI_I32) MOE355_TILED(EPI_I32, 4);
         else if (epi == EPI_SWIGLU) MOE355_TILED(EPI_SWIGLU, 4);
