@@ -8,6 +8,7 @@ from __future__ import annotations
 import torch
 
 from ..quantization.base import AscendMoEScheme
+from ..quantization.checkpoint import moe_weight_loader
 from .contracts import FusedExpertsResult, FusedMoEConfig
 from .moe_comm_method import setup_moe_comm_method
 from .router import AscendFusedTopKRouter
@@ -35,6 +36,8 @@ class AscendRoutedExperts(torch.nn.Module):
         for name, t in specs.items():
             self.register_parameter(name, torch.nn.Parameter(t.to(device), requires_grad=False))
         self.moe_comm_method = setup_moe_comm_method(moe_config)
+        # per-expert checkpoint tensors -> slices of the stacked parameters (quantization/checkpoint.py)
+        self.weight_loader = moe_weight_loader
 
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
         """Copy checkpoint-layout tensors into the registered parameters, then run the scheme's
