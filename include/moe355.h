@@ -64,6 +64,22 @@ int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols,
                          void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Router gate: logits = x.float() @ weight.T (+ bias) in fp32.
+ * Stands in for AscendGateLinear.forward (vllm_ascend/ops/fused_moe/gate_linear.py:55-63) and the
+ * internal-router branch of the layer (vllm_ascend/ops/fused_moe/fused_moe.py:264-271), both of which end in
+ * F.linear on fp32 operands.  Summation order (the reference leaves it to its BLAS): K in chunks of 128, a
+ * fused multiply-add chain over ascending k from +0 inside a chunk, chunk results added in ascending order to
+ * a total that starts at +0, bias last.
+ * x [T, hidden] bf16 or fp32; weight [E, hidden] fp32; bias [E] fp32 or NULL -> logits [T, E] fp32.
+ * hidden must be a multiple of 64.  Few tokens (fewer than 128 output tiles of 32 x 128) run one workgroup
+ * per K chunk and need the workspace (256-byte aligned); otherwise the workspace size is 0 and it may be NULL.
+ */
+size_t moe355_router_gate_workspace(int64_t num_tokens, int hidden, int num_experts);
+int moe355_router_gate(const void *x, int x_dtype, const float *weight, const float *bias, int64_t num_tokens,
+                       int hidden, int num_experts, float *logits, void *workspace, size_t workspace_bytes,
+                       void *stream);
+
+/* ---------------------------------------------------------------------------
  * Group-limited top-k gating.
  * Stands in for aclnnMoeGatingTopK behind torch.ops._C_ascend.moe_gating_top_k
  * (csrc/moe/moe_gating_top_k/moe_gating_top_k_torch_adpt.h:19-71, schema

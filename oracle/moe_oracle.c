@@ -34,6 +34,9 @@
  *   orc_unpermute       : dense torch_moe restatement (test_fused_moe.py:85-97)
  *                         accumulation order: PARITY UNPINNED (torch_npu binary)
  *   orc_dequant_swiglu_quant : numpy rendering of test_dequant_swiglu_quant.py:16-45
+ *   orc_router_gate     : float64 dot products (tolerance), exact integer cases, cases that tell the
+ *                         chunked fma order from a plain ascending sum, from multiply-then-add and from
+ *                         other chunk lengths; the order itself: PARITY UNPINNED (F.linear's BLAS)
  */
 #include <math.h>
 #include <stdint.h>
@@ -630,6 +633,37 @@ ORC_API int orc_w4_rows_to_bf16(const float *f, const float *s1, int64_t rows, i
     for (int64_t r = 0; r < rows; ++r)
         for (int64_t n = 0; n < N; ++n) o[r * N + n] = f32_to_bf16(f[r * N + n] * s1[r]);
     return 0;
+}
+
+/* ------------------------------------------------------------------ router gate
+ * logits = x.float() @ W.T in fp32: AscendGateLinear.forward (vllm_ascend/ops/fused_moe/gate_linear.py:55-63)
+ * and the internal-router branch of the layer (vllm_ascend/ops/fused_moe/fused_moe.py:264-271); both end in
+ * F.linear, whose summation order belongs to the BLAS behind it.  [fixed by build]: K in chunks of 128; inside
+ * a chunk acc = fmaf(x_k, w_k, acc) for ascending k from +0; chunk results are added in ascending order to a
+ * total that starts at +0; the bias, when present, is added last.  fmaf here is the correctly rounded fused
+ * multiply-add of C99 (an explicit call, not a contraction).
+ * x_is_bf16: x holds bf16 bit patterns (uint16), else float. */
+ORC_API void orc_router_gate(const void *x, int x_is_bf16, const float *w, const float *bias, int64_t T, int64_t H,
+                             int64_t E, float *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t) {
+        float *xf = (float *)malloc((size_t)H * sizeof(float));
+        for (int64_t k = 0; k < H; ++k)
+            xf[k] = x_is_bf16 ? bf16_to_f32(((const uint16_t *)x)[t * H + k]) : ((const float *)x)[t * H + k];
+        for (int64_t e = 0; e < E; ++e) {
+            const float *we = w + e * H;
+            float total = 0.0f;
+            for (int64_t k0 = 0; k0 < H; k0 += 128) {
+                const int64_t k1 = k0 + 128 < H ? k0 + 128 : H;
+                float acc = 0.0f;
+                for (int64_t k = k0; k < k1; ++k) acc = fmaf(xf[k], we[k], acc);
+                total = total + acc;
+            }
+            out[t * E + e] = bias ? total + bias[e] : total;
+        }
+        free(xf);
+    }
 }
 
 /* --- small conversion exports used by the Python wrapper ------------------- */

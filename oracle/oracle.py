@@ -139,6 +139,20 @@ def gating_top_k(x, k, *, bias=None, k_group=1, group_count=1, group_select_mode
     return narrow(y), idx, norm
 
 
+def router_gate(x, w, bias=None) -> np.ndarray:
+    """x [T, H] bf16 bit patterns (uint16) or float32, w [E, H] float32 -> logits [T, E] float32."""
+    is_bf16 = x.dtype == np.uint16
+    x = np.ascontiguousarray(x, dtype=np.uint16 if is_bf16 else np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    T, H = x.shape
+    E = w.shape[0]
+    assert w.shape[1] == H
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    out = np.empty((T, E), dtype=np.float32)
+    lib().orc_router_gate(_p(x), ctypes.c_int(int(is_bf16)), _p(w), _p(b), _i64(T), _i64(H), _i64(E), _p(out))
+    return out
+
+
 def dynamic_quant(x_bf16: np.ndarray):
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     rows, cols = x.shape

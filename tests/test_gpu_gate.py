@@ -1,0 +1,140 @@
+"""Router gate kernel against the checker, bit for bit (fp32 logits), both launch forms (one workgroup per K
+chunk for few tokens, one workgroup over all chunks otherwise), ragged token and expert counts, the order-pin
+cases of the CPU suite, and the layer computing its own logits."""
+import numpy as np
+import pytest
+import torch
+
+from _inputs import CONFIGS, bits, make_layer
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def K():
+    from vllm_ascend_amd import kernels
+
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import oracle
+
+    return oracle
+
+
+def _same_bits(a: torch.Tensor, b: np.ndarray):
+    return np.array_equal(a.cpu().numpy().view(np.uint32), b.view(np.uint32))
+
+
+# (T, H, E): decode (split over chunks), ragged everything, tail chunk of 64, more than 128 experts per row of
+# workgroups, enough tiles for the single-pass form, DeepSeek-V3's K
+@pytest.mark.parametrize("T,H,E", [(64, 2048, 128), (5, 192, 40), (1, 64, 8), (33, 320, 288), (4200, 256, 256),
+                                   (4100, 192, 130), (96, 7168, 256)])
+@pytest.mark.parametrize("x_dtype", ["bf16", "f32"])
+def test_router_gate_matches_the_checker(K, orc, T, H, E, x_dtype):
+    print(f"router gate T={T} H={H} E={E} x={x_dtype}", flush=True)
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g)
+    w = torch.randn(E, H, generator=g) * 0.05
+    b = torch.randn(E, generator=g)
+    if x_dtype == "bf16":
+        xb = x.to(torch.bfloat16)
+        x_np = bits(xb)
+        x_dev = xb.to(DEV)
+    else:
+        x_np = x.numpy()
+        x_dev = x.to(DEV)
+    got = K.router_gate(x_dev, w.to(DEV))
+    got_b = K.router_gate(x_dev, w.to(DEV), b.to(DEV))
+    torch.cuda.synchronize()
+    assert got.dtype == torch.float32 and tuple(got.shape) == (T, E)
+    assert _same_bits(got, orc.router_gate(x_np, w.numpy()))
+    assert _same_bits(got_b, orc.router_gate(x_np, w.numpy(), b.numpy()))
+    # and the value: float64 dot products within a few ulps of the magnitude sum
+    want = x_dev.double().cpu().numpy() @ w.double().numpy().T
+    mag = np.abs(x_dev.double().cpu().numpy()) @ np.abs(w.double().numpy()).T
+    assert np.all(np.abs(got.cpu().numpy() - want) <= 1e-6 * mag + 1e-30)
+
+
+def test_router_gate_order_cases_on_the_gpu(K, orc):
+    """The cases that tell the summation order apart, on both launch forms (1 token: split; 4200: single pass)."""
+    big = F(2.0 ** 24)
+    H = 320
+    rows = []
+    for pairs in ({0: big, 128: 1, 129: 1}, {0: big, 64: 1, 65: 1}, {0: 1, 1: 1, 2: big}, {5: 1, 130: 1, 260: big},
+                  {5: big, 130: 1, 260: 1}):
+        r = np.zeros(H, dtype=F)
+        for k, v in pairs.items():
+            r[k] = v
+        rows.append(r)
+    want_col = np.array([big + 2, big, big + 2, big + 2, big], dtype=F)
+    a = F(1.0) + F(2.0 ** -12)
+    fma_row = np.zeros(H, dtype=F)
+    fma_w = np.ones(H, dtype=F)
+    fma_row[0], fma_w[0] = 1.0, -(F(1.0) + F(2.0 ** -11))
+    fma_row[1], fma_w[1] = a, a
+    for T in (5, 4200):
+        x = np.zeros((T, H), dtype=F)
+        x[:5] = np.stack(rows)
+        w = np.ones((32, H), dtype=F)
+        got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV))
+        torch.cuda.synchronize()
+        assert np.array_equal(got[:5, 0].cpu().numpy(), want_col), T
+        assert _same_bits(got, orc.router_gate(x, w))
+        x[0] = fma_row
+        w[3] = fma_w
+        got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV))
+        assert got[0, 3].item() == 2.0 ** -24, T
+        # bias last: (1 + 2^24) + 1
+        x[1] = 0
+        x[1, 0], x[1, 128] = 1, big
+        w[3] = 1
+        got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV), torch.ones(32, device=DEV))
+        assert got[1, 3].item() == float(big), T
+
+
+def test_router_gate_argument_checks(K):
+    w = torch.zeros(8, 64, device=DEV)
+    assert tuple(K.router_gate(torch.zeros(0, 64, device=DEV), w).shape) == (0, 8)
+    assert tuple(K.router_gate(torch.zeros(2, 3, 64, device=DEV, dtype=torch.bfloat16), w).shape) == (2, 3, 8)
+    with pytest.raises(ValueError, match="features"):
+        K.router_gate(torch.zeros(4, 128, device=DEV), w)
+    with pytest.raises(TypeError, match="float32"):
+        K.router_gate(torch.zeros(4, 64, device=DEV), w.to(torch.bfloat16))
+    with pytest.raises(TypeError):
+        K.router_gate(torch.zeros(4, 64, device=DEV, dtype=torch.float16), w)
+    with pytest.raises(RuntimeError, match="GPU"):
+        K.router_gate(torch.zeros(4, 64), w)
+    with pytest.raises(RuntimeError):   # hidden not a multiple of 64
+        K.router_gate(torch.zeros(4, 32, device=DEV), torch.zeros(8, 32, device=DEV))
+
+
+def test_gate_linear_module_and_internal_router(K, orc):
+    from _layer_utils import build_layer
+    from vllm_ascend_amd.fused_moe.gate_linear import AscendGateLinear
+
+    cfg = CONFIGS["c1_tiny"]
+    d = make_layer(cfg, seed=7)
+    g = torch.Generator().manual_seed(11)
+    gate = AscendGateLinear(cfg.H, cfg.E, params_dtype=torch.bfloat16, device=DEV)
+    assert gate.weight.dtype == torch.float32 and gate.bias is None
+    w = torch.randn(cfg.E, cfg.H, generator=g) * 0.05
+    gate.weight_loader(gate.weight, w.to(torch.bfloat16))            # checkpoints may hold the gate in bf16
+    with pytest.raises(ValueError, match="does not fit"):
+        gate.weight_loader(gate.weight, torch.zeros(cfg.E, cfg.H + 1))
+    x = d["x"].to(DEV)
+    logits, second = gate(x)
+    assert second is None and logits.dtype == torch.float32
+    assert _same_bits(logits, orc.router_gate(bits(d["x"]), w.to(torch.bfloat16).float().numpy()))
+    half, _ = gate(x.to(torch.float16))                              # other dtypes are widened on the host side
+    assert _same_bits(half, orc.router_gate(x.to(torch.float16).float().cpu().numpy(),
+                                            w.to(torch.bfloat16).float().numpy()))
+    layer = build_layer(cfg, d)
+    with pytest.raises(ValueError, match="router_logits is required"):
+        layer(x)
+    layer.gate = gate
+    assert torch.equal(layer(x), layer(x, logits))

@@ -16,9 +16,12 @@ from .router import AscendFusedTopKRouter
 
 class AscendRoutedExperts(torch.nn.Module):
     def __init__(self, moe_config: FusedMoEConfig, quant_method: AscendMoEScheme, router: AscendFusedTopKRouter,
-                 params_dtype: torch.dtype = torch.bfloat16, device="cuda", shared_experts=None):
+                 params_dtype: torch.dtype = torch.bfloat16, device="cuda", shared_experts=None, gate=None):
         super().__init__()
         self.shared_experts = shared_experts
+        # the router's own gate (an AscendGateLinear) when the layer computes its logits itself
+        # (is_internal_router, vllm_ascend/ops/fused_moe/fused_moe.py:264-271)
+        self.gate = gate
         self.moe_config = moe_config
         self.quant_method = quant_method
         self.router = router
@@ -54,5 +57,9 @@ class AscendRoutedExperts(torch.nn.Module):
         result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
         return result
 
-    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None) -> torch.Tensor:
+        if router_logits is None:
+            if self.gate is None:
+                raise ValueError("router_logits is required: this layer was built without an internal gate")
+            router_logits, _ = self.gate(hidden_states)
         return self.forward_impl(hidden_states, router_logits).routed_out

@@ -51,6 +51,29 @@ def dynamic_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+def router_gate(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """x [..., H] bf16 / fp32, weight [E, H] fp32 -> fp32 logits [..., E] = x.float() @ weight.T (+ bias)."""
+    x = _dev(x, "x")
+    weight = _dev(weight, "weight")
+    if weight.dtype != torch.float32:
+        raise TypeError(f"weight: the router gate keeps its weight in float32, got {weight.dtype}")
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"x: bfloat16 or float32 tensor expected but got {x.dtype}")
+    E, H = weight.shape
+    if x.shape[-1] != H:
+        raise ValueError(f"x has {x.shape[-1]} features, the gate weight {H}")
+    if bias is not None:
+        bias = _dev(bias, "bias").to(torch.float32)
+    T = x.numel() // H if H else 0
+    lib = _lib.load()
+    out = torch.empty((*x.shape[:-1], E), dtype=torch.float32, device=x.device)
+    nbytes = lib.moe355_router_gate_workspace(T, H, E)
+    ws = _workspace(nbytes, x.device) if nbytes else None
+    check(lib.moe355_router_gate(_ptr(x), _dt(x, "x"), _ptr(weight), _ptr(bias), T, H, E, _ptr(out), _ptr(ws),
+                                 ws.numel() if ws is not None else 0, _stream(x)), "moe355_router_gate")
+    return out
+
+
 def gating_top_k(x, k, k_group, group_count, group_select_mode, renorm, norm_type, out_flag, routed_scaling_factor,
                  eps, bias, alt_dtype=None):
     """-> (y, expert_idx, out[, y_alt]); ``alt_dtype`` asks for a second copy of y cast to that dtype."""
