@@ -51,81 +51,85 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
     // The next stage travels global -> registers under the MFMAs of the current one, then into the other
     // LDS buffer.
     const int half = lane >> 5, l32 = lane & 31;
-    v2f_t xr[4], wr[16];
-    auto load_stage = [&](int stage) {
+    // A stage's 20 loads per lane (4 token rows, 16 expert rows) travel global -> registers -> LDS two stages
+    // ahead of their use.  The MFMAs of one accumulator chain issue 64 cycles apart and block the wavefront
+    // while they wait, so everything else (the loads of stage i + 2, the LDS writes of stage i + 1, the operand
+    // reads eight MFMAs ahead) is placed in the gaps between the MFMAs of stage i, one or two instructions per
+    // gap.
+    v2f_t xr[2][4], wr[2][16];
+    auto load_one = [&](int set, int stage, int j) {
         const int k0 = stage * kGateStage;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        if (j < 4) {
             int64_t t = t0 + wave * 8 + j * 2 + half;
             if (t > T - 1) t = T - 1;  // rows past the end duplicate the last token (never stored)
             if constexpr (X_DT == MOE355_DT_BF16) {
-                // two bf16 values stay packed until the stage is written to LDS: widening them here would
-                // make the wavefront wait for the load before the MFMAs that are meant to cover it
-                xr[j][0] = __uint_as_float(*(const uint32_t*)((const uint16_t*)xv + t * H + k0 + 2 * l32));
+                // two bf16 values stay packed until the stage is written to LDS
+                xr[set][j][0] = __uint_as_float(*(const uint32_t*)((const uint16_t*)xv + t * H + k0 + 2 * l32));
             } else {
-                xr[j] = *(const v2f_t*)((const float*)xv + t * H + k0 + 2 * l32);
+                xr[set][j] = *(const v2f_t*)((const float*)xv + t * H + k0 + 2 * l32);
             }
-        }
-        if (have) {
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                int e = e0 + j * 2 + half;
-                if (e > E - 1) e = E - 1;
-                wr[j] = *(const v2f_t*)(w + (int64_t)e * H + k0 + 2 * l32);
-            }
+        } else {
+            // wavefronts beyond the last expert group (and rows beyond the last expert) repeat the last expert:
+            // the loop stays free of branches, their results are never stored
+            int e = e0 + (j - 4) * 2 + half;
+            if (e > E - 1) e = E - 1;
+            wr[set][j - 4] = *(const v2f_t*)(w + (int64_t)e * H + k0 + 2 * l32);
         }
     };
-    auto store_stage = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v2f_t v = xr[j];
+    auto store_one = [&](int set, int buf, int j) {
+        if (j < 4) {
+            v2f_t v = xr[set][j];
             if constexpr (X_DT == MOE355_DT_BF16) {
-                const uint32_t u = __float_as_uint(xr[j][0]);
+                const uint32_t u = __float_as_uint(xr[set][j][0]);
                 v[0] = __uint_as_float(u << 16);
                 v[1] = __uint_as_float(u & 0xffff0000u);
             }
             *(v2f_t*)&xs[buf][(wave * 8 + j * 2 + half) * kGateStride + 2 * l32] = v;
-        }
-        if (have) {
-#pragma unroll
-            for (int j = 0; j < 16; ++j) *(v2f_t*)&ws[buf][wave][(j * 2 + half) * kGateStride + 2 * l32] = wr[j];
+        } else {
+            *(v2f_t*)&ws[buf][wave][((j - 4) * 2 + half) * kGateStride + 2 * l32] = wr[set][j - 4];
         }
     };
 
     v16f total = {0};
     v16f p = {0};
-    load_stage(s_begin);
-    store_stage(0);
+    const int n_local = s_end - s_begin;
+    const int s_last = s_end - 1;
+    // loads past the last stage are redirected to it and written to the buffer nobody reads any more, so that
+    // every stage issues the same instructions and the compiler's wait counts are exact
+#pragma unroll
+    for (int j = 0; j < 20; ++j) load_one(0, s_begin, j);
+#pragma unroll
+    for (int j = 0; j < 20; ++j) store_one(0, 0, j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 20; ++j) load_one(1, s_begin + 1 < s_last ? s_begin + 1 : s_last, j);
     __syncthreads();
-    for (int s = s_begin; s < s_end; ++s) {
-        const int buf = (s - s_begin) & 1;
-        if (s + 1 < s_end) load_stage(s + 1);
-        if (have) {
-            const float* xa = &xs[buf][l32 * kGateStride + half];
-            const float* wb = &ws[buf][wave][l32 * kGateStride + half];
-            // The MFMAs of one accumulator issue one after the other and block the wavefront while they do: the
-            // operands of the next eight are read from LDS before the current eight are issued.
-            float xo[2][8], wo[2][8];
-            auto read_ops = [&](int set, int batch) {
+
+    // stage with local index i (PAR = i % 2, a compile-time constant after inlining)
+    auto run_stage = [&](int PAR, int i) {
+        const int s = s_begin + i;
+        const int s_load = s + 2 < s_last ? s + 2 : s_last;
+        const float* xa = &xs[PAR][l32 * kGateStride + half];
+        const float* wb = &ws[PAR][wave][l32 * kGateStride + half];
+        float xo[2][8], wo[2][8];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    xo[set][j] = xa[batch * 16 + 2 * j];
-                    wo[set][j] = wb[batch * 16 + 2 * j];
-                }
-            };
-            read_ops(0, 0);
-#pragma unroll
-            for (int b = 0; b < kGateStage / 16; ++b) {
-                if (b + 1 < kGateStage / 16) read_ops((b + 1) & 1, b + 1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    p = __builtin_amdgcn_mfma_f32_32x32x2f32(xo[b & 1][j], wo[b & 1][j], p, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        for (int j = 0; j < 8; ++j) {
+            xo[0][j] = xa[2 * j];
+            wo[0][j] = wb[2 * j];
         }
-        // the other buffer was last read before the previous barrier
-        if (s + 1 < s_end) store_stage(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kGateStage / 2; ++j) {
+            const int b = j >> 3, jj = j & 7;
+            p = __builtin_amdgcn_mfma_f32_32x32x2f32(xo[b & 1][jj], wo[b & 1][jj], p, 0, 0, 0);
+            if (j + 8 < kGateStage / 2) {
+                xo[(b + 1) & 1][jj] = xa[2 * (j + 8)];
+                wo[(b + 1) & 1][jj] = wb[2 * (j + 8)];
+            }
+            if (j < 20) load_one(PAR, s_load, j);
+            if (j >= 10 && j < 30) store_one(PAR ^ 1, PAR ^ 1, j - 10);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         if ((s & 1) || s + 1 == n_stages) {  // the chunk ends with this stage
             if constexpr (!SPLIT) {
 #pragma unroll
@@ -134,7 +138,13 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
             }
         }
         __syncthreads();
+    };
+    int i = 0;
+    for (; i + 2 <= n_local; i += 2) {
+        run_stage(0, i);
+        run_stage(1, i + 1);
     }
+    if (i < n_local) run_stage(0, i);
     if constexpr (SPLIT) total = p;
     if (!have) return;
     // lane l holds expert e0 + l % 32 of tokens 8 (v / 4) + 4 (l / 32) + v % 4
@@ -161,7 +171,16 @@ __global__ __launch_bounds__(256) void router_gate_reduce_kernel(const float* __
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     float total = 0.0f;
-    for (int c = 0; c < n_chunks; ++c) total = total + part[(int64_t)c * n + i];
+    // eight loads in flight at a time; the additions keep the ascending chunk order
+    int c = 0;
+    for (; c + 8 <= n_chunks; c += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = part[(int64_t)(c + j) * n + i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) total = total + v[j];
+    }
+    for (; c < n_chunks; ++c) total = total + part[(int64_t)c * n + i];
     if (bias) total = total + bias[i % E];
     out[i] = total;
 }
