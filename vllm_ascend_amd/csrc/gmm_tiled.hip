@@ -91,9 +91,11 @@ struct TiledLds {
 // written like that every store would touch 64 different cache lines.  The wavefront instead
 // turns one 32-token block at a time through a private LDS patch (token-major, 128 data bytes per
 // token and tile) and stores whole 128-byte row segments: 8 lanes per token row.
-template <int EPI, int BMT>
-__device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&acc)[2][BMT], int64_t row0,
-                                               int64_t row_end, int nb0, int nb1, int8_t* patch, int lane)
+// LIMIT: the SwiGLU clamp is compiled in (as compares and selects it costs 8 of about 50 vector instructions
+// per output, and the epilogue is bound by their number); the caller branches once on the limit.
+template <int EPI, int BMT, bool LIMIT>
+__device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16i (&acc)[2][BMT], int64_t row0,
+                                                    int64_t row_end, int nb0, int nb1, int8_t* patch, int lane)
 {
     constexpr int ROWB = TiledLds<EPI, BMT, 3>::ROWB;
     const int tok = lane & 31;
@@ -148,7 +150,7 @@ __device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&a
                 for (int j = 0; j < 4; ++j) {
                     float gg = ((float)acc[0][b][4 * q + j] * rs) * s0[q][j];
                     float uu = ((float)acc[1][b][4 * q + j] * rs) * s1[q][j];
-                    if (a.limit > 0.0f) {
+                    if constexpr (LIMIT) {
                         gg = gg > a.limit ? a.limit : gg;
                         uu = uu > a.limit ? a.limit : uu;
                         uu = uu < -a.limit ? -a.limit : uu;
@@ -177,6 +179,19 @@ __device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&a
             }
         }
     }
+}
+
+template <int EPI, int BMT>
+__device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&acc)[2][BMT], int64_t row0,
+                                               int64_t row_end, int nb0, int nb1, int8_t* patch, int lane)
+{
+    if constexpr (EPI == EPI_SWIGLU) {
+        if (a.limit > 0.0f) {
+            tiled_epilogue_body<EPI, BMT, true>(a, e, acc, row0, row_end, nb0, nb1, patch, lane);
+            return;
+        }
+    }
+    tiled_epilogue_body<EPI, BMT, false>(a, e, acc, row0, row_end, nb0, nb1, patch, lane);
 }
 
 // One tile of BMT token blocks: rows [row0, row_end) of expert e (at most 32 * BMT of them are computed),

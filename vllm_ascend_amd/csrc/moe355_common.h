@@ -55,7 +55,7 @@ __device__ __forceinline__ uint16_t f32_to_f16(float f)
 // Mul/add only, no contraction.
 __device__ __forceinline__ float m_expf(float x)
 {
-    x = __builtin_fminf(__builtin_fmaxf(x, -87.0f), 88.72283f);
+    x = __builtin_amdgcn_fmed3f(x, -87.0f, 88.72283f);  // min(max(x, -87), 88.72283) in one instruction
     float n = __builtin_rintf(x * 1.44269504088896341f);
     float r = x - n * 0.693359375f;
     r = r - n * -2.12194440e-4f;
