@@ -304,18 +304,28 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
     read_frags(bf0, 0, 0);
 
     // One pipeline step on stage U (compile-time ring position) for K block I.
-#define MOE355_STEP(U, I)                                                          \
-    {                                                                              \
-        store_B(((U) + 1) % RING);          /* B(I+1): registers -> LDS */         \
-        read_frags(bf1, (U), 1);            /* second K step of this stage */      \
-        __builtin_amdgcn_sched_barrier(0);                                         \
-        mma_step(bf0, (U), 0);                                                     \
-        __syncthreads();                    /* B(I+1) visible to all wavefronts */ \
-        load_A((I) + RING - 1, ((U) + RING - 1) % RING);                           \
-        load_B((I) + RING, (U));                                                   \
-        read_frags(bf0, ((U) + 1) % RING, 0);  /* first K step of the next stage */ \
-        __builtin_amdgcn_sched_barrier(0);                                         \
-        mma_step(bf1, (U), 1);                                                     \
+#define MOE355_STEP(U, I)                                                                        \
+    {                                                                                            \
+        /* first K step: its MFMAs go first; the LDS traffic of the second K step and of the */  \
+        /* next stage is issued in the gaps while the matrix pipe is busy                    */  \
+        _Pragma("unroll") for (int b = 0; b < BMT; ++b)                                          \
+        {                                                                                        \
+            acc[0][b] = mfma_i8(Areg[(U)][0][0], bf0[b], acc[0][b]);                             \
+            acc[1][b] = mfma_i8(Areg[(U)][1][0], bf0[b], acc[1][b]);                             \
+            bf1[b] = *(const v4i*)(&Bs[(U)][((BMT + b) * 64 + lane) * 16]);                      \
+            if (b == 0) store_B(((U) + 1) % RING); /* B(I+1): registers -> LDS */                \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
+        __syncthreads(); /* B(I+1) visible to all wavefronts */                                  \
+        _Pragma("unroll") for (int b = 0; b < BMT; ++b)                                          \
+        {                                                                                        \
+            acc[0][b] = mfma_i8(Areg[(U)][0][1], bf1[b], acc[0][b]);                             \
+            acc[1][b] = mfma_i8(Areg[(U)][1][1], bf1[b], acc[1][b]);                             \
+            bf0[b] = *(const v4i*)(&Bs[((U) + 1) % RING][(b * 64 + lane) * 16]);                 \
+            if (b == 0) load_A((I) + RING - 1, ((U) + RING - 1) % RING);                         \
+            if (b == (BMT > 1 ? 1 : 0)) load_B((I) + RING, (U));                                 \
+            __builtin_amdgcn_sched_barrier(0);                                                   \
+        }                                                                                        \
     }
     // whole passes through the ring run without any condition inside (exact wait counts); the remainder is peeled
     const int n_full = (n_iter / RING) * RING;
