@@ -10,7 +10,9 @@
  *     byte count, pass a 256-byte aligned buffer of at least that size;
  *   - return value 0 = enqueued; negative = rejected, nothing was enqueued
  *     (see MOE355_E_*; moe355_strerror() gives the text);
- *   - tensors are dense row-major; "bf16" means raw bfloat16 bits;
+ *   - tensors are dense row-major; "bf16" means raw bfloat16 bits.  Wherever hidden states are bf16 they may
+ *     also be fp16 (MOE355_DT_F16 in the dtype argument), the model dtype of the reference: the same arithmetic
+ *     in fp32, narrowed to fp16 by round-to-nearest-even at the points where the text says bf16;
  *   - `dtype` arguments use MOE355_DT_*.
  *
  * Each entry point names the interface of the reference tree (vllm-ascend,
@@ -58,7 +60,7 @@ const char *moe355_strerror(int code);
  * vllm_ascend/device/device_op.py:192-206 (moe_mlp.py:237-242) and the shared
  * expert (vllm_ascend/ops/fused_moe/shared_experts.py:258).
  *   a = max|row| ; scale = a/127 ; q = clamp(rint(v/scale), -128, 127) ; a == 0 -> q = 0, scale = 0
- * x [rows, cols] bf16 -> q [rows, cols] int8, scale [rows] fp32.
+ * x [rows, cols] bf16 / fp16 -> q [rows, cols] int8, scale [rows] fp32.
  */
 int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q, float *scale,
                          void *stream);
@@ -70,7 +72,7 @@ int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols,
  * F.linear on fp32 operands.  Summation order (the reference leaves it to its BLAS): K in chunks of 128, a
  * fused multiply-add chain over ascending k from +0 inside a chunk, chunk results added in ascending order to
  * a total that starts at +0, bias last.
- * x [T, hidden] bf16 or fp32; weight [E, hidden] fp32; bias [E] fp32 or NULL -> logits [T, E] fp32.
+ * x [T, hidden] bf16, fp16 or fp32; weight [E, hidden] fp32; bias [E] fp32 or NULL -> logits [T, E] fp32.
  * hidden must be a multiple of 64.  Few tokens (fewer than 128 output tiles of 32 x 128) run one workgroup
  * per K chunk and need the workspace (256-byte aligned); otherwise the workspace size is 0 and it may be NULL.
  */
@@ -107,10 +109,10 @@ int moe355_gating_top_k(const void *x, int x_dtype, const void *bias, int64_t ro
  *   expanded_row_idx[t*k+j] = row of pair (t, j) in the expert-sorted array,
  *   the sort being stable in the flat index (vllm_ascend/lora/fused_moe.py:190-204).
  * quant_mode 1: expanded_x is int8 [R, H] and dynamic_scale [R] fp32 is written;
- * quant_mode -1: expanded_x is a bf16 [R, H] copy and dynamic_scale is ignored.
+ * quant_mode -1: expanded_x is a [R, H] copy in x's dtype and dynamic_scale is ignored.
  * expert_tokens [E] int64: per-expert counts (tokens_num_type 1) or their
  * running sum (tokens_num_type 0).
- * x [T, H] bf16, expert_idx [T, k] int32 in [0, E).  Ids outside the range are
+ * x [T, H] bf16 / fp16, expert_idx [T, k] int32 in [0, E).  Ids outside the range are
  * dropped (their expanded_row_idx is -1).  R = T*k must be < 2^31.
  */
 size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, int num_experts);
@@ -201,7 +203,7 @@ int moe355_w4_offset_correction(const uint8_t *weight_nz4, const float *weight_s
  * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,
  * group_type=0, split_item=2) as called from vllm_ascend/device/device_op.py:254-291:
  *   out[row, col] = bf16( (float(acc) * per_token_scale[row]) * scale[e, col] )
- * x [R, K] int8; weight tiled [E, N, K]; scale [E, N] fp32; out [R, N] bf16.
+ * x [R, K] int8; weight tiled [E, N, K]; scale [E, N] fp32; out [R, N] bf16 or fp16 (out_dtype).
  */
 size_t moe355_gmm2_dequant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts);
 int moe355_gmm2_dequant(const int8_t *x, const int8_t *weight_nz, const float *scale, const float *per_token_scale,
@@ -251,8 +253,8 @@ int moe355_dequant_swiglu_quant(const int32_t *x, const float *weight_scale, con
  * vllm_ascend/device/device_op.py:950-954 (token_dispatcher.py:451-461; math
  * csrc/mc2/dispatch_ffn_combine/op_kernel/unpermute/moe_token_unpermute.h:241-372):
  *   out[t, :] = bf16( sum_{j=0..k-1, slot order} float(probs[t, j]) * float(permuted[|idx[t*k+j]|, :]) )
- * permuted [R, H] bf16; sorted_indices [T*k] int32; probs [T, k] bf16 or NULL
- * (NULL = weight 1); residual [T, H] bf16 or NULL is added last in fp32
+ * permuted [R, H] bf16 / fp16 (dtype); sorted_indices [T*k] int32; probs [T, k] in the same dtype or NULL
+ * (NULL = weight 1); residual [T, H] in the same dtype or NULL is added last in fp32
  * (the shared-expert output; the reference adds it in upstream vLLM).
  */
 int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorted_indices, const void *probs,

@@ -143,6 +143,15 @@ ORC_API float orc_expf(float x)
     return ldexpf(y, (int)n);
 }
 
+/* Which 16-bit float the layer's hidden states use: 0 = bf16 (default), 1 = fp16.  The functions that read or
+ * write hidden states (quantiser, gather, down projection, combine, router gate) go through h2f / f2h; the
+ * reference supports both (the model dtype).  Set from the tests through orc_set_half_kind. */
+static int g_half_is_f16 = 0;
+ORC_API void orc_set_half_kind(int is_f16) { g_half_is_f16 = is_f16 != 0; }
+ORC_API int orc_get_half_kind(void) { return g_half_is_f16; }
+static inline float h2f(uint16_t h) { return g_half_is_f16 ? f16_to_f32(h) : bf16_to_f32(h); }
+static inline uint16_t f2h(float f) { return g_half_is_f16 ? f32_to_f16(f) : f32_to_bf16(f); }
+
 /*
  * Sum of n floats in the one order every implementation of this layer uses
  * [fixed by build]: 64 strided partial sums (partial[l] adds v[l], v[l+64], ...
@@ -317,7 +326,7 @@ ORC_API int orc_dynamic_quant_bf16(const uint16_t *x, int64_t rows, int64_t cols
         float *tmp = (float *)malloc(sizeof(float) * (size_t)cols);
 #pragma omp for
         for (int64_t r = 0; r < rows; ++r) {
-            for (int64_t c = 0; c < cols; ++c) tmp[c] = bf16_to_f32(x[r * cols + c]);
+            for (int64_t c = 0; c < cols; ++c) tmp[c] = h2f(x[r * cols + c]);
             quant_row_f32(tmp, cols, q + r * cols, scale + r);
         }
         free(tmp);
@@ -360,7 +369,7 @@ ORC_API int orc_init_routing(const int32_t *ids, int64_t T, int k, int E, const 
         int8_t *qrow = (int8_t *)malloc((size_t)H);
         for (int64_t t = 0; t < T; ++t) {
             float s;
-            for (int64_t c = 0; c < H; ++c) tmp[c] = bf16_to_f32(x[t * H + c]);
+            for (int64_t c = 0; c < H; ++c) tmp[c] = h2f(x[t * H + c]);
             quant_row_f32(tmp, H, qrow, &s);
             for (int j = 0; j < k; ++j) {
                 int64_t d = dst[t * k + j];
@@ -562,7 +571,7 @@ ORC_API int orc_gmm2_dequant(const int32_t *acc, const float *s1, const float *s
             float v = (float)acc[r * N + n];
             v = v * s1[r];
             v = v * s2[(int64_t)e * N + n];
-            o[r * N + n] = f32_to_bf16(v);
+            o[r * N + n] = f2h(v);
         }
     }
     return 0;
@@ -586,11 +595,11 @@ ORC_API int orc_unpermute(const uint16_t *o, const int32_t *dst, const uint16_t 
             for (int j = 0; j < k; ++j) {
                 int64_t d = dst[t * k + j];
                 d = d < 0 ? -d : d;
-                float p = bf16_to_f32(w[t * k + j]) * bf16_to_f32(o[d * H + h]);
+                float p = h2f(w[t * k + j]) * h2f(o[d * H + h]);
                 acc = acc + p;
             }
-            if (add) acc = acc + bf16_to_f32(add[t * H + h]);
-            out[t * H + h] = f32_to_bf16(acc);
+            if (add) acc = acc + h2f(add[t * H + h]);
+            out[t * H + h] = f2h(acc);
         }
     }
     return 0;
@@ -631,7 +640,7 @@ ORC_API int orc_dequant_swiglu_quant(const int32_t *x, const float *w_scale, con
 ORC_API int orc_w4_rows_to_bf16(const float *f, const float *s1, int64_t rows, int64_t N, uint16_t *o)
 {
     for (int64_t r = 0; r < rows; ++r)
-        for (int64_t n = 0; n < N; ++n) o[r * N + n] = f32_to_bf16(f[r * N + n] * s1[r]);
+        for (int64_t n = 0; n < N; ++n) o[r * N + n] = f2h(f[r * N + n] * s1[r]);
     return 0;
 }
 
@@ -650,7 +659,7 @@ ORC_API void orc_router_gate(const void *x, int x_is_bf16, const float *w, const
     for (int64_t t = 0; t < T; ++t) {
         float *xf = (float *)malloc((size_t)H * sizeof(float));
         for (int64_t k = 0; k < H; ++k)
-            xf[k] = x_is_bf16 ? bf16_to_f32(((const uint16_t *)x)[t * H + k]) : ((const float *)x)[t * H + k];
+            xf[k] = x_is_bf16 ? h2f(((const uint16_t *)x)[t * H + k]) : ((const float *)x)[t * H + k];
         for (int64_t e = 0; e < E; ++e) {
             const float *we = w + e * H;
             float total = 0.0f;

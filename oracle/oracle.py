@@ -11,6 +11,7 @@ unless a function says otherwise.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 import subprocess
@@ -77,6 +78,29 @@ def to_torch(a: np.ndarray, dtype=None):
     if dtype in (torch.bfloat16, torch.float16):
         return torch.from_numpy(a.view(np.int16).copy()).view(dtype)
     return torch.from_numpy(a.copy())
+
+
+@contextlib.contextmanager
+def half_kind(kind: str):
+    """Hidden states in ``'bf16'`` (default) or ``'f16'`` while the block runs: the functions whose arguments are
+    called ``*_bf16`` then take and return fp16 bit patterns."""
+    if kind not in ("bf16", "f16"):
+        raise ValueError(kind)
+    before = lib().orc_get_half_kind()
+    lib().orc_set_half_kind(ctypes.c_int(int(kind == "f16")))
+    try:
+        yield
+    finally:
+        lib().orc_set_half_kind(ctypes.c_int(before))
+
+
+def f32_to_half(a: np.ndarray) -> np.ndarray:
+    """fp32 -> the current kind of 16-bit float (see half_kind)."""
+    return f32_to_f16(a) if lib().orc_get_half_kind() else f32_to_bf16(a)
+
+
+def half_to_f32(a: np.ndarray) -> np.ndarray:
+    return f16_to_f32(a) if lib().orc_get_half_kind() else bf16_to_f32(a)
 
 
 def f32_to_bf16(a: np.ndarray) -> np.ndarray:
@@ -374,7 +398,7 @@ def moe_layer(x_bf16, logits_f32, w13, s13, w2, s2, *, top_k, bias=None, k_group
     y, ids, _ = gating_top_k(logits_f32, top_k, bias=bias, k_group=k_group, group_count=group_count,
                              group_select_mode=1, renorm=renorm, norm_type=norm_type,
                              routed_scaling_factor=routed_scaling_factor, x_dtype="f32")
-    w_bf16 = f32_to_bf16(y)
+    w_bf16 = f32_to_half(y)
     add = None
     extra = {}
     if shared is not None:
@@ -390,8 +414,8 @@ def fp32_dequant_reference(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2) -> n
     """Dense fp32 rendering without any activation quantisation (weights * scale in
     fp32), the tolerance reference for the bf16 output.  Restates torch_moe of
     tests/e2e/nightly/single_node/ops/singlecard_ops/test_fused_moe.py:85-97."""
-    x = bf16_to_f32(x_bf16).astype(np.float64)
-    w = bf16_to_f32(topk_w_bf16).astype(np.float64)
+    x = half_to_f32(x_bf16).astype(np.float64)
+    w = half_to_f32(topk_w_bf16).astype(np.float64)
     T, k = topk_ids.shape
     H = x.shape[1]
     I = w2.shape[2]
@@ -418,7 +442,7 @@ def quantized_fp64_reference(tr: LayerTrace, s2) -> np.ndarray:
     cum = np.cumsum(tr.expert_tokens)
     row_expert = np.searchsorted(cum, np.arange(tr.acc2.shape[0]), side="right")
     o = tr.acc2.astype(np.float64) * tr.s1.astype(np.float64)[:, None] * s2.astype(np.float64)[row_expert]
-    w = bf16_to_f32(tr.topk_weights).astype(np.float64)
+    w = half_to_f32(tr.topk_weights).astype(np.float64)
     T, k = w.shape
     dst = tr.expanded_row_idx.reshape(T, k)
     return (o[dst] * w[:, :, None]).sum(axis=1).astype(np.float32)

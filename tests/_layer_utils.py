@@ -57,7 +57,7 @@ def oracle_layer(cfg: LayerCfg, d: dict, keep_acc=True, shared=False):
         # scales travel as [E, N, G] in the checkpoint; the checker takes [E, G, N]
         sg13 = np.ascontiguousarray(d["s13"].numpy().transpose(0, 2, 1))
         sg2 = np.ascontiguousarray(d["s2"].numpy().transpose(0, 2, 1))
-        return orc.w4a8_experts_forward(bits(d["x"]), orc.f32_to_bf16(y), ids, d["w13"].numpy(), sg13,
+        return orc.w4a8_experts_forward(bits(d["x"]), orc.f32_to_half(y), ids, d["w13"].numpy(), sg13,
                                         d["w2"].numpy(), sg2, cfg.w4_group)
     sh = None
     if shared and cfg.shared:

@@ -224,6 +224,6 @@ def test_dense_quant_matmul_argument_checks():
     with pytest.raises(NotImplementedError, match="pertoken_scale"):
         npu_ops.npu_quant_matmul(x, w, s, output_dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError, match="output_dtype"):
-        npu_ops.npu_quant_matmul(x, w, s, pertoken_scale=torch.ones(2), output_dtype=torch.float16)
+        npu_ops.npu_quant_matmul(x, w, s, pertoken_scale=torch.ones(2), output_dtype=torch.float32)
     with pytest.raises(RuntimeError):   # CPU tensors never reach a kernel: there is no host fallback
         npu_ops.npu_quant_matmul(x, w, s, output_dtype=torch.int32)

@@ -106,7 +106,7 @@ def test_router_gate_argument_checks(K):
     with pytest.raises(TypeError, match="float32"):
         K.router_gate(torch.zeros(4, 64, device=DEV), w.to(torch.bfloat16))
     with pytest.raises(TypeError):
-        K.router_gate(torch.zeros(4, 64, device=DEV, dtype=torch.float16), w)
+        K.router_gate(torch.zeros(4, 64, device=DEV, dtype=torch.float64), w)
     with pytest.raises(RuntimeError, match="GPU"):
         K.router_gate(torch.zeros(4, 64), w)
     with pytest.raises(RuntimeError):   # hidden not a multiple of 64

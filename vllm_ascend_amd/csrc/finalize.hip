@@ -7,7 +7,8 @@ namespace moe355 {
 
 // TOPK > 0: the slot loop is unrolled and all TOPK row loads are issued before the first add,
 // so their latencies overlap; TOPK == 0: generic loop.
-template <int TOPK>
+// DT: bf16 or fp16 (rows, weights, residual and result share it).
+template <int TOPK, int DT = MOE355_DT_BF16>
 __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __restrict__ permuted,
                                                               const int32_t* __restrict__ idx,
                                                               const uint16_t* __restrict__ probs, int top_k_rt,
@@ -23,7 +24,7 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
         int32_t d = idx[t * top_k + threadIdx.x];
         d = d < 0 ? -d : d;
         srow[threadIdx.x] = ((int64_t)d < permuted_rows) ? d : -1;
-        sw[threadIdx.x] = probs ? bf16_to_f32(probs[t * top_k + threadIdx.x]) : 1.0f;
+        sw[threadIdx.x] = probs ? half_to_f32<DT>(probs[t * top_k + threadIdx.x]) : 1.0f;
     }
     __syncthreads();
     const int64_t nv = H >> 3;
@@ -44,7 +45,7 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
                 const float w = sw[s];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    float pr = w * bf16_to_f32(v[s][j]);
+                    float pr = w * half_to_f32<DT>(v[s][j]);
                     acc[j] = acc[j] + pr;
                 }
             }
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
                 const v8u16 v = ((const v8u16*)(permuted + (int64_t)d * H))[i];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    float pr = w * bf16_to_f32(v[j]);
+                    float pr = w * half_to_f32<DT>(v[j]);
                     acc[j] = acc[j] + pr;
                 }
             }
@@ -64,11 +65,11 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
         if (residual) {
             const v8u16 r = ((const v8u16*)(residual + t * H))[i];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = acc[j] + bf16_to_f32(r[j]);
+            for (int j = 0; j < 8; ++j) acc[j] = acc[j] + half_to_f32<DT>(r[j]);
         }
         v8u16 o;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = f32_to_bf16(acc[j]);
+        for (int j = 0; j < 8; ++j) o[j] = f32_to_half<DT>(acc[j]);
         ((v8u16*)(out + t * H))[i] = o;
     }
 }
@@ -82,22 +83,29 @@ extern "C" int moe355_token_unpermute(const void* permuted, int dtype, const int
                                       int64_t permuted_rows, const void* residual, void* out, void* stream)
 {
     if (num_tokens < 0 || top_k <= 0 || hidden <= 0 || permuted_rows < 0) return MOE355_E_ARG;
-    if (dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (dtype != MOE355_DT_BF16 && dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (top_k > 64 || hidden % 8 != 0 || num_tokens > 0x7fffffffLL) return MOE355_E_SHAPE;
     if (num_tokens == 0) return MOE355_OK;
     if (!permuted || !sorted_indices || !out) return MOE355_E_ARG;
     if (((uintptr_t)permuted & 15) || ((uintptr_t)out & 15) || ((uintptr_t)residual & 15)) return MOE355_E_SHAPE;
-#define MOE355_UNPERMUTE(K)                                                                                    \
-    hipLaunchKernelGGL(token_unpermute_kernel<K>, dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream, \
-                       (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,       \
+#define MOE355_UNPERMUTE(K, D)                                                                                    \
+    hipLaunchKernelGGL((token_unpermute_kernel<K, D>), dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream, \
+                       (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,             \
                        permuted_rows, (const uint16_t*)residual, (uint16_t*)out)
+    if (dtype == MOE355_DT_F16) {
+        // fp16 models: the common fan-outs unrolled, the rest through the generic loop
+        if (top_k == 8) MOE355_UNPERMUTE(8, MOE355_DT_F16);
+        else if (top_k == 2) MOE355_UNPERMUTE(2, MOE355_DT_F16);
+        else MOE355_UNPERMUTE(0, MOE355_DT_F16);
+        return launch_status();
+    }
     switch (top_k) {
-        case 1: MOE355_UNPERMUTE(1); break;
-        case 2: MOE355_UNPERMUTE(2); break;
-        case 4: MOE355_UNPERMUTE(4); break;
-        case 6: MOE355_UNPERMUTE(6); break;
-        case 8: MOE355_UNPERMUTE(8); break;
-        default: MOE355_UNPERMUTE(0); break;
+        case 1: MOE355_UNPERMUTE(1, MOE355_DT_BF16); break;
+        case 2: MOE355_UNPERMUTE(2, MOE355_DT_BF16); break;
+        case 4: MOE355_UNPERMUTE(4, MOE355_DT_BF16); break;
+        case 6: MOE355_UNPERMUTE(6, MOE355_DT_BF16); break;
+        case 8: MOE355_UNPERMUTE(8, MOE355_DT_BF16); break;
+        default: MOE355_UNPERMUTE(0, MOE355_DT_BF16); break;
     }
 #undef MOE355_UNPERMUTE
     return launch_status();

@@ -26,7 +26,7 @@ constexpr int kGateChunk = 128;
 constexpr int kGateStage = 64;
 constexpr int kGateStride = kGateStage + 2;
 
-// X_DT: MOE355_DT_BF16 or MOE355_DT_F32.  SPLIT: blockIdx.z is the chunk and `out` is the scratch
+// X_DT: MOE355_DT_BF16, MOE355_DT_F16 or MOE355_DT_F32.  SPLIT: blockIdx.z is the chunk and `out` is the scratch
 // [chunks][T][E]; otherwise the workgroup walks all chunks and `out` is logits [T][E] (+ bias).
 template <int X_DT, bool SPLIT>
 __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict__ xv, const float* __restrict__ w,
@@ -62,8 +62,8 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
         if (j < 4) {
             int64_t t = t0 + wave * 8 + j * 2 + half;
             if (t > T - 1) t = T - 1;  // rows past the end duplicate the last token (never stored)
-            if constexpr (X_DT == MOE355_DT_BF16) {
-                // two bf16 values stay packed until the stage is written to LDS
+            if constexpr (X_DT != MOE355_DT_F32) {
+                // two 16-bit values stay packed until the stage is written to LDS
                 xr[set][j][0] = __uint_as_float(*(const uint32_t*)((const uint16_t*)xv + t * H + k0 + 2 * l32));
             } else {
                 xr[set][j] = *(const v2f_t*)((const float*)xv + t * H + k0 + 2 * l32);
@@ -83,6 +83,10 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
                 const uint32_t u = __float_as_uint(xr[set][j][0]);
                 v[0] = __uint_as_float(u << 16);
                 v[1] = __uint_as_float(u & 0xffff0000u);
+            } else if constexpr (X_DT == MOE355_DT_F16) {
+                const uint32_t u = __float_as_uint(xr[set][j][0]);
+                v[0] = f16_to_f32((uint16_t)(u & 0xffffu));
+                v[1] = f16_to_f32((uint16_t)(u >> 16));
             }
             *(v2f_t*)&xs[buf][(wave * 8 + j * 2 + half) * kGateStride + 2 * l32] = v;
         } else {
@@ -211,33 +215,31 @@ extern "C" int moe355_router_gate(const void* x, int x_dtype, const float* weigh
     if (num_tokens < 0 || hidden <= 0 || num_experts <= 0) return MOE355_E_ARG;
     if (num_tokens == 0) return MOE355_OK;
     if (!x || !weight || !logits) return MOE355_E_ARG;
-    if (x_dtype != MOE355_DT_BF16 && x_dtype != MOE355_DT_F32) return MOE355_E_UNSUPPORTED;
+    if (x_dtype != MOE355_DT_BF16 && x_dtype != MOE355_DT_F32 && x_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (hidden % kGateStage != 0) return MOE355_E_SHAPE;
     if (num_tokens > 0x7fffffffLL / 32 * 32) return MOE355_E_SHAPE;
     hipStream_t st = (hipStream_t)stream;
     const int n_chunks = (hidden + kGateChunk - 1) / kGateChunk;
     const bool split = gate_splits(num_tokens, num_experts);
     const dim3 grid((unsigned)((num_tokens + 31) / 32), (unsigned)((num_experts + 127) / 128), split ? n_chunks : 1);
+#define MOE355_GATE(D_, S_, B_, O_)                                                                              \
+    hipLaunchKernelGGL((router_gate_kernel<D_, S_>), grid, dim3(256), 0, st, x, weight, B_, O_, num_tokens, hidden, \
+                       num_experts)
     if (split) {
         const size_t need = moe355_router_gate_workspace(num_tokens, hidden, num_experts);
         if (!workspace || ((uintptr_t)workspace & 255) || workspace_bytes < need) return MOE355_E_WORKSPACE;
         float* part = (float*)workspace;
-        if (x_dtype == MOE355_DT_BF16)
-            hipLaunchKernelGGL((router_gate_kernel<MOE355_DT_BF16, true>), grid, dim3(256), 0, st, x, weight, nullptr,
-                               part, num_tokens, hidden, num_experts);
-        else
-            hipLaunchKernelGGL((router_gate_kernel<MOE355_DT_F32, true>), grid, dim3(256), 0, st, x, weight, nullptr, part,
-                               num_tokens, hidden, num_experts);
+        if (x_dtype == MOE355_DT_BF16) MOE355_GATE(MOE355_DT_BF16, true, nullptr, part);
+        else if (x_dtype == MOE355_DT_F16) MOE355_GATE(MOE355_DT_F16, true, nullptr, part);
+        else MOE355_GATE(MOE355_DT_F32, true, nullptr, part);
         const int64_t n = num_tokens * num_experts;
         hipLaunchKernelGGL(router_gate_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, part, bias,
                            logits, n, num_experts, n_chunks);
     } else {
-        if (x_dtype == MOE355_DT_BF16)
-            hipLaunchKernelGGL((router_gate_kernel<MOE355_DT_BF16, false>), grid, dim3(256), 0, st, x, weight, bias,
-                               logits, num_tokens, hidden, num_experts);
-        else
-            hipLaunchKernelGGL((router_gate_kernel<MOE355_DT_F32, false>), grid, dim3(256), 0, st, x, weight, bias,
-                               logits, num_tokens, hidden, num_experts);
+        if (x_dtype == MOE355_DT_BF16) MOE355_GATE(MOE355_DT_BF16, false, bias, logits);
+        else if (x_dtype == MOE355_DT_F16) MOE355_GATE(MOE355_DT_F16, false, bias, logits);
+        else MOE355_GATE(MOE355_DT_F32, false, bias, logits);
     }
+#undef MOE355_GATE
     return launch_status();
 }

@@ -426,7 +426,7 @@ static int gmm2_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* con
     const void* wany = weight_list ? (const void*)weight_list : (const void*)weight_nz;
     int rc = check_gmm(x, wany, group_list, group_list_type, rows, k, n, num_experts);
     if (rc != MOE355_OK) return rc;
-    if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (out_dtype != MOE355_DT_BF16 && out_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (rows > 0 && (!workspace || ((uintptr_t)workspace & 255) ||
                      workspace_bytes < moe355_gmm2_dequant_workspace(rows, n, k, num_experts)))
         return MOE355_E_WORKSPACE;
@@ -447,6 +447,7 @@ static int gmm2_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* con
     a.ch_scale = scale;
     a.s_list = scale_list;
     a.out = (uint16_t*)out;
+    a.out_f16 = out_dtype == MOE355_DT_F16;
     return launch_gemm_auto<EPI_DEQUANT>(a, workspace, (hipStream_t)stream);
 }
 

@@ -33,7 +33,8 @@ struct GmmArgs {
     // outputs
     int32_t* acc;           // EPI_I32   [R, N]
     float* y;               // EPI_SWIGLU [R, N/2] fp32 SwiGLU values
-    uint16_t* out;          // EPI_DEQUANT [R, N] bf16
+    uint16_t* out;          // EPI_DEQUANT [R, N] bf16, or fp16 when out_f16 is set
+    int out_f16;
 };
 
 // tiled weights / channel scales of expert e
@@ -90,8 +91,9 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
         v4u16 o0, o1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            o0[j] = f32_to_bf16(((float)g[j] * rs) * s0[j]);
-            o1[j] = f32_to_bf16(((float)u[j] * rs) * s1[j]);
+            const float v0 = ((float)g[j] * rs) * s0[j], v1 = ((float)u[j] * rs) * s1[j];
+            o0[j] = a.out_f16 ? f32_to_f16(v0) : f32_to_bf16(v0);
+            o1[j] = a.out_f16 ? f32_to_f16(v1) : f32_to_bf16(v1);
         }
         *(v4u16*)(a.out + row * a.N + n0 + ch) = o0;
         *(v4u16*)(a.out + row * a.N + n1 + ch) = o1;

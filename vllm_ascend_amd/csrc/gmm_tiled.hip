@@ -91,9 +91,10 @@ struct TiledLds {
 // written like that every store would touch 64 different cache lines.  The wavefront instead
 // turns one 32-token block at a time through a private LDS patch (token-major, 128 data bytes per
 // token and tile) and stores whole 128-byte row segments: 8 lanes per token row.
-// LIMIT: the SwiGLU clamp is compiled in (as compares and selects it costs 8 of about 50 vector instructions
-// per output, and the epilogue is bound by their number); the caller branches once on the limit.
-template <int EPI, int BMT, bool LIMIT>
+// FLAG, SwiGLU epilogue: the clamp is compiled in (as compares and selects it costs 8 of about 50 vector
+// instructions per output, and the epilogue is bound by their number); dequant epilogue: the output is fp16
+// instead of bf16.  The caller branches once.
+template <int EPI, int BMT, bool FLAG>
 __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16i (&acc)[2][BMT], int64_t row0,
                                                     int64_t row_end, int nb0, int nb1, int8_t* patch, int lane)
 {
@@ -138,8 +139,8 @@ __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16
                 v4u16 o0, o1;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    o0[j] = f32_to_bf16(((float)acc[0][b][4 * q + j] * rs) * s0[q][j]);
-                    o1[j] = f32_to_bf16(((float)acc[1][b][4 * q + j] * rs) * s1[q][j]);
+                    o0[j] = f32_to_half<FLAG ? MOE355_DT_F16 : MOE355_DT_BF16>(((float)acc[0][b][4 * q + j] * rs) * s0[q][j]);
+                    o1[j] = f32_to_half<FLAG ? MOE355_DT_F16 : MOE355_DT_BF16>(((float)acc[1][b][4 * q + j] * rs) * s1[q][j]);
                 }
                 // both tiles are adjacent in the output row: 64 bf16 = 128 bytes per token
                 *(v4u16*)(patch + tok * ROWB + ch * 2) = o0;
@@ -150,7 +151,7 @@ __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16
                 for (int j = 0; j < 4; ++j) {
                     float gg = ((float)acc[0][b][4 * q + j] * rs) * s0[q][j];
                     float uu = ((float)acc[1][b][4 * q + j] * rs) * s1[q][j];
-                    if constexpr (LIMIT) {
+                    if constexpr (FLAG) {
                         gg = gg > a.limit ? a.limit : gg;
                         uu = uu > a.limit ? a.limit : uu;
                         uu = uu < -a.limit ? -a.limit : uu;
@@ -187,6 +188,12 @@ __device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&a
 {
     if constexpr (EPI == EPI_SWIGLU) {
         if (a.limit > 0.0f) {
+            tiled_epilogue_body<EPI, BMT, true>(a, e, acc, row0, row_end, nb0, nb1, patch, lane);
+            return;
+        }
+    }
+    if constexpr (EPI == EPI_DEQUANT) {
+        if (a.out_f16) {
             tiled_epilogue_body<EPI, BMT, true>(a, e, acc, row0, row_end, nb0, nb1, patch, lane);
             return;
         }

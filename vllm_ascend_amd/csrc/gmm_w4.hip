@@ -116,8 +116,8 @@ __device__ __forceinline__ void epilogue_run_w4(const GmmArgs& a, int64_t row, b
         v4u16 o0, o1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            o0[j] = f32_to_bf16(g[j] * rs);
-            o1[j] = f32_to_bf16(u[j] * rs);
+            o0[j] = a.out_f16 ? f32_to_f16(g[j] * rs) : f32_to_bf16(g[j] * rs);
+            o1[j] = a.out_f16 ? f32_to_f16(u[j] * rs) : f32_to_bf16(u[j] * rs);
         }
         *(v4u16*)(a.out + row * a.N + c0) = o0;
         *(v4u16*)(a.out + row * a.N + c1) = o1;
@@ -512,7 +512,7 @@ extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4
 {
     int rc = check_w4(x, weight_nz4, scale, group_list, group_list_type, rows, k, n, num_experts, group_size);
     if (rc != MOE355_OK) return rc;
-    if (out_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (out_dtype != MOE355_DT_BF16 && out_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (rows == 0) return MOE355_OK;
     if (!per_token_scale || !out) return MOE355_E_ARG;
     if (((uintptr_t)bias & 15) || ((uintptr_t)out & 7)) return MOE355_E_SHAPE;
@@ -526,6 +526,7 @@ extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4
     p.g.E = num_experts;
     p.g.row_scale = per_token_scale;
     p.g.out = (uint16_t*)out;
+    p.g.out_f16 = out_dtype == MOE355_DT_F16;
     p.w4 = weight_nz4;
     p.gscale = scale;
     p.bias = bias;

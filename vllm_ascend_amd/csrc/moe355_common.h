@@ -44,10 +44,29 @@ __device__ __forceinline__ float f16_to_f32(uint16_t h)
 
 __device__ __forceinline__ uint16_t f32_to_f16(float f)
 {
+    // The empty statement pins f as an fp32 value in a register.  Without it the compiler folds a preceding
+    // multiply or add into v_fma_mixlo_f16, which rounds the exact product once, to fp16: on values whose fp32
+    // rounding lands on an fp16 tie that differs from rounding twice (first to fp32, then to fp16), and the
+    // arithmetic here is defined on fp32 intermediates.
+    asm volatile("" : "+v"(f));
     _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
     uint16_t h;
     __builtin_memcpy(&h, &v, 2);
     return h;
+}
+
+// 16-bit float of kind DT (MOE355_DT_BF16 or MOE355_DT_F16) <-> fp32; narrowing rounds to nearest even.
+template <int DT>
+__device__ __forceinline__ float half_to_f32(uint16_t h)
+{
+    if constexpr (DT == MOE355_DT_F16) return f16_to_f32(h);
+    else return bf16_to_f32(h);
+}
+template <int DT>
+__device__ __forceinline__ uint16_t f32_to_half(float f)
+{
+    if constexpr (DT == MOE355_DT_F16) return f32_to_f16(f);
+    else return f32_to_bf16(f);
 }
 
 // exp(x): argument clamped to [-87, 88.72283] (result always normal or +inf; NaN counts as -87),

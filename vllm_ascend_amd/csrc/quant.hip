@@ -21,9 +21,9 @@ __device__ __forceinline__ float block_max_256(float v, float* lds4)
     return m;
 }
 
-// x [rows, cols] bf16 -> q int8, scale fp32.  VEC: cols % 8 == 0 and 16-byte aligned rows.
-template <bool VEC>
-__global__ __launch_bounds__(256) void dynamic_quant_bf16_kernel(const uint16_t* __restrict__ x, int64_t cols,
+// x [rows, cols] bf16 or fp16 (DT) -> q int8, scale fp32.  VEC: cols % 8 == 0 and 16-byte aligned rows.
+template <bool VEC, int DT>
+__global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __restrict__ x, int64_t cols,
                                                                  int8_t* __restrict__ q, float* __restrict__ scale)
 {
     __shared__ float lds4[4];
@@ -38,13 +38,13 @@ __global__ __launch_bounds__(256) void dynamic_quant_bf16_kernel(const uint16_t*
             v8u16 v = xv[i];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                float f = __builtin_fabsf(bf16_to_f32(v[j]));
+                float f = __builtin_fabsf(half_to_f32<DT>(v[j]));
                 a = f > a ? f : a;
             }
         }
     } else {
         for (int64_t i = threadIdx.x; i < cols; i += 256) {
-            float f = __builtin_fabsf(bf16_to_f32(xr[i]));
+            float f = __builtin_fabsf(half_to_f32<DT>(xr[i]));
             a = f > a ? f : a;
         }
     }
@@ -60,14 +60,14 @@ __global__ __launch_bounds__(256) void dynamic_quant_bf16_kernel(const uint16_t*
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(v[j]) / s);
+                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(v[j]) / s);
                 w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
             }
             qv[i] = make_uint2(w[0], w[1]);
         }
     } else {
         for (int64_t i = threadIdx.x; i < cols; i += 256)
-            qr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(xr[i]) / s);
+            qr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(xr[i]) / s);
     }
 }
 
@@ -125,16 +125,21 @@ extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, in
     if (rows < 0 || cols <= 0) return MOE355_E_ARG;
     if (rows == 0) return MOE355_OK;
     if (!x || !q || !scale) return MOE355_E_ARG;
-    if (x_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (x_dtype != MOE355_DT_BF16 && x_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
     hipStream_t st = (hipStream_t)stream;
     const bool vec = (cols % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)q & 7) == 0);
-    if (vec)
-        hipLaunchKernelGGL(dynamic_quant_bf16_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st,
-                           (const uint16_t*)x, cols, q, scale);
-    else
-        hipLaunchKernelGGL(dynamic_quant_bf16_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st,
-                           (const uint16_t*)x, cols, q, scale);
+#define MOE355_DQ(V_, D_)                                                                                      \
+    hipLaunchKernelGGL((dynamic_quant_kernel<V_, D_>), dim3((unsigned)rows), dim3(256), 0, st, (const uint16_t*)x, \
+                       cols, q, scale)
+    if (x_dtype == MOE355_DT_BF16) {
+        if (vec) MOE355_DQ(true, MOE355_DT_BF16);
+        else MOE355_DQ(false, MOE355_DT_BF16);
+    } else {
+        if (vec) MOE355_DQ(true, MOE355_DT_F16);
+        else MOE355_DQ(false, MOE355_DT_F16);
+    }
+#undef MOE355_DQ
     return launch_status();
 }
 

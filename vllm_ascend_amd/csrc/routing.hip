@@ -248,8 +248,9 @@ __global__ __launch_bounds__(256) void route_small_kernel(const int32_t* __restr
     }
 }
 
-// One workgroup per token: quantise the row once, write it to its k destinations.
-template <bool QUANT>
+// One workgroup per token: quantise the row once, write it to its k destinations.  DT: bf16 or fp16 rows
+// (the copy without quantisation moves 16-bit patterns and does not care).
+template <bool QUANT, int DT = MOE355_DT_BF16>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
                                                           const int32_t* __restrict__ dst, void* __restrict__ xs,
                                                           float* __restrict__ sx)
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
             v8u16 v = xv[i];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                float f = __builtin_fabsf(bf16_to_f32(v[j]));
+                float f = __builtin_fabsf(half_to_f32<DT>(v[j]));
                 a = f > a ? f : a;
             }
         }
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(bf16_to_f32(v[j]) / s);
+                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(v[j]) / s);
                 w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
             }
             const uint2 pk = make_uint2(w[0], w[1]);
@@ -326,7 +327,7 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     if (num_tokens < 0 || hidden <= 0 || top_k <= 0 || num_experts <= 0) return MOE355_E_ARG;
     if (quant_mode != 1 && quant_mode != -1) return MOE355_E_UNSUPPORTED;
     if (tokens_num_type != 0 && tokens_num_type != 1) return MOE355_E_UNSUPPORTED;
-    if (x_dtype != MOE355_DT_BF16) return MOE355_E_UNSUPPORTED;
+    if (x_dtype != MOE355_DT_BF16 && x_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (top_k > 64 || num_experts > 2048) return MOE355_E_SHAPE;
     const int64_t R = num_tokens * top_k;
     if (R >= 0x7fffffffLL) return MOE355_E_SHAPE;
@@ -359,7 +360,10 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
                            ws.chunk_hist, ws.off, expanded_row_idx);
     }
     if (R > 0) {
-        if (quant_mode == 1)
+        if (quant_mode == 1 && x_dtype == MOE355_DT_F16)
+            hipLaunchKernelGGL((gather_rows_kernel<true, MOE355_DT_F16>), dim3((unsigned)num_tokens), dim3(256), 0, st,
+                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+        else if (quant_mode == 1)
             hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, st,
                                (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
         else

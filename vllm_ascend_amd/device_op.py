@@ -89,8 +89,9 @@ class MI355XDeviceAdaptor:
             first = weight_scale[0] if isinstance(weight_scale, list) else weight_scale
             fallback_output_dtype = first.dtype
         if fallback_output_dtype == torch.float32:
-            # fp32 channel scales (the configured shapes): the product is still written as bf16
-            fallback_output_dtype = torch.bfloat16
+            # fp32 channel scales (the kernels take them in fp32): the product is written in the dtype of the
+            # layer's hidden states
+            fallback_output_dtype = input_dtype if input_dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
         return npu_ops.npu_grouped_matmul(
             x=[hidden_states], weight=weight, scale=weight_scale, bias=bias, per_token_scale=[per_token_scale],
             split_item=2, group_list_type=group_list_type, group_type=0, group_list=group_list,

@@ -150,6 +150,9 @@ class MoEMlpComputeInput:
     expanded_row_idx: torch.Tensor | None = None
     topk_ids: torch.Tensor | None = None
     lora_context: Any = None
+    # dtype of the layer's hidden states (the dispatcher may already have quantised them to int8): what the down
+    # projection writes.  Not in the reference, which takes it from the dtype of the w2 scale.
+    output_dtype: torch.dtype | None = None
 
 
 @dataclass
@@ -226,4 +229,5 @@ def build_mlp_compute_input(*, fused_experts_input: MoEFusedExpertsInput,
         expanded_row_idx=getattr(d.combine_metadata, "expanded_row_idx", None),
         topk_ids=f.topk_ids,
         lora_context=f.lora_context,
+        output_dtype=f.hidden_states.dtype if f.hidden_states.dtype in (torch.bfloat16, torch.float16) else None,
     )

@@ -36,7 +36,7 @@ class AscendGateLinear(torch.nn.Module):
         param.data.copy_(loaded_weight.to(torch.float32))
 
     def forward(self, x: torch.Tensor):
-        if x.dtype not in (torch.float32, torch.bfloat16):
-            x = x.to(torch.float32)  # bf16 is widened inside the kernel (exact); anything else here
+        if x.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            x = x.to(torch.float32)  # bf16 and fp16 are widened inside the kernel (exact); anything else here
         logits = kernels.router_gate(x, self.weight.data, None if self.bias is None else self.bias.data)
         return logits, None

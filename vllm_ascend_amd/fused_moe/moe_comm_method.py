@@ -54,7 +54,7 @@ class AllGatherCommImpl:
 
     def fused_experts(self, fused_experts_input: MoEFusedExpertsInput) -> FusedExpertsResult:
         f = fused_experts_input
-        assert f.hidden_states.dtype in (torch.bfloat16, torch.int8), (
+        assert f.hidden_states.dtype in (torch.bfloat16, torch.float16, torch.int8), (
             f"Unsupported hidden_states dtype: {f.hidden_states.dtype}")
         assert _EXTRA_CTX.moe_comm_method is not None, "Missing communication context"
         stream = torch.cuda.current_stream() if f.hidden_states.is_cuda else None

@@ -48,7 +48,7 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
                     dynamic_scale=None, w1_scale_bias=None, w2_scale_bias=None, w1_offset=None, w2_offset=None,
                     fusion: bool = False, dynamic_eplb: bool = False, activation=None, swiglu_limit: float = 0.0,
                     swiglu_alpha: float = 1.0, swiglu_beta: float = 0.0,
-                    use_w4a8_per_channel_gmm_swiglu: bool = False, **unsupported):
+                    use_w4a8_per_channel_gmm_swiglu: bool = False, output_dtype=None, **unsupported):
     act_name = getattr(activation, "value", activation) or "silu"
     if act_name != "silu":
         raise NotImplementedError(f"activation {act_name!r}: only 'silu' (SwiGLU) has a fused MI355X kernel")
@@ -60,7 +60,7 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
         raise NotImplementedError("MXFP quantisation is not supported on this path")
     if w1_scale_bias is not None or use_w4a8_per_channel_gmm_swiglu:
         raise NotImplementedError("W4A8 weights go through the W4A8 scheme's own MLP")
-    input_dtype = hidden_states.dtype
+    input_dtype = hidden_states.dtype if hidden_states.dtype != torch.int8 else (output_dtype or torch.bfloat16)
 
     if dynamic_scale is None:
         hidden_states, pertoken_scale = DeviceOperator.npu_dynamic_quant(hidden_states=hidden_states)
@@ -76,7 +76,7 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
         out = DeviceOperator.npu_grouped_matmul_gmm2(
             hidden_states=hidden_states, weight=list(w2), weight_scale=list(w2_scale),
             per_token_scale=swiglu_out_scale, group_list=group_list, group_list_type=group_list_type,
-            input_dtype=input_dtype if input_dtype != torch.int8 else torch.bfloat16)
+            input_dtype=input_dtype)
         return out, before_gmm2_evt
     # gmm1: gate_up_proj + dequant + SwiGLU + dynamic re-quant in one op
     hidden_states, swiglu_out_scale, _ = DeviceOperator.npu_grouped_matmul_swiglu_quant(
@@ -89,7 +89,7 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
     out = DeviceOperator.npu_grouped_matmul_gmm2(
         hidden_states=hidden_states, weight=_single(w2, "w2"), weight_scale=_single(w2_scale, "w2_scale"), per_token_scale=swiglu_out_scale,
         group_list=group_list, group_list_type=group_list_type,
-        input_dtype=input_dtype if input_dtype != torch.int8 else torch.bfloat16)
+        input_dtype=input_dtype)
     return out, before_gmm2_evt
 
 
@@ -108,4 +108,4 @@ def unified_apply_mlp(*, mlp_compute_input: MoEMlpComputeInput):
         w1_scale_bias=w.w1_scale_bias, w2_scale_bias=w.w2_scale_bias, w1_offset=w.w1_offset, w2_offset=w.w2_offset,
         fusion=m.fusion, dynamic_eplb=m.dynamic_eplb, activation=m.activation, swiglu_limit=m.swiglu_limit,
         swiglu_alpha=m.swiglu_alpha, swiglu_beta=m.swiglu_beta,
-        use_w4a8_per_channel_gmm_swiglu=m.quant.use_w4a8_per_channel_gmm_swiglu)
+        use_w4a8_per_channel_gmm_swiglu=m.quant.use_w4a8_per_channel_gmm_swiglu, output_dtype=m.output_dtype)

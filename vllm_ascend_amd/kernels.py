@@ -33,13 +33,19 @@ def _dt(t: torch.Tensor, name: str) -> int:
         raise TypeError(f"{name}: float16, float32 or bfloat16 tensor expected but got {t.dtype}") from None
 
 
+def _half_dtype(dtype) -> torch.dtype:
+    if dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"output dtype must be bfloat16 or float16, got {dtype}")
+    return dtype
+
+
 def _workspace(nbytes: int, device) -> torch.Tensor:
     # torch's caching allocator hands out 512-byte aligned blocks
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
 def dynamic_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """bf16 [..., H] -> (int8 [..., H], fp32 [...]) per-row absmax/127 quantisation."""
+    """bf16 / fp16 [..., H] -> (int8 [..., H], fp32 [...]) per-row absmax/127 quantisation."""
     x = _dev(x, "x")
     lib = _lib.load()
     cols = x.shape[-1]
@@ -52,13 +58,13 @@ def dynamic_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 
 
 def router_gate(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
-    """x [..., H] bf16 / fp32, weight [E, H] fp32 -> fp32 logits [..., E] = x.float() @ weight.T (+ bias)."""
+    """x [..., H] bf16 / fp16 / fp32, weight [E, H] fp32 -> fp32 logits [..., E] = x.float() @ weight.T (+ bias)."""
     x = _dev(x, "x")
     weight = _dev(weight, "weight")
     if weight.dtype != torch.float32:
         raise TypeError(f"weight: the router gate keeps its weight in float32, got {weight.dtype}")
-    if x.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError(f"x: bfloat16 or float32 tensor expected but got {x.dtype}")
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"x: float16, float32 or bfloat16 tensor expected but got {x.dtype}")
     E, H = weight.shape
     if x.shape[-1] != H:
         raise ValueError(f"x has {x.shape[-1]} features, the gate weight {H}")
@@ -171,7 +177,7 @@ def gmm2_dequant(x, weight_nz, scale, per_token_scale, group_list, group_list_ty
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz.shape[0]
-    out = torch.empty((rows, n), dtype=out_dtype, device=x.device)
+    out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm2_dequant(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_dev(scale, "scale")),
                                   _ptr(_dev(per_token_scale, "per_token_scale")), _ptr(_gl(group_list)),
@@ -263,16 +269,17 @@ def gmm1_swiglu_quant_w4(x, weight_nz4, weight_scale, group_size, x_scale, group
     return out, out_scale
 
 
-def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_list, group_list_type, n, k, bias=None):
+def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_list, group_list_type, n, k, bias=None,
+                    out_dtype=torch.bfloat16):
     x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz4.shape[0]
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
+    out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     check(lib.moe355_gmm2_dequant_w4(_ptr(x), _ptr(_dev(weight_nz4, "weight")), _ptr(_dev(scale, "scale")),
                                      group_size, _ptr(bias), _ptr(_dev(per_token_scale, "per_token_scale")),
                                      _ptr(_gl(group_list)), _gl_type(group_list_type), rows, k, n, E, _ptr(out),
-                                     DT_BF16, _stream(x)), "moe355_gmm2_dequant_w4")
+                                     _DT[out.dtype], _stream(x)), "moe355_gmm2_dequant_w4")
     return out
 
 
@@ -317,18 +324,19 @@ def gmm1_swiglu_quant_list(x, weight_list, scale_list, x_scale, group_list, grou
     return out, out_scale
 
 
-def gmm2_dequant_list(x, weight_list, scale_list, per_token_scale, group_list, group_list_type):
+def gmm2_dequant_list(x, weight_list, scale_list, per_token_scale, group_list, group_list_type,
+                      out_dtype=torch.bfloat16):
     x = _dev(x, "x")
     lib = _lib.load()
     _check_list(weight_list, "weight", torch.int8)
     _check_list(scale_list, "scale", torch.float32)
     k, n = weight_list[0].shape
     rows, E = x.shape[0], len(weight_list)
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
+    out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm2_dequant_list(_ptr(x), _ptr(_ptr_table(weight_list)), _ptr(_ptr_table(scale_list)),
                                        _ptr(_dev(per_token_scale, "per_token_scale")), _ptr(_gl(group_list)),
-                                       _gl_type(group_list_type), rows, k, n, E, _ptr(out), DT_BF16, _ptr(ws),
+                                       _gl_type(group_list_type), rows, k, n, E, _ptr(out), _DT[out.dtype], _ptr(ws),
                                        ws.numel(), _stream(x)), "moe355_gmm2_dequant_list")
     return out
 

@@ -78,19 +78,22 @@ def npu_grouped_matmul(x, weight, *, bias=None, scale=None, offset=None, antiqua
     ps = per_token_scale if isinstance(per_token_scale, (list, tuple)) else [per_token_scale]
     if len(xs) == 1 and len(ps) == 1 and len(ws) > 1 and len(ws) == len(ss):
         # one tiled [K, N] weight and one [N] scale per expert
-        if output_dtype not in (None, torch.bfloat16):
+        if output_dtype not in (None, torch.bfloat16, torch.float16):
             raise NotImplementedError(f"npu_grouped_matmul: output_dtype {output_dtype} is not supported")
         scales = [s_ if s_.dtype == torch.float32 else s_.to(torch.float32) for s_ in ss]
-        return [kernels.gmm2_dequant_list(xs[0], list(ws), scales, ps[0], group_list, group_list_type)]
+        return [kernels.gmm2_dequant_list(xs[0], list(ws), scales, ps[0], group_list, group_list_type,
+                                          output_dtype or torch.bfloat16)]
     if len(xs) != 1 or len(ws) != 1 or len(ss) != 1 or len(ps) != 1 or ss[0] is None or ps[0] is None:
         raise NotImplementedError("npu_grouped_matmul: expects exactly one x, weight, scale and per_token_scale")
     a, w, s, p = xs[0], ws[0], ss[0], ps[0]
     if a.dtype != torch.int8 or w.dtype != torch.int8:
         raise NotImplementedError("npu_grouped_matmul: only the int8 x int8 form is supported")
-    if output_dtype not in (None, torch.bfloat16):
-        raise NotImplementedError(f"npu_grouped_matmul: output_dtype {output_dtype} is not supported (bfloat16 only)")
+    if output_dtype not in (None, torch.bfloat16, torch.float16):
+        raise NotImplementedError(
+            f"npu_grouped_matmul: output_dtype {output_dtype} is not supported (bfloat16 or float16)")
     k, n = w.shape[1], w.shape[2]
-    out = kernels.gmm2_dequant(a, w, s.to(torch.float32), p, group_list, group_list_type, n, k)
+    out = kernels.gmm2_dequant(a, w, s.to(torch.float32), p, group_list, group_list_type, n, k,
+                               output_dtype or torch.bfloat16)
     return [out]
 
 
@@ -119,7 +122,7 @@ def npu_quant_matmul(x1, x2, scale, *, offset=None, pertoken_scale=None, bias=No
     (``vllm_ascend/ops/fused_moe/shared_experts.py:262-301``): ``x1`` int8 ``[M, K]``, ``x2`` int8
     ``[K, N]`` in the tiled storage of :func:`npu_format_cast`, ``scale`` ``[N]``.
     ``output_dtype=torch.int32``: the raw accumulators (scales ignored, as in the reference call);
-    ``output_dtype=torch.bfloat16``: ``bf16((acc * pertoken_scale[m]) * scale[n])``.
+    ``output_dtype=torch.bfloat16`` / ``torch.float16``: ``half((acc * pertoken_scale[m]) * scale[n])``.
     One expert that owns every row: the grouped kernels with E = 1."""
     if offset is not None or bias is not None:
         raise NotImplementedError("npu_quant_matmul: offset / bias are not supported")
@@ -132,10 +135,11 @@ def npu_quant_matmul(x1, x2, scale, *, offset=None, pertoken_scale=None, bias=No
     w = x2.unsqueeze(0)
     if output_dtype == torch.int32:
         out = kernels.gmm_i32(a, w, gl, 0, n, k)
-    elif output_dtype in (None, torch.bfloat16):
+    elif output_dtype in (None, torch.bfloat16, torch.float16):
         if pertoken_scale is None:
-            raise NotImplementedError("npu_quant_matmul: bf16 output needs pertoken_scale")
-        out = kernels.gmm2_dequant(a, w, scale.to(torch.float32).reshape(1, n), pertoken_scale.reshape(-1), gl, 0, n, k)
+            raise NotImplementedError("npu_quant_matmul: bf16 / fp16 output needs pertoken_scale")
+        out = kernels.gmm2_dequant(a, w, scale.to(torch.float32).reshape(1, n), pertoken_scale.reshape(-1), gl, 0, n, k,
+                                   output_dtype or torch.bfloat16)
     else:
         raise NotImplementedError(f"npu_quant_matmul: output_dtype {output_dtype} is not supported")
     return out.reshape(lead + (n,))

@@ -132,5 +132,6 @@ def w4a8_apply_mlp(m: MoEMlpComputeInput):
     q1, q1_scale = kernels.gmm1_swiglu_quant_w4(x, w1, s1, g1, m.dynamic_scale, m.group_list, m.group_list_type, n1, k1,
                                                 swiglu_limit=m.swiglu_limit)
     evt = torch.cuda.current_stream().record_event() if x.is_cuda else None
-    out = kernels.gmm2_dequant_w4(q1, w2, s2, g2, q1_scale, m.group_list, m.group_list_type, n2, k2)
+    out = kernels.gmm2_dequant_w4(q1, w2, s2, g2, q1_scale, m.group_list, m.group_list_type, n2, k2,
+                                  out_dtype=m.output_dtype or torch.bfloat16)
     return out, evt
