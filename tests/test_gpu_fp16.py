@@ -104,9 +104,7 @@ def test_fp16_stages_match_the_checker(K, orc):
 def test_fp16_layer_matches_the_checker(orc, name):
     from _layer_utils import build_layer, oracle_layer
 
-    if name == "c2_small":
-        cfg = dataclasses.replace(CONFIGS["c2_qwen3_decode"], name=name, T=48, E=32, k=4)
-    elif name == "w4a8_small":
+    if name == "w4a8_small":
         cfg = dataclasses.replace(CONFIGS["c5_w4a8_zipf"], name=name, T=48, E=8, H=512, I=256, n_group=1, topk_group=1)
     else:
         cfg = CONFIGS[name]
@@ -174,3 +172,25 @@ def test_fp16_output_rounds_the_fp32_product_not_the_exact_one(K, orc):
                          torch.from_numpy(cum).to(DEV), 0, N, Kd, out_dtype=torch.float16)
     torch.cuda.synchronize()
     assert np.array_equal(bits(got.cpu()), want)
+
+
+@pytest.mark.parametrize("variant", ["shared", "shared_overlap", "weight_lists"])
+def test_fp16_layer_with_shared_expert_and_weight_lists(orc, variant):
+    from _layer_utils import build_layer, oracle_layer
+
+    shared = variant.startswith("shared")
+    cfg = CONFIGS["c4_small"] if shared else CONFIGS["c2_small"]
+    print(f"fp16 layer variant {variant}", flush=True)
+    d = make_layer(cfg, seed=2)
+    d["x"] = d["x"].to(torch.float16)
+    layer = build_layer(cfg, d, DEV, shared=shared, overlap=variant == "shared_overlap",
+                        dynamic_eplb=variant == "weight_lists")
+    layer.quant_method.in_dtype = torch.float16
+    res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
+    torch.cuda.synchronize()
+    with orc.half_kind("f16"):
+        tr = oracle_layer(cfg, d, shared=shared)
+    assert res.routed_out.dtype == torch.float16
+    if shared:
+        assert np.array_equal(bits(res.shared_out), tr.extra["shared_out"])
+    assert np.array_equal(bits(res.routed_out), tr.out)
