@@ -114,7 +114,7 @@ def _rand_groups(g, E, R, empty_some=True):
 
 
 # (rows, experts, K, N).  rows/experts picks the kernel: < 48 weight streaming, >= 48 LDS-tiled with
-# 128-row tiles, >= 192 with 256-row tiles; K % 64 != 0 always streams.
+# 128-row tiles, 48..256 with K >= 4096 the 256-row weight-streaming tiles; K % 64 != 0 always streams.
 GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100, 16, 768, 2048),
              (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256), (3000, 4, 768, 2048),
              (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096)]
@@ -466,3 +466,52 @@ def test_grouped_gemms_with_one_expert_owning_every_row(K, orc):
         torch.cuda.synchronize()
         assert np.array_equal(q.cpu().numpy(), q_want)
         assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
+# Seeded random problems around the borders of the kernel choice (average rows per expert 47 / 48 / 256 / 257,
+# K 4032 / 4096) with skewed group sizes: all three epilogues of whichever kernel the library picks.
+def _random_gemm_problem(seed):
+    rng = np.random.default_rng(seed)
+    E = int(rng.integers(1, 13))
+    avg = int(rng.choice([3, 30, 47, 48, 49, 100, 200, 256, 257, 400]))
+    Kd = int(rng.choice([64, 192, 512, 4032, 4096, 4160]))
+    N = int(rng.choice([64, 128, 320, 576]))
+    R = max(1, E * avg + int(rng.integers(0, E)))
+    w = rng.random(E) ** 3                      # a few experts take most rows
+    if E > 2:
+        w[rng.permutation(E)[: E // 3]] = 0
+    if w.sum() == 0:
+        w[0] = 1
+    cnt = np.floor(w / w.sum() * R).astype(np.int64)
+    cnt[int(np.argmax(w))] += R - cnt.sum()
+    return E, R, Kd, N, cnt
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_grouped_gemms_on_random_problems(K, orc, seed):
+    from vllm_ascend_amd._lib import W_ENK
+
+    E, R, Kd, N, cnt = _random_gemm_problem(seed)
+    print(f"random gemm seed={seed} E={E} R={R} K={Kd} N={N} counts={cnt.tolist()}", flush=True)
+    g = torch.Generator().manual_seed(1000 + seed)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    cnt_t = torch.from_numpy(cnt)
+    cum = torch.cumsum(cnt_t, 0)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    acc = K.gmm_i32(x.to(DEV), wnz, cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    want = orc.gmm2_dequant(ref, sx.numpy(), sw.numpy(), cum.numpy())
+    got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt_t.to(DEV), 1, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got.cpu()), want)
+    limit = 0.0 if seed % 3 else 1.5
+    q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw.numpy(), cum.numpy()), swiglu_limit=limit)
+    q, s_ = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd, swiglu_limit=limit)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
