@@ -174,3 +174,41 @@ def test_empty_and_single_token_batches(name):
     torch.cuda.synchronize()
     tr = oracle_layer(dataclasses.replace(cfg, T=1), d1, shared=cfg.shared)
     assert np.array_equal(bits(res.routed_out), tr.out)
+
+
+def _random_layer_cfg(seed):
+    """A random but valid layer: softmax or sigmoid, with or without expert groups / bias / shared expert /
+    Zipf-skewed routing / int4 weights, sizes small enough for the CPU checker."""
+    from _inputs import LayerCfg
+
+    rng = np.random.default_rng(seed)
+    n_group = int(rng.choice([1, 1, 2, 4]))
+    per_group = int(rng.choice([2, 4, 8]))
+    E = n_group * per_group
+    topk_group = int(rng.integers(1, n_group + 1))
+    k = int(rng.integers(1, min(8, topk_group * per_group) + 1))
+    w4 = seed % 4 == 3
+    H = int(rng.choice([256, 512])) if w4 else int(rng.choice([128, 192, 320, 512]))
+    I = int(rng.choice([128, 256])) if w4 else int(rng.choice([32, 96, 160, 256]))
+    return LayerCfg(
+        f"random_{seed}", T=int(rng.choice([1, 7, 33, 130, 600])), H=H, E=E, k=k, I=I,
+        scoring=str(rng.choice(["softmax", "sigmoid"])), n_group=n_group, topk_group=topk_group,
+        renorm=int(rng.integers(0, 2)), routed_scaling_factor=float(rng.choice([1.0, 2.5])),
+        bias=bool(rng.integers(0, 2)), shared=bool(rng.integers(0, 2)) and not w4,
+        w4_group=int(rng.choice([0, 128])) if w4 else -1, zipf=float(rng.choice([0.0, 1.1])))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_layer_on_random_configurations(seed):
+    cfg = _random_layer_cfg(seed)
+    print(f"random layer {cfg}", flush=True)
+    d = make_layer(cfg, seed=100 + seed)
+    layer = build_layer(cfg, d, DEV, shared=cfg.shared)
+    res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
+    torch.cuda.synchronize()
+    tr = oracle_layer(cfg, d, shared=cfg.shared)
+    if cfg.shared:
+        assert np.array_equal(bits(res.shared_out), tr.extra["shared_out"])
+    assert np.array_equal(bits(res.routed_out), tr.out)
+    assert np.array_equal(res.expert_tokens.cpu().numpy() if res.expert_tokens is not None else tr.expert_tokens,
+                          tr.expert_tokens)
