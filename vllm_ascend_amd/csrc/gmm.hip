@@ -157,6 +157,9 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
 // ------------------------------------------------------------------ SwiGLU re-quantisation
 // One wavefront per row: SwiGLU values y fp32 [R, I] -> row absmax -> int8 + scale.
 // Rows at or beyond the last group are left untouched.
+// NV > 0: the row (at most NV x 256 values) stays in registers between the two passes, so y is read once;
+// NV == 0: any length, second pass re-reads the row.
+template <int NV>
 __global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __restrict__ y,
                                                              const int64_t* __restrict__ gl, int gl_type, int E,
                                                              int64_t R, int I, int8_t* __restrict__ q,
@@ -169,13 +172,30 @@ __global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __rest
     expert_rows(gl, gl_type, E - 1, lane, r0, total);
     if (row >= total) return;
     const v4f* yr = (const v4f*)(y + row * I);
+    const int nvec = I >> 2;
     float amax = 0.0f;
-    for (int i = lane; i < (I >> 2); i += 64) {
-        const v4f v = yr[i];
+    v4f held[NV > 0 ? NV : 1];
+    if constexpr (NV > 0) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float ab = __builtin_fabsf(v[j]);
-            amax = ab > amax ? ab : amax;
+        for (int n = 0; n < NV; ++n) {
+            const int i = lane + 64 * n;
+            held[n] = i < nvec ? yr[i] : (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float ab = __builtin_fabsf(held[n][j]);
+                amax = ab > amax ? ab : amax;
+            }
+    } else {
+        for (int i = lane; i < nvec; i += 64) {
+            const v4f v = yr[i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float ab = __builtin_fabsf(v[j]);
+                amax = ab > amax ? ab : amax;
+            }
         }
     }
     amax = wave_max(amax);
@@ -183,23 +203,37 @@ __global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __rest
     const float inv = 1.0f / s;
     if (lane == 0) qs[row] = (amax == 0.0f) ? 0.0f : s;
     uint32_t* qr = (uint32_t*)(q + row * I);
-    for (int i = lane; i < (I >> 2); i += 64) {
-        const v4f v = yr[i];
+    auto pack = [&](v4f v) {
         uint32_t pk = 0u;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             int8_t b = (amax == 0.0f) ? (int8_t)0 : sat_rint_i8(v[j] * inv);
             pk |= (uint32_t)(uint8_t)b << (8 * j);
         }
-        qr[i] = pk;
+        return pk;
+    };
+    if constexpr (NV > 0) {
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            const int i = lane + 64 * n;
+            if (i < nvec) qr[i] = pack(held[n]);
+        }
+    } else {
+        for (int i = lane; i < nvec; i += 64) qr[i] = pack(yr[i]);
     }
 }
 
 void launch_swiglu_requant(const float* y, const int64_t* gl, int gl_type, int E, int64_t R, int I, int8_t* q,
                            float* qs, hipStream_t st)
 {
-    hipLaunchKernelGGL(swiglu_requant_kernel, dim3((unsigned)((R + 3) / 4)), dim3(256), 0, st, y, gl, gl_type, E, R, I,
-                       q, qs);
+    const dim3 grid((unsigned)((R + 3) / 4));
+#define MOE355_REQUANT(NV_) \
+    hipLaunchKernelGGL(swiglu_requant_kernel<NV_>, grid, dim3(256), 0, st, y, gl, gl_type, E, R, I, q, qs)
+    if (I <= 4 * 256) MOE355_REQUANT(4);
+    else if (I <= 8 * 256) MOE355_REQUANT(8);
+    else if (I <= 16 * 256) MOE355_REQUANT(16);
+    else MOE355_REQUANT(0);
+#undef MOE355_REQUANT
 }
 
 static int check_gmm(const void* x, const void* w, const int64_t* gl, int gl_type, int64_t rows, int64_t k, int64_t n,

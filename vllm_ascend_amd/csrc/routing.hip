@@ -23,6 +23,7 @@ constexpr int kChunk = 256;
 struct RouteWs {
     int32_t* chunk_hist;  // [nchunks][E]   histogram, then start row of (chunk, expert)
     int32_t* off;         // [E + 1]        first row of each expert
+    int32_t* pbase;       // [parts][E]     rows of expert e in the chunk partitions before part p (scan kernel)
 };
 
 __host__ __device__ inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -46,36 +47,56 @@ __global__ __launch_bounds__(256) void route_hist_kernel(const int32_t* __restri
     for (int e = threadIdx.x; e < E; e += 256) dstp[e] = hist[e];
 }
 
-// One workgroup of 256.  Thread t owns experts [t*seg, (t+1)*seg).
-__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E,
-                                                         int tokens_num_type, int32_t* __restrict__ off,
-                                                         int64_t* __restrict__ expert_tokens)
+// One workgroup of 1024.  The chunks are cut into `parts` contiguous partitions of `cpp` chunks; thread (p, e)
+// scans partition p of column e (its loads do not depend on each other, 32 are in flight at a time), so the
+// column scan takes nchunks / parts steps instead of nchunks.  chunk_hist[c][e] becomes the number of rows of
+// expert e in the earlier chunks of c's partition; pbase[p][e] the number in the partitions before p.
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E,
+                                                                  int parts, int cpp, int tokens_num_type,
+                                                                  int32_t* __restrict__ off,
+                                                                  int32_t* __restrict__ pbase,
+                                                                  int64_t* __restrict__ expert_tokens)
 {
-    extern __shared__ int32_t cnt[];  // [E] counts, then [256] partials
+    extern __shared__ int32_t cnt[];  // [E] counts, [256] partials, [parts * E] partition totals
     int32_t* partial = cnt + E;
-    // column scan over chunks: chunk_hist[c][e] <- number of rows of expert e in chunks before c
-    // (32 chunks at a time: the loads of a batch are independent, so their latencies overlap)
-    for (int e = threadIdx.x; e < E; e += 256) {
+    int32_t* ptot = partial + 256;
+    for (int idx = threadIdx.x; idx < parts * E; idx += kScanThreads) {
+        const int p = idx / E, e = idx - p * E;
+        const int c_begin = p * cpp;
+        const int c_end = c_begin + cpp < nchunks ? c_begin + cpp : nchunks;
         int32_t run = 0;
-        for (int c0 = 0; c0 < nchunks; c0 += 32) {
+        for (int c0 = c_begin; c0 < c_end; c0 += 32) {
             int32_t v[32];
 #pragma unroll
-            for (int j = 0; j < 32; ++j) v[j] = (c0 + j < nchunks) ? chunk_hist[(int64_t)(c0 + j) * E + e] : 0;
+            for (int j = 0; j < 32; ++j) v[j] = (c0 + j < c_end) ? chunk_hist[(int64_t)(c0 + j) * E + e] : 0;
 #pragma unroll
             for (int j = 0; j < 32; ++j) {
-                if (c0 + j < nchunks) chunk_hist[(int64_t)(c0 + j) * E + e] = run;
+                if (c0 + j < c_end) chunk_hist[(int64_t)(c0 + j) * E + e] = run;
                 run += v[j];
             }
         }
-        cnt[e] = run;
+        ptot[idx] = run;
     }
     __syncthreads();
+    for (int idx = threadIdx.x; idx < parts * E; idx += kScanThreads) {
+        const int p = idx / E, e = idx - p * E;
+        int32_t before = 0;
+        for (int pp = 0; pp < p; ++pp) before += ptot[pp * E + e];
+        pbase[idx] = before;
+        if (p == parts - 1) cnt[e] = before + ptot[idx];
+    }
+    __syncthreads();
+    // exclusive scan over the experts: the first 256 threads own experts [t * seg, (t + 1) * seg)
+    const bool owner = threadIdx.x < 256;
     const int seg = (E + 255) / 256;
     const int e0 = threadIdx.x * seg;
-    int32_t s = 0;
-    for (int j = 0; j < seg; ++j)
-        if (e0 + j < E) s += cnt[e0 + j];
-    partial[threadIdx.x] = s;
+    if (owner) {
+        int32_t s = 0;
+        for (int j = 0; j < seg; ++j)
+            if (e0 + j < E) s += cnt[e0 + j];
+        partial[threadIdx.x] = s;
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
         int32_t run = 0;
@@ -86,14 +107,16 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ c
         }
     }
     __syncthreads();
-    int32_t run = partial[threadIdx.x];
-    for (int j = 0; j < seg; ++j) {
-        int e = e0 + j;
-        if (e < E) {
-            off[e] = run;
-            run += cnt[e];
-            expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
-            if (e == E - 1) off[E] = run;
+    if (owner) {
+        int32_t run = partial[threadIdx.x];
+        for (int j = 0; j < seg; ++j) {
+            int e = e0 + j;
+            if (e < E) {
+                off[e] = run;
+                run += cnt[e];
+                expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
+                if (e == E - 1) off[E] = run;
+            }
         }
     }
 }
@@ -102,12 +125,14 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ c
 __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __restrict__ ids, int64_t R, int E,
                                                            int nbits, const int32_t* __restrict__ chunk_start,
                                                            const int32_t* __restrict__ off,
+                                                           const int32_t* __restrict__ pbase, int cpp,
                                                            int32_t* __restrict__ dst)
 {
     extern __shared__ int32_t cursor[];  // [E] next free row of each expert for this chunk
     const int lane = threadIdx.x;
     const int32_t* cs = chunk_start + (int64_t)blockIdx.x * E;
-    for (int e = lane; e < E; e += 64) cursor[e] = off[e] + cs[e];
+    const int32_t* pb = pbase + (int64_t)((int)blockIdx.x / cpp) * E;
+    for (int e = lane; e < E; e += 64) cursor[e] = off[e] + pb[e] + cs[e];
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kChunk;
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -315,7 +340,9 @@ extern "C" size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, i
     if (num_tokens < 0 || top_k <= 0 || num_experts <= 0) return 0;
     const int64_t R = num_tokens * top_k;
     size_t n = nchunks_of(R > 0 ? R : 1);
-    return align256(n * (size_t)num_experts * 4) + align256(((size_t)num_experts + 1) * 4);
+    // chunk histograms, expert offsets, partition bases of the scan (parts * E <= max(1024, E) entries)
+    const size_t pb = num_experts > 1024 ? (size_t)num_experts : 1024;
+    return align256(n * (size_t)num_experts * 4) + align256(((size_t)num_experts + 1) * 4) + align256(pb * 4);
 }
 
 extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
@@ -345,6 +372,11 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     RouteWs ws;
     ws.chunk_hist = (int32_t*)workspace;
     ws.off = (int32_t*)((char*)workspace + align256((size_t)nch * E * 4));
+    ws.pbase = (int32_t*)((char*)ws.off + align256(((size_t)E + 1) * 4));
+    int parts = E < kScanThreads ? kScanThreads / E : 1;
+    if (parts > nch) parts = nch;
+    const int cpp = (nch + parts - 1) / parts;
+    parts = (nch + cpp - 1) / cpp;  // no empty partition
     int nbits = 0;
     while ((1 << nbits) < E) ++nbits;
 
@@ -354,10 +386,10 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     } else {
         hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E,
                            ws.chunk_hist);
-        hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), ((size_t)E + 256) * 4, st, ws.chunk_hist, nch, E,
-                           tokens_num_type, ws.off, expert_tokens);
+        hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), ((size_t)E + 256 + (size_t)parts * E) * 4, st,
+                           ws.chunk_hist, nch, E, parts, cpp, tokens_num_type, ws.off, ws.pbase, expert_tokens);
         hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
-                           ws.chunk_hist, ws.off, expanded_row_idx);
+                           ws.chunk_hist, ws.off, ws.pbase, cpp, expanded_row_idx);
     }
     if (R > 0) {
         if (quant_mode == 1 && x_dtype == MOE355_DT_F16)
