@@ -72,6 +72,9 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __re
 }
 
 // x [rows, n] int32 -> dequant (weight scale, then activation scale) -> SwiGLU -> dynamic int8.
+// NH > 0: a thread keeps its (at most NH) SwiGLU values between the absmax and the rounding pass;
+// NH == 0: any row length, the values are computed again in the second pass.
+template <int NH>
 __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t* __restrict__ x,
                                                                    const float* __restrict__ w_scale,
                                                                    const float* __restrict__ a_scale, int64_t n,
@@ -85,8 +88,7 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
     const float as = a_scale[row];
     const int64_t goff = activate_left ? 0 : half;
     const int64_t uoff = activate_left ? half : 0;
-    float a = 0.0f;
-    for (int64_t i = threadIdx.x; i < half; i += 256) {
+    auto value = [&](int64_t i) {
         float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
         float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
         if (limit > 0.0f) {
@@ -94,24 +96,38 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
             u = u > limit ? limit : u;
             u = u < -limit ? -limit : u;
         }
-        float v = __builtin_fabsf(m_silu(g) * u);
-        a = v > a ? v : a;
+        return m_silu(g) * u;
+    };
+    float held[NH > 0 ? NH : 1];
+    float a = 0.0f;
+    if constexpr (NH > 0) {
+#pragma unroll
+        for (int j = 0; j < NH; ++j) {
+            const int64_t i = threadIdx.x + 256 * j;
+            held[j] = i < half ? value(i) : 0.0f;
+            const float v = __builtin_fabsf(held[j]);
+            a = v > a ? v : a;
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < half; i += 256) {
+            const float v = __builtin_fabsf(value(i));
+            a = v > a ? v : a;
+        }
     }
     a = block_max_256(a, lds4);
     const float s = a / 127.0f;
     const float inv = 1.0f / s;
     if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
     int8_t* yr = y + row * half;
-    for (int64_t i = threadIdx.x; i < half; i += 256) {
-        float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
-        float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
-        if (limit > 0.0f) {
-            g = g > limit ? limit : g;
-            u = u > limit ? limit : u;
-            u = u < -limit ? -limit : u;
+    if constexpr (NH > 0) {
+#pragma unroll
+        for (int j = 0; j < NH; ++j) {
+            const int64_t i = threadIdx.x + 256 * j;
+            if (i < half) yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(held[j] * inv);
         }
-        float v = m_silu(g) * u;
-        yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(v * inv);
+    } else {
+        for (int64_t i = threadIdx.x; i < half; i += 256)
+            yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(value(i) * inv);
     }
 }
 
@@ -151,7 +167,13 @@ extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight
     if (rows == 0) return MOE355_OK;
     if (!x || !weight_scale || !activation_scale || !y || !scale) return MOE355_E_ARG;
     if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
-    hipLaunchKernelGGL(dequant_swiglu_quant_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
-                       weight_scale, activation_scale, n, activate_left, clamp_limit, y, scale);
+#define MOE355_DSQ(NH_)                                                                                         \
+    hipLaunchKernelGGL(dequant_swiglu_quant_kernel<NH_>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x, \
+                       weight_scale, activation_scale, n, activate_left, clamp_limit, y, scale)
+    const int64_t half = n / 2;
+    if (half <= 4 * 256) MOE355_DSQ(4);
+    else if (half <= 16 * 256) MOE355_DSQ(16);
+    else MOE355_DSQ(0);
+#undef MOE355_DSQ
     return launch_status();
 }
