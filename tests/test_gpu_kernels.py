@@ -120,7 +120,9 @@ def _rand_groups(g, E, R, empty_some=True):
 # 128-row tiles, 48..256 with K >= 4096 the 256-row weight-streaming tiles; K % 64 != 0 always streams.
 GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100, 16, 768, 2048),
              (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256), (3000, 4, 768, 2048),
-             (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096)]
+             (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096),
+             # long rows of the SwiGLU re-quantisation: 2112 values (held in registers), 4160 (two passes)
+             (40, 4, 64, 4224), (24, 2, 64, 8320)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
@@ -224,7 +226,8 @@ def test_token_unpermute(K, orc, T, k, H, residual):
     assert np.array_equal(bits(out), ref)
 
 
-@pytest.mark.parametrize("rows,n", [(2, 192), (4, 192), (8, 384), (1, 256), (300, 2048)])
+# n / 2 up to 1024 and up to 4096 are held in registers between the passes, longer rows are computed twice
+@pytest.mark.parametrize("rows,n", [(2, 192), (4, 192), (8, 384), (1, 256), (300, 2048), (3, 4096), (2, 8448)])
 @pytest.mark.parametrize("left", [True, False])
 def test_dequant_swiglu_quant(K, orc, rows, n, left):
     g = torch.Generator().manual_seed(rows + n)
