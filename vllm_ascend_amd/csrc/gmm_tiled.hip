@@ -20,8 +20,8 @@ namespace moe355 {
 __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict__ gl, int gl_type, int E, int BM,
                                                        int max_tiles, TileMap tm)
 {
-    __shared__ int32_t part_rows[256];
-    __shared__ int32_t part_tiles[256];
+    __shared__ int32_t part_rows[16];
+    __shared__ int32_t part_tiles[16];
     const int tid = threadIdx.x;
     const int seg = (E + 255) / 256;
     const int e0 = tid * seg;
@@ -38,23 +38,13 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
             tiles += (int32_t)((m + BM - 1) / BM);
         }
     }
-    part_rows[tid] = rows;
-    part_tiles[tid] = tiles;
-    __syncthreads();
-    if (tid == 0) {
-        int32_t r = 0, t = 0;
-        for (int i = 0; i < 256; ++i) {
-            const int32_t a = part_rows[i], b = part_tiles[i];
-            part_rows[i] = r;
-            part_tiles[i] = t;
-            r += a;
-            t += b;
-        }
-        tm.count[0] = t < max_tiles ? t : max_tiles;
-    }
-    __syncthreads();
-    int64_t row = part_rows[tid];
-    int32_t t = part_tiles[tid];
+    // exclusive prefix of rows and tiles over the threads (experts in order)
+    int32_t all_rows, all_tiles;
+    const int32_t rows_before = block_scan_exclusive_i32(rows, part_rows, all_rows);
+    const int32_t tiles_before = block_scan_exclusive_i32(tiles, part_tiles, all_tiles);
+    if (tid == 0) tm.count[0] = all_tiles < max_tiles ? all_tiles : max_tiles;
+    int64_t row = rows_before;
+    int32_t t = tiles_before;
     for (int j = 0; j < seg; ++j) {
         const int e = e0 + j;
         if (e < E) {

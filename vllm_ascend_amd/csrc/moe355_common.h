@@ -133,6 +133,38 @@ __device__ __forceinline__ int wave_sum_i32(int v)
     return __builtin_amdgcn_readlane(v, 63);
 }
 
+// Inclusive prefix sum over the wavefront (the same DPP steps: shifts inside rows of 16, then the row totals).
+__device__ __forceinline__ int wave_scan_inclusive_i32(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+    return v;
+}
+
+// Exclusive prefix sum of v over the threads of a workgroup (thread order), and the total.  Every thread of
+// the workgroup calls it; lds holds one int per wavefront (at most 16) and can be reused after the call.
+__device__ __forceinline__ int block_scan_exclusive_i32(int v, int* lds, int& total)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nwaves = (blockDim.x + 63) >> 6;
+    const int inc = wave_scan_inclusive_i32(v);
+    if (lane == 63) lds[wave] = inc;
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int w = 0; w < nwaves; ++w) {
+        const int t = lds[w];
+        before += w < wave ? t : 0;
+        all += t;
+    }
+    __syncthreads();
+    total = all;
+    return before + inc - v;
+}
+
 // "a ranks before b": larger value first, ties to the lower index.
 __device__ __forceinline__ bool ranks_before(float va, int ia, float vb, int ib)
 {

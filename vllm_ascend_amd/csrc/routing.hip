@@ -87,36 +87,21 @@ __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* __res
         if (p == parts - 1) cnt[e] = before + ptot[idx];
     }
     __syncthreads();
-    // exclusive scan over the experts: the first 256 threads own experts [t * seg, (t + 1) * seg)
-    const bool owner = threadIdx.x < 256;
-    const int seg = (E + 255) / 256;
+    // exclusive scan over the experts: thread t owns experts [t * seg, (t + 1) * seg)
+    const int seg = (E + kScanThreads - 1) / kScanThreads;
     const int e0 = threadIdx.x * seg;
-    if (owner) {
-        int32_t s = 0;
-        for (int j = 0; j < seg; ++j)
-            if (e0 + j < E) s += cnt[e0 + j];
-        partial[threadIdx.x] = s;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int32_t run = 0;
-        for (int t = 0; t < 256; ++t) {
-            int32_t v = partial[t];
-            partial[t] = run;
-            run += v;
-        }
-    }
-    __syncthreads();
-    if (owner) {
-        int32_t run = partial[threadIdx.x];
-        for (int j = 0; j < seg; ++j) {
-            int e = e0 + j;
-            if (e < E) {
-                off[e] = run;
-                run += cnt[e];
-                expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
-                if (e == E - 1) off[E] = run;
-            }
+    int32_t s = 0;
+    for (int j = 0; j < seg; ++j)
+        if (e0 + j < E) s += cnt[e0 + j];
+    int32_t all;
+    int32_t run = block_scan_exclusive_i32(s, partial, all);
+    for (int j = 0; j < seg; ++j) {
+        int e = e0 + j;
+        if (e < E) {
+            off[e] = run;
+            run += cnt[e];
+            expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
+            if (e == E - 1) off[E] = run;
         }
     }
 }
