@@ -290,14 +290,18 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
 
     // ---- prologue.  After it the loads still in flight are, oldest first, A(0) B(1) A(1) B(2) ...: the same
     // order every iteration leaves behind, so the wait counts the compiler derives at the loop head are exact.
+    // Every load of the prologue is requested before the first wait, so that the fill of the pipeline costs
+    // one memory latency, not two.
     load_B(0, 0);
-    store_B(0);
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int r = 0; r + 1 < RING; ++r) {
         load_A(r, r);
         load_B(r + 1, r + 1);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    store_B(0);
+    __syncthreads();
     read_frags(bf0, 0, 0);
 
     // One pipeline step on stage U (compile-time ring position) for K block I.
