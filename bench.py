@@ -153,6 +153,19 @@ def main() -> int:
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     tokens_per_s = cfg.T / (ms_per_step * 1e-3)
 
+    # ---------------- spread of single steps: each of up to 100 steps between its own pair of events
+    n_pct = min(args.steps, 100)
+    pev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_pct)]
+    for s, e in pev:
+        s.record()
+        run()
+        e.record()
+    torch.cuda.synchronize()
+    step_us = sorted(s.elapsed_time(e) * 1e3 for s, e in pev)
+
+    def pct(p):
+        return round(step_us[min(len(step_us) - 1, int(p * len(step_us)))], 2)
+
     # ---------------- eager pass with events around the dominant kernel only
     roofline = None
     eager_ms = None
@@ -277,6 +290,7 @@ def main() -> int:
         "layer_frac_of_peak": {"hbm": round(lbytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                "mfma": round(lops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
                                "layer_algorithmic_bytes": lbytes, "layer_algorithmic_ops": lops},
+        "us_per_layer_single_steps": {"p10": pct(0.10), "p50": pct(0.50), "p90": pct(0.90), "n": n_pct},
         "eager_ms_per_step": None if eager_ms is None else round(eager_ms, 5),
         "roofline": roofline,
         "cpu_baseline": cpu,

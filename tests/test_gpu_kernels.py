@@ -75,6 +75,8 @@ def test_gating_top_k(K, orc, case):
 
 @pytest.mark.parametrize("T,k,E,H", [(3, 2, 2, 64), (64, 8, 128, 2048), (1, 1, 8, 64), (700, 8, 256, 512),
                                      (2000, 4, 16, 128), (40, 6, 2048, 64),
+                                     # the single-launch path ends at 2048 rows; 64 slots per token is its widest
+                                     (256, 8, 128, 256), (257, 8, 128, 256), (4, 64, 128, 64), (32, 64, 64, 64),
                                      # more than 2048 rows: the chunked path, whose scan splits the chunks into
                                      # 1024 / E partitions (E not a power of two, E above the thread count)
                                      (500, 6, 2048, 64), (3000, 3, 1000, 64), (1500, 2, 100, 64)])

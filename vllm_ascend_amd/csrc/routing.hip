@@ -13,7 +13,8 @@
 //      themselves by lane number, and the lowest lane advances the running
 //      per-expert cursor kept in LDS.
 // A fourth launch quantises every token row once and writes it to its k
-// destination rows.
+// destination rows.  Batches of at most 2048 pairs take one launch for all of it
+// (route_gather_small_kernel).
 #include "moe355_common.h"
 
 namespace moe355 {
@@ -152,39 +153,27 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
     }
 }
 
-// Small batches (R <= 2048 pairs): histogram, scan and stable ranks in ONE workgroup, ids held
-// in registers.  Wavefronts take their turn in order when they advance the per-expert cursors,
-// which keeps the permutation stable in the flat index.
+// Small batches (R <= 2048 pairs): routing and gather in ONE launch of num_tokens + 1 workgroups.
+// Workgroup t < num_tokens finds the destinations of its own token's k pairs by counting, over all R ids,
+// the pairs that a stable sort by expert puts in front of each of them (a smaller expert, or the same expert at a
+// smaller flat index), then quantises and writes the token's row; no workgroup waits for another one.
+// The last workgroup computes the per-expert counts and their running sum.
 constexpr int kSmallMaxIters = 8;  // 8 * 256 = 2048 pairs
+constexpr int kInvalidExpert = 0x7fffffff;
 
-__global__ __launch_bounds__(256) void route_small_kernel(const int32_t* __restrict__ ids, int R, int E, int nbits,
-                                                          int tokens_num_type, int32_t* __restrict__ off,
-                                                          int64_t* __restrict__ expert_tokens,
-                                                          int32_t* __restrict__ dst)
+__device__ __forceinline__ void small_hist_scan(const int32_t* __restrict__ ids, int R, int E, int tokens_num_type,
+                                                int32_t* __restrict__ off, int64_t* __restrict__ expert_tokens,
+                                                int32_t* sm)
 {
-    extern __shared__ int32_t sm[];  // [E] counts, [E] cursors, [256] partials
-    int32_t* cnt = sm;
-    int32_t* cursor = sm + E;
-    int32_t* partial = sm + 2 * E;
+    int32_t* cnt = sm;          // [E]
+    int32_t* partial = sm + E;  // [256]
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
     for (int e = tid; e < E; e += 256) cnt[e] = 0;
-    int my_e[kSmallMaxIters];
-#pragma unroll
-    for (int it = 0; it < kSmallMaxIters; ++it) {
-        const int f = it * 256 + tid;
-        int e = -1;
-        if (f < R) {
-            e = ids[f];
-            if (e < 0 || e >= E) e = -1;
-        }
-        my_e[it] = e;
-    }
     __syncthreads();
-#pragma unroll
-    for (int it = 0; it < kSmallMaxIters; ++it)
-        if (my_e[it] >= 0) atomicAdd(&cnt[my_e[it]], 1);
+    for (int f = tid; f < R; f += 256) {
+        const int e = ids[f];
+        if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    }
     __syncthreads();
     // exclusive scan of the counts: thread t owns experts [t*seg, (t+1)*seg)
     const int seg = (E + 255) / 256;
@@ -192,84 +181,26 @@ __global__ __launch_bounds__(256) void route_small_kernel(const int32_t* __restr
     int32_t s = 0;
     for (int j = 0; j < seg; ++j)
         if (e0 + j < E) s += cnt[e0 + j];
-    partial[tid] = s;
-    __syncthreads();
-    if (wave == 0) {
-        // 256 partials, four per lane, scanned with the wavefront
-        int32_t v[4], run = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v[j] = partial[lane * 4 + j];
-            run += v[j];
-        }
-        int32_t incl = run;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            int32_t t = __shfl_up(incl, o, 64);
-            if (lane >= o) incl += t;
-        }
-        int32_t base = incl - run;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            partial[lane * 4 + j] = base;
-            base += v[j];
-        }
-    }
-    __syncthreads();
-    int32_t run = partial[tid];
+    int total;
+    int32_t run = block_scan_exclusive_i32(s, partial, total);
     for (int j = 0; j < seg; ++j) {
         const int e = e0 + j;
         if (e < E) {
             off[e] = run;
-            cursor[e] = run;
             run += cnt[e];
             expert_tokens[e] = (tokens_num_type == 1) ? (int64_t)cnt[e] : (int64_t)run;
             if (e == E - 1) off[E] = run;
         }
     }
-    __syncthreads();
-    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    const int iters = (R + 255) / 256;
-    for (int it = 0; it < iters; ++it) {
-        int e = -1;
-#pragma unroll
-        for (int j = 0; j < kSmallMaxIters; ++j)
-            if (j == it) e = my_e[j];
-        const bool valid = e >= 0;
-        unsigned long long same = __ballot(valid);
-        for (int b = 0; b < nbits; ++b) {
-            const bool bit = (e >> b) & 1;
-            unsigned long long bal = __ballot(valid && bit);
-            same &= bit ? bal : ~bal;
-        }
-        const int rank = __popcll(same & below);
-        const int leader = valid ? (__ffsll((long long)same) - 1) : lane;
-        int32_t start = 0;
-        for (int w = 0; w < 4; ++w) {
-            if (wave == w && valid && lane == leader) {
-                start = cursor[e];
-                cursor[e] = start + __popcll(same);
-            }
-            __syncthreads();
-        }
-        start = __shfl(start, leader, 64);
-        const int f = it * 256 + tid;
-        if (f < R) dst[f] = valid ? start + rank : -1;
-    }
 }
 
-// One workgroup per token: quantise the row once, write it to its k destinations.  DT: bf16 or fp16 rows
-// (the copy without quantisation moves 16-bit patterns and does not care).
-template <bool QUANT, int DT = MOE355_DT_BF16>
-__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
-                                                          const int32_t* __restrict__ dst, void* __restrict__ xs,
-                                                          float* __restrict__ sx)
+// The token's row to its k destinations drow[0..k) (LDS, written before the call; -1 = dropped), quantised
+// per row when QUANT.  DT: bf16 or fp16 rows (the copy without quantisation moves 16-bit patterns).
+template <bool QUANT, int DT>
+__device__ __forceinline__ void gather_token_row(const uint16_t* __restrict__ xr, int64_t H, int top_k,
+                                                 const int32_t* drow, float* lds4, void* __restrict__ xs,
+                                                 float* __restrict__ sx)
 {
-    __shared__ float lds4[4];
-    __shared__ int32_t drow[64];
-    const int64_t t = blockIdx.x;
-    const uint16_t* xr = x + t * H;
-    if (threadIdx.x < top_k) drow[threadIdx.x] = dst[t * top_k + threadIdx.x];
     const int64_t nv = H >> 3;
     const v8u16* xv = (const v8u16*)xr;
     if constexpr (!QUANT) {
@@ -312,6 +243,72 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
                 if (drow[j] >= 0) ((uint2*)((int8_t*)xs + (int64_t)drow[j] * H))[i] = pk;
         }
     }
+}
+
+template <bool QUANT, int DT = MOE355_DT_BF16>
+__global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* __restrict__ ids, int R, int E,
+                                                                 int tokens_num_type, int32_t* __restrict__ off,
+                                                                 int64_t* __restrict__ expert_tokens,
+                                                                 int32_t* __restrict__ dst,
+                                                                 const uint16_t* __restrict__ x, int64_t H, int top_k,
+                                                                 void* __restrict__ xs, float* __restrict__ sx)
+{
+    extern __shared__ int32_t sm[];  // the counting workgroup: [E] counts, [256] scan scratch
+    __shared__ float lds4[4];
+    __shared__ int32_t drow[64];
+    __shared__ int32_t wsum[4][64];
+    const int num_tokens = (int)gridDim.x - 1;
+    if ((int)blockIdx.x == num_tokens) {
+        small_hist_scan(ids, R, E, tokens_num_type, off, expert_tokens, sm);
+        return;
+    }
+    const int t = blockIdx.x;
+    const int tid = threadIdx.x;
+    int my_e[kSmallMaxIters];
+#pragma unroll
+    for (int it = 0; it < kSmallMaxIters; ++it) {
+        const int f = it * 256 + tid;
+        int e = kInvalidExpert;
+        if (f < R) {
+            e = ids[f];
+            if (e < 0 || e >= E) e = kInvalidExpert;
+        }
+        my_e[it] = e;
+    }
+    for (int j = 0; j < top_k; ++j) {
+        const int fj = t * top_k + j;
+        const int ej = ids[fj];
+        int c = 0;
+#pragma unroll
+        for (int it = 0; it < kSmallMaxIters; ++it) {
+            const int f = it * 256 + tid;
+            c += (my_e[it] < ej || (my_e[it] == ej && f < fj)) ? 1 : 0;
+        }
+        c = wave_sum_i32(c);
+        if ((tid & 63) == 0) wsum[tid >> 6][j] = c;
+    }
+    __syncthreads();
+    if (tid < top_k) {
+        const int ej = ids[t * top_k + tid];
+        const bool valid = ej >= 0 && ej < E;
+        const int d = valid ? wsum[0][tid] + wsum[1][tid] + wsum[2][tid] + wsum[3][tid] : -1;
+        dst[t * top_k + tid] = d;
+        drow[tid] = d;
+    }
+    gather_token_row<QUANT, DT>(x + (int64_t)t * H, H, top_k, drow, lds4, xs, sx);
+}
+
+// One workgroup per token: quantise the row once, write it to its k destinations.
+template <bool QUANT, int DT = MOE355_DT_BF16>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
+                                                          const int32_t* __restrict__ dst, void* __restrict__ xs,
+                                                          float* __restrict__ sx)
+{
+    __shared__ float lds4[4];
+    __shared__ int32_t drow[64];
+    const int64_t t = blockIdx.x;
+    if (threadIdx.x < top_k) drow[threadIdx.x] = dst[t * top_k + threadIdx.x];
+    gather_token_row<QUANT, DT>(x + t * H, H, top_k, drow, lds4, xs, sx);
 }
 
 }  // namespace moe355
@@ -366,26 +363,35 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     while ((1 << nbits) < E) ++nbits;
 
     if (R <= kSmallMaxIters * 256) {
-        hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(256), ((size_t)2 * E + 256) * 4, st, expert_idx, (int)R, E,
-                           nbits, tokens_num_type, ws.off, expert_tokens, expanded_row_idx);
-    } else {
-        hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E,
-                           ws.chunk_hist);
-        hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), ((size_t)E + 256 + (size_t)parts * E) * 4, st,
-                           ws.chunk_hist, nch, E, parts, cpp, tokens_num_type, ws.off, ws.pbase, expert_tokens);
-        hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
-                           ws.chunk_hist, ws.off, ws.pbase, cpp, expanded_row_idx);
-    }
-    if (R > 0) {
+        const dim3 grid((unsigned)num_tokens + 1);
+        const size_t lds = ((size_t)E + 256) * 4;
         if (quant_mode == 1 && x_dtype == MOE355_DT_F16)
-            hipLaunchKernelGGL((gather_rows_kernel<true, MOE355_DT_F16>), dim3((unsigned)num_tokens), dim3(256), 0, st,
-                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+            hipLaunchKernelGGL((route_gather_small_kernel<true, MOE355_DT_F16>), grid, dim3(256), lds, st, expert_idx,
+                               (int)R, E, tokens_num_type, ws.off, expert_tokens, expanded_row_idx,
+                               (const uint16_t*)x, hidden, top_k, expanded_x, dynamic_scale);
         else if (quant_mode == 1)
-            hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, st,
-                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+            hipLaunchKernelGGL((route_gather_small_kernel<true>), grid, dim3(256), lds, st, expert_idx, (int)R, E,
+                               tokens_num_type, ws.off, expert_tokens, expanded_row_idx, (const uint16_t*)x, hidden,
+                               top_k, expanded_x, dynamic_scale);
         else
-            hipLaunchKernelGGL(gather_rows_kernel<false>, dim3((unsigned)num_tokens), dim3(256), 0, st,
-                               (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+            hipLaunchKernelGGL((route_gather_small_kernel<false>), grid, dim3(256), lds, st, expert_idx, (int)R, E,
+                               tokens_num_type, ws.off, expert_tokens, expanded_row_idx, (const uint16_t*)x, hidden,
+                               top_k, expanded_x, dynamic_scale);
+        return launch_status();
     }
+    hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E, ws.chunk_hist);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), ((size_t)E + 256 + (size_t)parts * E) * 4, st,
+                       ws.chunk_hist, nch, E, parts, cpp, tokens_num_type, ws.off, ws.pbase, expert_tokens);
+    hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
+                       ws.chunk_hist, ws.off, ws.pbase, cpp, expanded_row_idx);
+    if (quant_mode == 1 && x_dtype == MOE355_DT_F16)
+        hipLaunchKernelGGL((gather_rows_kernel<true, MOE355_DT_F16>), dim3((unsigned)num_tokens), dim3(256), 0, st,
+                           (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+    else if (quant_mode == 1)
+        hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, st,
+                           (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<false>, dim3((unsigned)num_tokens), dim3(256), 0, st,
+                           (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
     return launch_status();
 }
