@@ -11,6 +11,8 @@
 // sequential one), then f (+ bias) * token_scale goes through the shared epilogues.
 #include <hip/hip_ext.h>
 
+#include <type_traits>
+
 #include "gmm_common.h"
 
 namespace moe355 {
@@ -140,10 +142,10 @@ __device__ __forceinline__ void epilogue_run_w4(const GmmArgs& a, int64_t row, b
 }
 
 // Chunk c of the list "rows of expert 0 in pieces of CHUNK rows, then expert 1, ...": which expert, which
-// rows.  Every lane returns the same answer; false past the last chunk.  Lane l owns experts
+// rows, and whether it is the expert's only chunk.  Every lane returns the same answer; false past the last chunk.  Lane l owns experts
 // [l*seg, (l+1)*seg): local counts, a wavefront scan, then a short walk inside the owning lane's segment.
 __device__ __forceinline__ bool find_chunk(const int64_t* gl, int gl_type, int E, int c, int CHUNK, int lane, int& e,
-                                           int64_t& row0, int64_t& row1)
+                                           int64_t& row0, int64_t& row1, bool& only_chunk)
 {
     auto rows_of = [&](int i) -> int {
         const int64_t m = (gl_type == MOE355_GL_COUNT) ? gl[i] : gl[i] - (i > 0 ? gl[i - 1] : 0);
@@ -183,6 +185,7 @@ __device__ __forceinline__ bool find_chunk(const int64_t* gl, int gl_type, int E
             e = i;
             row0 = rr + (int64_t)(c - cc) * CHUNK;
             row1 = rr + m;
+            only_chunk = nc == 1;
             return true;
         }
         cc += nc;
@@ -218,7 +221,8 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     const int pi = have ? pi_raw : 0;
     int e = 0;
     int64_t row0 = 0, row1 = 0;
-    if (!find_chunk(a.gl, a.gl_type, a.E, chunk, kW4Chunk, lane, e, row0, row1)) return;
+    bool single_chunk = false;
+    if (!find_chunk(a.gl, a.gl_type, a.E, chunk, kW4Chunk, lane, e, row0, row1, single_chunk)) return;
     if (row1 > a.R) row1 = a.R;
     if (row1 <= row0) return;
     const int nb0 = (EPI == EPI_SWIGLU) ? pi : 2 * pi;
@@ -231,10 +235,18 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     // token block that was requested late would also wait for every weight block requested before it.
     constexpr int RW = 6;
     v4i a0[RW], a1[RW];
-    auto load_weights = [&](int slot, int kb) {
+    // STREAM: the expert has a single chunk, nobody else reads these weights: non-temporal loads (the faster
+    // pure stream).  Otherwise the sibling chunks of the expert run at the same time on the same XCD (their
+    // workgroup numbers differ by a multiple of 16) and ordinary loads let them share one fetch in L2.
+    auto load_weights = [&](auto stream, int slot, int kb) {
         const int k = kb < KB64 ? kb : KB64 - 1;  // past the end: a valid block that is never used
-        a0[slot] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
-        a1[slot] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
+        if constexpr (decltype(stream)::value) {
+            a0[slot] = __builtin_nontemporal_load((const v4i*)(w0 + (int64_t)k * 1024));
+            a1[slot] = __builtin_nontemporal_load((const v4i*)(w1 + (int64_t)k * 1024));
+        } else {
+            a0[slot] = *(const v4i*)(w0 + (int64_t)k * 1024);
+            a1[slot] = *(const v4i*)(w1 + (int64_t)k * 1024);
+        }
     };
 
     const int tok = lane & 31;
@@ -287,22 +299,19 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
                 if (g0 + j < n_groups) Ss[wave][(g0 + j) * 64 + lane] = t[j];
         }
     }
-#pragma unroll
-    for (int i = 0; i < RW - 1; ++i) load_weights(i, i);
     int in_group = 0, grp = 0;
     // f += float(acc / 16) * scale[e, grp, channel]
     auto fold_with = [&](const v4f* s0, const v4f* s1) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int b = 0; b < 2; ++b) {
+            if (b == 1 && !two) break;  // no rows in the second token block: its accumulators stay zero
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     f0[b][4 * q + j] = f0[b][4 * q + j] + (float)(c0[b][4 * q + j] >> 4) * s0[q][j];
                     f1[b][4 * q + j] = f1[b][4 * q + j] + (float)(c1[b][4 * q + j] >> 4) * s1[q][j];
                 }
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
             c0[b] = (v16i){0};
             c1[b] = (v16i){0};
         }
@@ -338,7 +347,7 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 #pragma unroll
     for (int i = 1; i < RW; ++i) treg[i] = load_tokens(i);
     __syncthreads();
-    auto step = [&](int slot, int kb) {  // one 64-wide K block; slot = kb % RW (compile time)
+    auto step = [&](auto stream, int slot, int kb) {  // one 64-wide K block; slot = kb % RW (compile time)
         v4i bl[2], bh[2];  // [token block]: K 0..31 / 32..63 of the block
         const int8_t* st = Bs[kb & 1];
 #pragma unroll
@@ -350,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         treg[slot] = load_tokens(kb + RW);   // block kb has left its register in the step before
         const v4i l0 = nib_lo(a0[slot]), h0 = nib_hi(a0[slot]);
         const v4i l1 = nib_lo(a1[slot]), h1 = nib_hi(a1[slot]);
-        load_weights((slot + RW - 1) % RW, kb + RW - 1);  // the slot block kb - 1 has just left
+        load_weights(stream, (slot + RW - 1) % RW, kb + RW - 1);  // the slot block kb - 1 has just left
         c0[0] = mfma_i8(l0, bl[0], c0[0]);
         c0[0] = mfma_i8(h0, bh[0], c0[0]);
         c1[0] = mfma_i8(l1, bl[0], c1[0]);
@@ -366,13 +375,19 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     };
     // whole passes through the ring without a condition on kb; the remainder is peeled
     const int kb_full = (KB64 / RW) * RW;
-    for (int kb = 0; kb < kb_full; kb += RW) {
+    auto k_loop = [&](auto stream) {
 #pragma unroll
-        for (int i = 0; i < RW; ++i) step(i, kb + i);
-    }
+        for (int i = 0; i < RW - 1; ++i) load_weights(stream, i, i);
+        for (int kb = 0; kb < kb_full; kb += RW) {
 #pragma unroll
-    for (int i = 0; i < RW - 1; ++i)
-        if (kb_full + i < KB64) step(i, kb_full + i);
+            for (int i = 0; i < RW; ++i) step(stream, i, kb + i);
+        }
+#pragma unroll
+        for (int i = 0; i < RW - 1; ++i)
+            if (kb_full + i < KB64) step(stream, i, kb_full + i);
+    };
+    if (single_chunk) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
     if (!have) return;  // (after the last barrier)
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
