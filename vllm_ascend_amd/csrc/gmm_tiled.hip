@@ -112,6 +112,11 @@ __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16
             if (row >= row_end) rs_all[b] = 0.0f;
         }
     }
+    // ... and has arrived before it: the stores below sit behind "row < row_end" branches, and a wait for a
+    // load that is still in flight at that point would have to assume that none of them was issued, which
+    // turns it into a wait for every store of the block before
+#pragma unroll
+    for (int b = 0; b < BMT; ++b) asm volatile("" : "+v"(rs_all[b]));
 #pragma unroll
     for (int b = 0; b < BMT; ++b) {
         const int64_t row = row0 + b * 32 + tok;
