@@ -98,10 +98,34 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     const int tok = lane & 31;
     const int kh = lane >> 5;
 
+    // The channel scales of the runs this wavefront finishes (all four quarters, or quarter `wave` when K is
+    // split) are requested together and before the first store of the epilogue: a load placed behind a store
+    // waits for it (the memory counter retires in order), one round trip per run.  With K split they are two
+    // registers and are requested in front of the K loop; the unsplit form requests them when the K loop has
+    // ended, two quarters at a time (all eight together cost a wavefront of occupancy).
+    constexpr int NQ = (KSPLIT == 1) ? 2 : 1;  // quarters whose scales are held at a time
+    v4f cs0[NQ], cs1[NQ];
+    auto load_channel_scales = [&](int q_first) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            cs0[i] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            cs1[i] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (EPI != EPI_I32) {
+                const float* cs = expert_scales(a, e);
+                const int ch = quad_channel(KSPLIT == 1 ? q_first + i : wave, lane);
+                cs0[i] = gload4f(cs + nb0 * 32 + ch);
+                cs1[i] = gload4f(cs + nb1 * 32 + ch);
+            }
+        }
+    };
+    if constexpr (KSPLIT > 1) load_channel_scales(0);
+
     for (int64_t r0 = row0; r0 < row1; r0 += 32) {
         const int64_t row = r0 + tok;
         const bool valid = row < row1;
         const int8_t* xr = a.x + row * a.K + kh * 16;
+        float rs = 0.0f;
+        if constexpr (EPI != EPI_I32) rs = a.row_scale[valid ? row : row0];
         v16i c0 = {0}, c1 = {0};
         if (r0 != row0) load_weights(kb_begin);
         for (int kb = kb_begin; kb < kb_end; kb += UN) {
@@ -141,14 +165,17 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
                 g[j] = red[(4 * wave + j) * 64 + lane];
                 u[j] = red[(16 + 4 * wave + j) * 64 + lane];
             }
-            epilogue_quad<EPI>(a, e, row, valid, nb0 * 32, nb1 * 32, wave, g, u, lane);
+            const int ch = quad_channel(wave, lane);
+            epilogue_run<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u, rs, cs0[0], cs1[0]);
             __syncthreads();
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
+                if (q % NQ == 0) load_channel_scales(q);  // two quarters per round trip
                 int g[4] = {c0[4 * q], c0[4 * q + 1], c0[4 * q + 2], c0[4 * q + 3]};
                 int u[4] = {c1[4 * q], c1[4 * q + 1], c1[4 * q + 2], c1[4 * q + 3]};
-                epilogue_quad<EPI>(a, e, row, valid, nb0 * 32, nb1 * 32, q, g, u, lane);
+                const int ch = quad_channel(q, lane);
+                epilogue_run<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u, rs, cs0[q % NQ], cs1[q % NQ]);
             }
         }
     }

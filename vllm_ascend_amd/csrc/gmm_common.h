@@ -70,24 +70,20 @@ __device__ __forceinline__ v4i mfma_i8_16(v4i a, v4i b, v4i c)
 }
 
 // One token row, one run of four consecutive channels starting at c0 (tile 0) and c1 (tile 1).
+// rs: the row's token scale; s0 / s1: the channel scales of the two runs.  The caller loads them before its
+// K loop: a load issued here, behind the stores of an earlier run, would wait for those stores (the memory
+// counter retires in order), one store round trip per run.
 template <int EPI>
-__device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t row, bool valid, int c0, int c1,
-                                             const int* g, const int* u)
+__device__ __forceinline__ void epilogue_run(const GmmArgs& a, int64_t row, bool valid, int c0, int c1, const int* g,
+                                             const int* u, float rs, v4f s0, v4f s1)
 {
-    const int n0 = c0, n1 = c1;
-    constexpr int ch = 0;
+    if (!valid) return;
     if constexpr (EPI == EPI_I32) {
-        if (!valid) return;
         v4i o0 = {g[0], g[1], g[2], g[3]};
         v4i o1 = {u[0], u[1], u[2], u[3]};
-        *(v4i*)(a.acc + row * a.N + n0 + ch) = o0;
-        *(v4i*)(a.acc + row * a.N + n1 + ch) = o1;
+        *(v4i*)(a.acc + row * a.N + c0) = o0;
+        *(v4i*)(a.acc + row * a.N + c1) = o1;
     } else if constexpr (EPI == EPI_DEQUANT) {
-        if (!valid) return;
-        const float rs = a.row_scale[row];
-        const float* cs = expert_scales(a, e);
-        const v4f s0 = gload4f(cs + n0 + ch);
-        const v4f s1 = gload4f(cs + n1 + ch);
         v4u16 o0, o1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -95,44 +91,30 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int e, int64_t ro
             o0[j] = a.out_f16 ? f32_to_f16(v0) : f32_to_bf16(v0);
             o1[j] = a.out_f16 ? f32_to_f16(v1) : f32_to_bf16(v1);
         }
-        *(v4u16*)(a.out + row * a.N + n0 + ch) = o0;
-        *(v4u16*)(a.out + row * a.N + n1 + ch) = o1;
+        *(v4u16*)(a.out + row * a.N + c0) = o0;
+        *(v4u16*)(a.out + row * a.N + c1) = o1;
     } else {
-        // tile 0 = gate, tile 1 = the matching up tile (n1 = n0 + N/2)
-        if (!valid) return;
+        // tile 0 = gate, tile 1 = the matching up tile (c1 = c0 + N/2)
         const int I = a.N >> 1;
-        const float rs = a.row_scale[row];
-        const float* cs = expert_scales(a, e);
-        const v4f sg = gload4f(cs + n0 + ch);
-        const v4f su = gload4f(cs + n1 + ch);
         v4f yv;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float gg = ((float)g[j] * rs) * sg[j];
-            float uu = ((float)u[j] * rs) * su[j];
+            float gg = ((float)g[j] * rs) * s0[j];
+            float uu = ((float)u[j] * rs) * s1[j];
             if (a.limit > 0.0f) {
                 gg = gg > a.limit ? a.limit : gg;
                 uu = uu > a.limit ? a.limit : uu;
                 uu = uu < -a.limit ? -a.limit : uu;
             }
-            float yy = m_silu(gg) * uu;
-            yv[j] = yy;
+            yv[j] = m_silu(gg) * uu;
         }
-        *(v4f*)(a.y + row * I + n0 + ch) = yv;
+        *(v4f*)(a.y + row * I + c0) = yv;
     }
 }
 
-// Epilogue for one quarter of a pair of 32x32 accumulator tiles: the lane's token row and the
-// run of four consecutive channels  8*q + 4*(lane/32) + 0..3  of both tiles.
-// g[4]/u[4]: the int32 accumulators of that run in tile 0 / tile 1 (first channels n0 / n1).
-template <int EPI>
-__device__ __forceinline__ void epilogue_quad(const GmmArgs& a, int e, int64_t row, bool valid, int n0, int n1,
-                                              int q, const int* g, const int* u, int lane)
-{
-    const int hi = lane >> 5;
-    const int ch = 8 * q + 4 * hi;
-    epilogue_run<EPI>(a, e, row, valid, n0 + ch, n1 + ch, g, u);
-}
+// First channel, inside a 32-channel tile, of the run that quarter q of a 32x32 accumulator tile holds in
+// this lane: 8*q + 4*(lane/32), four consecutive channels.
+__device__ __forceinline__ int quad_channel(int q, int lane) { return 8 * q + 4 * (lane >> 5); }
 
 // Measurement hook (gmm.hip): hands out, once, the events that moe355_profile_next_gemm armed on this thread
 // (both null when nothing is armed); the caller records them around exactly one kernel launch.

@@ -110,10 +110,9 @@ __device__ __forceinline__ v4i nib_hi(v4i v)
 // applied here, last.
 template <int EPI>
 __device__ __forceinline__ void epilogue_run_w4(const GmmArgs& a, int64_t row, bool valid, int c0, int c1,
-                                                const float* g, const float* u)
+                                                const float* g, const float* u, float rs)
 {
     if (!valid) return;
-    const float rs = a.row_scale[row];
     if constexpr (EPI == EPI_DEQUANT) {
         v4u16 o0, o1;
 #pragma unroll
@@ -263,6 +262,11 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         row[b] = row0 + 32 * b + tok;
         valid[b] = row[b] < row1;
     }
+    // token scales for the epilogue, requested in front of the K loop (a load placed behind the epilogue's
+    // stores would wait for them: the memory counter retires in order)
+    float rs_pre[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) rs_pre[b] = a.row_scale[valid[b] ? row[b] : row0];
     // staging: thread t carries row (t % 16) + 16 * (t / 64), 16-byte piece (t / 16) % 4 of the K block
     const int srow = (threadIdx.x & 15) + 16 * wave;
     const int skc = (threadIdx.x >> 4) & 3;
@@ -410,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
                     u[j] = u[j] + bu[j];
                 }
             }
-            epilogue_run_w4<EPI>(a, row[b], valid[b], nb0 * 32 + ch, nb1 * 32 + ch, g, u);
+            epilogue_run_w4<EPI>(a, row[b], valid[b], nb0 * 32 + ch, nb1 * 32 + ch, g, u, rs_pre[b]);
         }
     }
 }
