@@ -196,17 +196,26 @@ __device__ __forceinline__ void small_hist_scan(const int32_t* __restrict__ ids,
 
 // The token's row to its k destinations drow[0..k) (LDS, written before the call; -1 = dropped), quantised
 // per row when QUANT.  DT: bf16 or fp16 rows (the copy without quantisation moves 16-bit patterns).
+// held: the thread's first 16-byte piece of the row (first_piece()), requested by the caller before it worked
+// out the destinations; rows of up to 2048 values are then read from memory once.
+__device__ __forceinline__ v8u16 first_piece(const uint16_t* __restrict__ xr, int64_t H)
+{
+    v8u16 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if ((int64_t)threadIdx.x < (H >> 3)) v = ((const v8u16*)xr)[threadIdx.x];
+    return v;
+}
+
 template <bool QUANT, int DT>
 __device__ __forceinline__ void gather_token_row(const uint16_t* __restrict__ xr, int64_t H, int top_k,
                                                  const int32_t* drow, float* lds4, void* __restrict__ xs,
-                                                 float* __restrict__ sx)
+                                                 float* __restrict__ sx, v8u16 held)
 {
     const int64_t nv = H >> 3;
     const v8u16* xv = (const v8u16*)xr;
     if constexpr (!QUANT) {
         __syncthreads();
         for (int64_t i = threadIdx.x; i < nv; i += 256) {
-            v8u16 v = xv[i];
+            v8u16 v = i < 256 ? held : xv[i];
             for (int j = 0; j < top_k; ++j)
                 if (drow[j] >= 0) ((v8u16*)((uint16_t*)xs + (int64_t)drow[j] * H))[i] = v;
         }
@@ -214,7 +223,7 @@ __device__ __forceinline__ void gather_token_row(const uint16_t* __restrict__ xr
     } else {
         float a = 0.0f;
         for (int64_t i = threadIdx.x; i < nv; i += 256) {
-            v8u16 v = xv[i];
+            v8u16 v = i < 256 ? held : xv[i];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float f = __builtin_fabsf(half_to_f32<DT>(v[j]));
@@ -231,7 +240,7 @@ __device__ __forceinline__ void gather_token_row(const uint16_t* __restrict__ xr
         const float s = a / 127.0f;
         if (threadIdx.x < top_k && drow[threadIdx.x] >= 0) sx[drow[threadIdx.x]] = (a == 0.0f) ? 0.0f : s;
         for (int64_t i = threadIdx.x; i < nv; i += 256) {
-            v8u16 v = xv[i];
+            v8u16 v = i < 256 ? held : xv[i];
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -264,6 +273,7 @@ __global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* 
     }
     const int t = blockIdx.x;
     const int tid = threadIdx.x;
+    const v8u16 held = first_piece(x + (int64_t)t * H, H);
     int my_e[kSmallMaxIters];
 #pragma unroll
     for (int it = 0; it < kSmallMaxIters; ++it) {
@@ -295,7 +305,7 @@ __global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* 
         dst[t * top_k + tid] = d;
         drow[tid] = d;
     }
-    gather_token_row<QUANT, DT>(x + (int64_t)t * H, H, top_k, drow, lds4, xs, sx);
+    gather_token_row<QUANT, DT>(x + (int64_t)t * H, H, top_k, drow, lds4, xs, sx, held);
 }
 
 // One workgroup per token: quantise the row once, write it to its k destinations.
@@ -307,8 +317,9 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
     __shared__ float lds4[4];
     __shared__ int32_t drow[64];
     const int64_t t = blockIdx.x;
+    const v8u16 held = first_piece(x + t * H, H);
     if (threadIdx.x < top_k) drow[threadIdx.x] = dst[t * top_k + threadIdx.x];
-    gather_token_row<QUANT, DT>(x + t * H, H, top_k, drow, lds4, xs, sx);
+    gather_token_row<QUANT, DT>(x + t * H, H, top_k, drow, lds4, xs, sx, held);
 }
 
 }  // namespace moe355
