@@ -32,8 +32,14 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
 # scaled by a copy kernel of known size); filled in from the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/moe_layer_qwen3_decode_hbm_traffic.md: 194221.0 KiB x 2.00 fetched + 4260.2 KiB x 1.00 written
+    # profiles/moe_layer_qwen3_decode_hbm_traffic.md: 194220.8 KiB x 2.00 fetched + 1536.0 KiB x 1.00 written
     "c2_qwen3_decode": 399_300_000,
+    # profiles/moe_layer_qwen3_prefill_kernel_trace.md: 390005.6 KiB x 2.00 + 196608.0 KiB
+    "c3_qwen3_prefill": 1_000_100_000,
+    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3849432.4 KiB x 2.00 + 262144.0 KiB
+    "c4_dsv3_prefill": 8_152_100_000,
+    # profiles/moe_layer_w4a8_zipf_kernel_trace.md: 904625.9 KiB x 2.00 + 37416.5 KiB
+    "c5_w4a8_zipf": 1_891_000_000,
 }
 
 
