@@ -294,7 +294,11 @@ def test_grouped_matmul_swiglu_quant_v2_against_the_reference_golden(orc):
 W4_COUNTS = [0, 1, 31, 32, 33, 63, 64, 65, 0, 130, 200, 7]
 
 
-@pytest.mark.parametrize("Kd,N,group", [(256, 128, 128), (512, 192, 256), (128, 64, 128), (256, 128, 0)])
+@pytest.mark.parametrize("Kd,N,group", [(256, 128, 128), (512, 192, 256), (128, 64, 128), (256, 128, 0),
+                                        # more than 32 scale groups: the scales no longer fit LDS and are read
+                                        # from memory group by group (40 K blocks: whole passes of that
+                                        # variant's ring; 36: a remainder)
+                                        (2560, 64, 64), (2304, 128, 64)])
 @pytest.mark.parametrize("gl_type", [0, 1])
 def test_w4_gemms_at_chunk_boundaries(K, orc, Kd, N, group, gl_type):
     print(f"w4 gemms K={Kd} N={N} group={group} gl_type={gl_type}", flush=True)

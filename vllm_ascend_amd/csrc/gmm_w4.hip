@@ -232,7 +232,7 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     // weights and tokens: rings of RW single K blocks, requested RW - 1 blocks ahead of their MFMAs.  Both
     // rings have the same depth on purpose: the memory counter retires loads in order, so waiting for a
     // token block that was requested late would also wait for every weight block requested before it.
-    constexpr int RW = 6;
+    constexpr int RW = LDS_SCALES ? 6 : 5;  // scales read from memory inside the fold need the registers of one ring slot
     v4i a0[RW], a1[RW];
     // STREAM: the expert has a single chunk, nobody else reads these weights: non-temporal loads (the faster
     // pure stream).  Otherwise the sibling chunks of the expert run at the same time on the same XCD (their
@@ -262,11 +262,6 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
         row[b] = row0 + 32 * b + tok;
         valid[b] = row[b] < row1;
     }
-    // token scales for the epilogue, requested in front of the K loop (a load placed behind the epilogue's
-    // stores would wait for them: the memory counter retires in order)
-    float rs_pre[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b) rs_pre[b] = a.row_scale[valid[b] ? row[b] : row0];
     // staging: thread t carries row (t % 16) + 16 * (t / 64), 16-byte piece (t / 16) % 4 of the K block
     const int srow = (threadIdx.x & 15) + 16 * wave;
     const int skc = (threadIdx.x >> 4) & 3;
@@ -393,6 +388,11 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     if (single_chunk) k_loop(std::true_type{});
     else k_loop(std::false_type{});
     if (!have) return;  // (after the last barrier)
+    // both token scales are requested before the first store of the epilogue (a load placed behind a store
+    // would wait for it: the memory counter retires in order)
+    float rs_pre[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) rs_pre[b] = a.row_scale[valid[b] ? row[b] : row0];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
         if (b == 1 && !two) break;
