@@ -119,26 +119,28 @@ static inline uint16_t f32_to_f16(float f)
 }
 
 /*
- * exp(x) in binary32 from explicit multiplies and adds only [fixed by build].
+ * exp(x) in binary32 as one fixed sequence of operations [fixed by build].
  * The argument is first clamped to [-87, 88.72283] (so the result is always a normal
  * number or +inf; a NaN argument is treated as -87), then Cephes-style: n = rint(x*log2e),
  * Cody-Waite reduction with a two-part ln2, degree-5 polynomial, exact scaling by 2^n
- * (ldexp).  The GPU kernels run the identical operation sequence.
+ * (ldexp).  Every multiply-add of the reduction and of the polynomial is ONE fused operation
+ * (fmaf: a single rounding), written out explicitly; the GPU kernels run the identical sequence
+ * (v_fma_f32), so both sides agree bit for bit.
  */
 ORC_API float orc_expf(float x)
 {
     x = fminf(fmaxf(x, -87.0f), 88.72283f);
     float n = rintf(x * 1.44269504088896341f);
-    float r = x - n * 0.693359375f;
-    r = r - n * -2.12194440e-4f;
+    float r = fmaf(n, -0.693359375f, x);
+    r = fmaf(n, 2.12194440e-4f, r);
     float p = 1.9875691500e-4f;
-    p = p * r + 1.3981999507e-3f;
-    p = p * r + 8.3334519073e-3f;
-    p = p * r + 4.1665795894e-2f;
-    p = p * r + 1.6666665459e-1f;
-    p = p * r + 5.0000001201e-1f;
+    p = fmaf(p, r, 1.3981999507e-3f);
+    p = fmaf(p, r, 8.3334519073e-3f);
+    p = fmaf(p, r, 4.1665795894e-2f);
+    p = fmaf(p, r, 1.6666665459e-1f);
+    p = fmaf(p, r, 5.0000001201e-1f);
     float r2 = r * r;
-    float y = p * r2 + r;
+    float y = fmaf(p, r2, r);
     y = y + 1.0f;
     return ldexpf(y, (int)n);
 }

@@ -1,9 +1,9 @@
 // Shared device helpers for the gfx950 MoE kernels.
 //
 // Arithmetic contract shared by every kernel: IEEE binary32, round to nearest
-// even, no fused multiply-add (the library is compiled with -ffp-contract=off),
-// one exp() built from explicit multiplies and adds.  A CPU program executing
-// the same operation sequence produces the same bits.
+// even, no fused multiply-add except where one is written out (the library is
+// compiled with -ffp-contract=off; exp() and the router gate use explicit fmaf).
+// A CPU program executing the same operation sequence produces the same bits.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -71,21 +71,22 @@ __device__ __forceinline__ uint16_t f32_to_half(float f)
 
 // exp(x): argument clamped to [-87, 88.72283] (result always normal or +inf; NaN counts as -87),
 // n = rint(x*log2e), two-part ln2 reduction, degree-5 polynomial, exact scaling by 2^n.
-// Mul/add only, no contraction.
+// The multiply-adds of the reduction and the polynomial are explicit fused operations (one rounding each,
+// v_fma_f32); a CPU program calling fmaf in the same places produces the same bits.
 __device__ __forceinline__ float m_expf(float x)
 {
     x = __builtin_amdgcn_fmed3f(x, -87.0f, 88.72283f);  // min(max(x, -87), 88.72283) in one instruction
     float n = __builtin_rintf(x * 1.44269504088896341f);
-    float r = x - n * 0.693359375f;
-    r = r - n * -2.12194440e-4f;
+    float r = __builtin_fmaf(n, -0.693359375f, x);
+    r = __builtin_fmaf(n, 2.12194440e-4f, r);
     float p = 1.9875691500e-4f;
-    p = p * r + 1.3981999507e-3f;
-    p = p * r + 8.3334519073e-3f;
-    p = p * r + 4.1665795894e-2f;
-    p = p * r + 1.6666665459e-1f;
-    p = p * r + 5.0000001201e-1f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
     float r2 = r * r;
-    float y = p * r2 + r;
+    float y = __builtin_fmaf(p, r2, r);
     y = y + 1.0f;
     return __builtin_ldexpf(y, (int)n);
 }
