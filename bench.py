@@ -34,12 +34,12 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 MEASURED_TRAFFIC_BYTES = {
     # profiles/moe_layer_qwen3_decode_hbm_traffic.md: 194220.8 KiB x 2.00 fetched + 1536.0 KiB x 1.00 written
     "c2_qwen3_decode": 399_300_000,
-    # profiles/moe_layer_qwen3_prefill_kernel_trace.md: 390005.6 KiB x 2.00 + 196608.0 KiB
-    "c3_qwen3_prefill": 1_000_100_000,
-    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3849432.4 KiB x 2.00 + 262144.0 KiB
-    "c4_dsv3_prefill": 8_152_100_000,
-    # profiles/moe_layer_w4a8_zipf_kernel_trace.md: 904625.9 KiB x 2.00 + 37416.5 KiB
-    "c5_w4a8_zipf": 1_891_000_000,
+    # profiles/moe_layer_qwen3_prefill_kernel_trace.md: 384107.5 KiB x 2.00 + 196608.0 KiB
+    "c3_qwen3_prefill": 988_000_000,
+    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3850134.4 KiB x 2.00 + 262144.0 KiB
+    "c4_dsv3_prefill": 8_153_500_000,
+    # profiles/moe_layer_w4a8_zipf_kernel_trace.md: 900832.3 KiB x 2.00 + 32921.8 KiB
+    "c5_w4a8_zipf": 1_878_600_000,
 }
 
 
