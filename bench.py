@@ -231,7 +231,8 @@ def main() -> int:
                 # the same rule as the library's choice of GEMM kernel (rows per expert and K)
                 "kernel": ("gmm_w4_stream_kernel<EPI_SWIGLU>" if cfg.w4_group >= 0 else
                            "gmm_stream_kernel<EPI_SWIGLU>" if (R // cfg.E < 48 or cfg.H % 64 != 0) else
-                           "gmm_wide_kernel<EPI_SWIGLU>" if (R // cfg.E <= 256 and cfg.H >= 4096) else
+                           "gmm_wide_kernel<EPI_SWIGLU>" if ((R // cfg.E <= 256 and cfg.H >= 4096) or
+                                                             (96 <= R // cfg.E <= 192 and cfg.H >= 1024)) else
                            "gmm_tiled_kernel<EPI_SWIGLU>") + " (gate_up grouped GEMM + dequant + SwiGLU)",
                 "kernel_avg_us": round(avg_ms * 1e3, 2),
                 "kernel_p50_us": round(durs[len(durs) // 2] * 1e3, 2),

@@ -119,7 +119,7 @@ def _rand_groups(g, E, R, empty_some=True):
 
 
 # (rows, experts, K, N).  rows/experts picks the kernel: < 48 weight streaming, >= 48 LDS-tiled with
-# 128-row tiles, 48..256 with K >= 4096 the 256-row weight-streaming tiles; K % 64 != 0 always streams.
+# 128-row tiles, 48..256 with K >= 4096 (96..192 from K = 1024) the weight-streaming tiles; K % 64 != 0 always streams.
 GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100, 16, 768, 2048),
              (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256), (3000, 4, 768, 2048),
              (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096),
@@ -333,14 +333,16 @@ def test_w4_gemms_at_chunk_boundaries(K, orc, Kd, N, group, gl_type):
     assert np.array_equal(bits(got_b.cpu()), orc.w4_rows_to_bf16(fb, sx.numpy()))
 
 
-# rows per expert around the 128-row tile of the LDS-tiled kernel and its 64-row short-tile path
-TILE_COUNTS = [128, 64, 65, 129, 192, 193, 1, 0, 256, 63, 127, 320]
+# rows per expert around the 128-row tile of the LDS-tiled kernel and its 64-row short-tile path, and around the
+# 128 / 160 / 256-row shapes of the weight-streaming tiles
+TILE_COUNTS = [128, 64, 65, 129, 192, 193, 1, 0, 256, 63, 127, 320, 160, 161, 144, 145]
 
 
-# K >= 4096 at about 128 rows per expert selects the 256-row weight-streaming tiles (tall and wide ones occur in
-# TILE_COUNTS); the K values leave every remainder of the four- and five-stage rings
-@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320), (4096, 256), (4160, 320), (4224, 128),
-                                  (4288, 256), (4352, 192), (4416, 1152)])
+# K >= 1024 at about 128 rows per expert selects the weight-streaming tiles (tall ones and wide ones of four and of
+# five token blocks occur in TILE_COUNTS); the K values leave every remainder of the three-, four- and five-stage
+# rings
+@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320), (1024, 256), (2112, 128), (4096, 256),
+                                  (4160, 320), (4224, 128), (4288, 256), (4352, 192), (4416, 1152)])
 def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     print(f"tiled gemms at tile boundaries K={Kd} N={N}", flush=True)
     from vllm_ascend_amd._lib import W_ENK
@@ -390,7 +392,8 @@ def test_w4_group_sum_order_on_the_gpu(K, orc):
 
 
 # streaming / LDS-tiled / 256-row weight-streaming kernel
-@pytest.mark.parametrize("R,E,Kd,N", [(24, 8, 256, 128), (1538, 12, 256, 256), (1538, 12, 4096, 128)])
+@pytest.mark.parametrize("R,E,Kd,N", [(24, 8, 256, 128), (sum(TILE_COUNTS), len(TILE_COUNTS), 256, 256),
+                                      (sum(TILE_COUNTS), len(TILE_COUNTS), 4096, 128)])
 def test_gmm1_swiglu_clamp(K, orc, R, E, Kd, N):
     """swiglu_limit > 0: gate <= L, up in [-L, L] before the activation (the reference's clamp,
     csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:461-485)."""
@@ -402,7 +405,7 @@ def test_gmm1_swiglu_clamp(K, orc, R, E, Kd, N):
     w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
     sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
     sx = torch.rand(R, generator=g) * 0.05 + 0.001
-    cnt = torch.tensor(TILE_COUNTS, dtype=torch.int64) if R == 1538 else _rand_groups(g, E, R)
+    cnt = torch.tensor(TILE_COUNTS, dtype=torch.int64) if R == sum(TILE_COUNTS) else _rand_groups(g, E, R)
     cum = torch.cumsum(cnt, 0)
     f = orc.dequant_acc(orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy()), sx.numpy(), sw.numpy(), cum.numpy())
     limit = float(np.percentile(np.abs(f), 60))  # bites on a large share of the values

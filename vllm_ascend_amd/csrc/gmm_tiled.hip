@@ -407,14 +407,17 @@ __device__ __forceinline__ void wait_vmcnt()
 #define MOE355_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define MOE355_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-template <int EPI, bool WIDE>
+// NBLK: 32-row token blocks per wavefront (4; a wide tile of 5 takes up to 160 rows, so that an expert a little
+// above 128 rows keeps the wide shape instead of paying the token traffic of a tall tile).
+template <int EPI, bool WIDE, int NBLK = 4>
 __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
                                                  int8_t* lds)
 {
+    static_assert(NBLK == 4 || (WIDE && NBLK > 4 && NBLK <= 8), "tall tiles have two halves of four blocks");
     constexpr int GROUPS = WIDE ? 8 : 4;            // channel groups (two storage tiles each) per workgroup
     constexpr int A_BYTES = GROUPS * 4096;          // weights of a stage
-    constexpr int STAGE = A_BYTES + (WIDE ? 8192 : 16384);
-    constexpr int S = kWideLdsBytes / STAGE;        // 4 wide, 5 tall
+    constexpr int STAGE = A_BYTES + (WIDE ? NBLK * 2048 : 16384);
+    constexpr int S = kWideLdsBytes / STAGE;        // 4 wide (3 with more than four token blocks), 5 tall
     constexpr int NA = WIDE ? 4 : 2;                // weight loads per wavefront and stage
     constexpr int ROWB = TiledLds<EPI, 4, 3>::ROWB;
     constexpr int PATCHES = TiledLds<EPI, 4, 3>::PATCHES;
@@ -462,11 +465,16 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     // chunk, 64 bytes apart) over all banks.  Wavefront w copies rows 32 w .. 32 w + 31 (tall: two loads) or
     // 16 w .. 16 w + 15 (wide); 16-row blocks that lie past the expert's last row are not loaded at all
     // (their products are never stored).
+    // A wide tile of more than four blocks has more than eight 16-row pieces: wavefront w also copies piece
+    // w + 8 when that exists.
     constexpr int XROWS = WIDE ? 16 : 32;
+    constexpr int XSECOND = WIDE ? 8 * 16 : 16;     // rows between the first and the second piece of a wavefront
+    constexpr bool X2 = !WIDE || NBLK > 4;
     const int xchunk = ((lane & 3) - (lane >> 4)) & 3;
     const int64_t xfirst = row0 + wave * XROWS;
-    const int n_xloads = xfirst >= row_end ? 0 : ((!WIDE && xfirst + 16 < row_end) ? 2 : 1);
-    int64_t xr0 = xfirst + (lane >> 2), xr1 = xr0 + 16;
+    const bool x2 = X2 && (WIDE ? wave + 8 < 2 * NBLK : true) && xfirst + XSECOND < row_end;
+    const int n_xloads = xfirst >= row_end ? 0 : (x2 ? 2 : 1);
+    int64_t xr0 = xfirst + (lane >> 2), xr1 = xr0 + XSECOND;
     if (xr0 > row_end - 1) xr0 = row_end - 1;  // rows past the expert's end duplicate its last row
     if (xr1 > row_end - 1) xr1 = row_end - 1;
     const int8_t* xsrc0 = a.x + xr0 * a.K + xchunk * 16;
@@ -503,18 +511,20 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
         if (n_xloads >= 1)
             __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc0 + (int64_t)itc * kBK),
                                              MOE355_LPTR(base + A_BYTES + wave * (XROWS * 64)), 16, 0, 0);
-        if constexpr (!WIDE) {
+        if constexpr (X2) {
             if (n_xloads >= 2)
                 __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc1 + (int64_t)itc * kBK),
-                                                 MOE355_LPTR(base + A_BYTES + wave * 2048 + 1024), 16, 0, 0);
+                                                 MOE355_LPTR(base + A_BYTES + (WIDE ? (wave + 8) * 1024
+                                                                                    : wave * 2048 + 1024)),
+                                                 16, 0, 0);
         }
     };
 
-    v16i acc[2][4];
+    v16i acc[2][NBLK];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) acc[t][b] = (v16i){0};
+        for (int b = 0; b < NBLK; ++b) acc[t][b] = (v16i){0};
 
 #pragma unroll
     for (int r = 0; r + 1 < S; ++r) load_stage(r, r);
@@ -535,7 +545,7 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
                 const v4i a0 = *(const v4i*)(base + a_off + s * 1024);
                 const v4i a1 = *(const v4i*)(base + a_off + 2048 + s * 1024);
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
+                for (int b = 0; b < NBLK; ++b) {
                     const v4i f = *(const v4i*)(base + (s ? frag_s1 : frag_s0) + b * 2048);
                     acc[0][b] = mfma_i8(a0, f, acc[0][b]);
                     acc[1][b] = mfma_i8(a1, f, acc[1][b]);
@@ -555,7 +565,7 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     wait_vmcnt<0>();  // the redirected loads past the end still write LDS
     __builtin_amdgcn_s_barrier();
     if (!active) return;
-    tiled_epilogue<EPI, 4>(a, e, acc, hrow0, row_end, nb0, nb1, lds + wave * (PATCHES * 32 * ROWB), lane);
+    tiled_epilogue<EPI, NBLK>(a, e, acc, hrow0, row_end, nb0, nb1, lds + wave * (PATCHES * 32 * ROWB), lane);
 }
 
 template <int EPI>
@@ -579,6 +589,9 @@ __global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm,
         // a wide tile spans two column blocks: the first half of this tile's workgroups does the work
         if (nt * 2 >= n_col_blocks) return;
         stream_tile_body<EPI, true>(a, e, row0, row_end, nt, wide_lds);
+    } else if (row_end - row0 <= 160) {
+        if (nt * 2 >= n_col_blocks) return;
+        stream_tile_body<EPI, true, 5>(a, e, row0, row_end, nt, wide_lds);
     } else {
         stream_tile_body<EPI, false>(a, e, row0, row_end, nt, wide_lds);
     }
