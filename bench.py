@@ -36,8 +36,8 @@ MEASURED_TRAFFIC_BYTES = {
     "c2_qwen3_decode": 399_300_000,
     # profiles/moe_layer_qwen3_prefill_kernel_trace.md: 384107.5 KiB x 2.00 + 196608.0 KiB
     "c3_qwen3_prefill": 988_000_000,
-    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3850134.4 KiB x 2.00 + 262144.0 KiB
-    "c4_dsv3_prefill": 8_153_500_000,
+    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3842493.7 KiB x 2.00 + 262144.0 KiB
+    "c4_dsv3_prefill": 8_137_900_000,
     # profiles/moe_layer_w4a8_zipf_kernel_trace.md: 900832.3 KiB x 2.00 + 32921.8 KiB
     "c5_w4a8_zipf": 1_878_600_000,
 }
