@@ -483,13 +483,14 @@ def test_grouped_gemms_with_one_expert_owning_every_row(K, orc):
         assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
-# Seeded random problems around the borders of the kernel choice (average rows per expert 47 / 48 / 256 / 257,
-# K 4032 / 4096) with skewed group sizes: all three epilogues of whichever kernel the library picks.
+# Seeded random problems around the borders of the kernel choice (average rows per expert 47 / 48 / 95 / 96 / 192 /
+# 193 / 256 / 257, K 960 / 1024 / 4032 / 4096) with skewed group sizes: all three epilogues of whichever kernel
+# the library picks.
 def _random_gemm_problem(seed):
     rng = np.random.default_rng(seed)
     E = int(rng.integers(1, 13))
-    avg = int(rng.choice([3, 30, 47, 48, 49, 100, 200, 256, 257, 400]))
-    Kd = int(rng.choice([64, 192, 512, 4032, 4096, 4160]))
+    avg = int(rng.choice([3, 30, 47, 48, 49, 95, 96, 100, 150, 192, 193, 200, 256, 257, 400]))
+    Kd = int(rng.choice([64, 192, 512, 960, 1024, 2048, 4032, 4096, 4160]))
     N = int(rng.choice([64, 128, 320, 576]))
     R = max(1, E * avg + int(rng.integers(0, E)))
     w = rng.random(E) ** 3                      # a few experts take most rows
@@ -502,7 +503,7 @@ def _random_gemm_problem(seed):
     return E, R, Kd, N, cnt
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(24))
 def test_grouped_gemms_on_random_problems(K, orc, seed):
     from vllm_ascend_amd._lib import W_ENK
 
