@@ -89,6 +89,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2_qwen3_decode")
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
+    ap.add_argument("--with-gate", action="store_true",
+                    help="start the step one operator earlier: the fp32 router gate GEMM (hidden states -> logits, "
+                         "random fp32 weight) runs inside every step; the headline metric starts at the logits")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     args = ap.parse_args()
@@ -116,7 +119,16 @@ def main() -> int:
     x, logits = d["x"].to(dev), d["logits"].to(dev)
     del d["w13"], d["w2"]  # the host copies are only needed again for the CPU baseline
 
+    gate = None
+    if args.with_gate:
+        from vllm_ascend_amd.fused_moe.gate_linear import AscendGateLinear
+
+        gate = AscendGateLinear(cfg.H, cfg.E, device=dev)
+        gate.weight.data.copy_(torch.randn(cfg.E, cfg.H, generator=torch.Generator().manual_seed(1)) * 0.05)
+
     def step():
+        if gate is not None:
+            return layer.forward_impl(x, gate(x)[0])
         return layer.forward_impl(x, logits)
 
     res = step()
@@ -244,7 +256,7 @@ def main() -> int:
 
     # ---------------- CPU baseline: the C checker on this host, same batch
     cpu = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and gate is None:  # the CPU baseline covers the path from the logits on
         from oracle import oracle as orc
 
         d2 = make_layer(cfg, seed=0)
@@ -292,7 +304,7 @@ def main() -> int:
         "data": "synthetic (seed 0: bf16 N(0,1) activations, N(0,1) router logits, int8 U[-127,127] weights, "
                 "fp32 U(0.001,0.01) channel scales)",
         "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E, "top_k": cfg.k,
-                   "moe_intermediate": cfg.I, "scoring": cfg.scoring, "launch": mode,
+                   "moe_intermediate": cfg.I, "scoring": cfg.scoring, "launch": mode, "router_gate": gate is not None,
                    "experts_touched": int((counts > 0).sum()), "rows": R},
         "layer_frac_of_peak": {"hbm": round(lbytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                "mfma": round(lops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
