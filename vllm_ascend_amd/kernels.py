@@ -12,7 +12,15 @@ from ._lib import DT_BF16, DT_F16, DT_F32, GL_COUNT, GL_CUMSUM, W_EKN, W_ENK, ch
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """hipStream_t of torch's current stream on t's device (the raw handle: several times cheaper to look up than
+    a torch.cuda.Stream object, and this runs once per kernel launch)."""
+    if _raw_stream is not None:
+        index = t.device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
