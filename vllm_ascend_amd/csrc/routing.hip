@@ -285,14 +285,17 @@ __global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* 
         }
         my_e[it] = e;
     }
+    const int iters = (R + 255) >> 8;  // 256-pair slices that hold pairs at all
     for (int j = 0; j < top_k; ++j) {
         const int fj = t * top_k + j;
         const int ej = ids[fj];
         int c = 0;
 #pragma unroll
         for (int it = 0; it < kSmallMaxIters; ++it) {
-            const int f = it * 256 + tid;
-            c += (my_e[it] < ej || (my_e[it] == ej && f < fj)) ? 1 : 0;
+            if (it < iters) {
+                const int f = it * 256 + tid;
+                c += (my_e[it] < ej || (my_e[it] == ej && f < fj)) ? 1 : 0;
+            }
         }
         c = wave_sum_i32(c);
         if ((tid & 63) == 0) wsum[tid >> 6][j] = c;
