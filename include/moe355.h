@@ -121,6 +121,21 @@ int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t 
                         int32_t *expanded_row_idx, int64_t *expert_tokens, float *dynamic_scale, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* The same operation without a workspace argument: for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the reference.
+ * The scratch of the routing kernels (chunk histograms, expert offsets, partition bases) lives in a fixed
+ * device array of MOE355_INIT_ROUTING_STATIC_BYTES that every GPU the library runs on holds until the process
+ * ends; its address is looked up once per device, on the first call with that device current.  The call itself
+ * allocates and frees nothing.  Batches whose scratch (moe355_init_routing_workspace) does not fit the array are
+ * rejected with MOE355_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU (different streams, different threads) race and must be serialised by the caller.  Results are identical
+ * to moe355_init_routing's. */
+#define MOE355_INIT_ROUTING_STATIC_BYTES (2u << 20)
+int moe355_init_routing_static(const void *x, int x_dtype, int64_t num_tokens, int64_t hidden,
+                               const int32_t *expert_idx, int top_k, int num_experts, int quant_mode,
+                               int tokens_num_type, void *expanded_x, int32_t *expanded_row_idx,
+                               int64_t *expert_tokens, float *dynamic_scale, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Weight format cast: dense int8 weights -> the MFMA-tiled storage the grouped
  * GEMMs stream ("NZ" of this build).  Stands in for

@@ -15,6 +15,8 @@
 // A fourth launch quantises every token row once and writes it to its k
 // destination rows.  Batches of at most 2048 pairs take one launch for all of it
 // (route_gather_small_kernel).
+#include <mutex>
+
 #include "moe355_common.h"
 
 namespace moe355 {
@@ -341,11 +343,11 @@ extern "C" size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, i
     return align256(n * (size_t)num_experts * 4) + align256(((size_t)num_experts + 1) * 4) + align256(pb * 4);
 }
 
-extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
-                                   const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
-                                   int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
-                                   int64_t* expert_tokens, float* dynamic_scale, void* workspace,
-                                   size_t workspace_bytes, void* stream)
+static int init_routing_impl(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
+                             const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
+                             int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
+                             int64_t* expert_tokens, float* dynamic_scale, void* workspace, size_t workspace_bytes,
+                             void* stream)
 {
     if (num_tokens < 0 || hidden <= 0 || top_k <= 0 || num_experts <= 0) return MOE355_E_ARG;
     if (quant_mode != 1 && quant_mode != -1) return MOE355_E_UNSUPPORTED;
@@ -408,4 +410,58 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
         hipLaunchKernelGGL(gather_rows_kernel<false>, dim3((unsigned)num_tokens), dim3(256), 0, st,
                            (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
     return launch_status();
+}
+
+extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
+                                   const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
+                                   int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
+                                   int64_t* expert_tokens, float* dynamic_scale, void* workspace,
+                                   size_t workspace_bytes, void* stream)
+{
+    return init_routing_impl(x, x_dtype, num_tokens, hidden, expert_idx, top_k, num_experts, quant_mode,
+                             tokens_num_type, expanded_x, expanded_row_idx, expert_tokens, dynamic_scale, workspace,
+                             workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------------ the form that allocates nothing
+// The chunk histograms, expert offsets and partition bases of the routing kernels live in a fixed array in
+// device memory instead of a caller's workspace.  Every GPU the library runs on holds its own copy of the array
+// at its own address; the address is looked up once per device and from then on only that address is used in
+// host code (the array's name is a host-side handle, not a device pointer).
+static __device__ __align__(256) unsigned char scratch[MOE355_INIT_ROUTING_STATIC_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device; nullptr when the runtime refuses
+void* scratch_of_current_device()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int moe355_init_routing_static(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
+                                          const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
+                                          int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
+                                          int64_t* expert_tokens, float* dynamic_scale, void* stream)
+{
+    if (num_tokens < 0 || top_k <= 0 || num_experts <= 0) return MOE355_E_ARG;
+    const size_t need = moe355_init_routing_workspace(num_tokens, top_k, num_experts);
+    if (need > (size_t)MOE355_INIT_ROUTING_STATIC_BYTES) return MOE355_E_WORKSPACE;  // batch too large for the array
+    void* ws = scratch_of_current_device();
+    if (!ws) return MOE355_E_LAUNCH;
+    // Nothing in the array has to start at zero: the histogram kernel writes every entry that is read later.
+    return init_routing_impl(x, x_dtype, num_tokens, hidden, expert_idx, top_k, num_experts, quant_mode,
+                             tokens_num_type, expanded_x, expanded_row_idx, expert_tokens, dynamic_scale, ws,
+                             (size_t)MOE355_INIT_ROUTING_STATIC_BYTES, stream);
 }
