@@ -10,10 +10,13 @@
  * closed third-party binary (torch_npu / CANN), the rule fixed here is marked
  * [fixed by build].
  *
- * Arithmetic contract: IEEE-754 binary32, round-to-nearest-even, no fused
- * multiply-add anywhere (compile with -ffp-contract=off), one shared exp()
- * built from explicit multiplies and adds so that a GPU kernel executing the
- * same sequence gives the same bits.
+ * Arithmetic contract: IEEE-754 binary32, round-to-nearest-even, no
+ * contraction of a multiply and an add into a fused operation (compile with
+ * -ffp-contract=off).  Fused multiply-adds exist only where fmaf() is written
+ * out: the range reduction and the polynomial of the shared exp() (orc_expf)
+ * and the dot products of the router gate (orc_router_gate); a GPU kernel that
+ * executes the same sequence with v_fma_f32 in the same places gives the same
+ * bits.
  *
  * Parity pins (what checks each function against something other than itself;
  * the tests live in tests/test_oracle_*.py):
@@ -23,7 +26,8 @@
  *                         test_npu_moe_gating_top_k.py:33-112) over its grid,
  *                         brute-force enumeration on tiny inputs, closed forms
  *   orc_init_routing    : known-answer vector tests/ut/lora/test_lora.py:151-165,
- *                         numpy stable argsort, bincount
+ *                         numpy stable argsort, bincount; dropped (out-of-range) ids against a
+ *                         filtered numpy sort
  *   orc_dynamic_quant   : closed forms (identity rows, zero rows, .5 ties)
  *                         rounding rule itself: PARITY UNPINNED (torch_npu binary)
  *   orc_gmm_i32         : numpy int64 matmul (exact)
@@ -31,9 +35,18 @@
  *                         (test_gmm_swiglu_quant_weight_nz_tensor_list.py:14-99), +-1 LSB
  *   orc_gmm2_dequant    : numpy float64 product, bf16 rounding closed forms
  *                         multiplication order: PARITY UNPINNED (torch_npu binary)
- *   orc_unpermute       : dense torch_moe restatement (test_fused_moe.py:85-97)
+ *   orc_unpermute       : dense torch_moe restatement (test_fused_moe.py:85-97); the residual
+ *                         add: exact small-integer cases, a case that tells "added last in fp32"
+ *                         from "added after rounding" and from "added first"; skipped rows
  *                         accumulation order: PARITY UNPINNED (torch_npu binary)
- *   orc_dequant_swiglu_quant : numpy rendering of test_dequant_swiglu_quant.py:16-45
+ *   orc_dequant_swiglu_quant : numpy rendering of test_dequant_swiglu_quant.py:16-45, both
+ *                         values of activate_left (the golden's own branch, and the identity
+ *                         "swap the halves of x and of the weight scale")
+ *   shared expert (oracle.py: shared_expert_forward, composed of the functions above in the order of
+ *                         vllm_ascend/ops/fused_moe/shared_experts.py:254-301): dense float64 MLP on the
+ *                         dequantised weights within the quantisation noise, exact agreement with the
+ *                         grouped path run with one expert (which differs only in the order of the two
+ *                         scale multiplications) on power-of-two scales
  *   orc_router_gate     : float64 dot products (tolerance), exact integer cases, cases that tell the
  *                         chunked fma order from a plain ascending sum, from multiply-then-add and from
  *                         other chunk lengths; the order itself: PARITY UNPINNED (F.linear's BLAS)
@@ -356,15 +369,12 @@ ORC_API int orc_init_routing(const int32_t *ids, int64_t T, int k, int E, const 
     const int64_t R = T * k;
     int64_t *off = (int64_t *)calloc((size_t)E + 1, sizeof(int64_t));
     for (int e = 0; e < E; ++e) cnt[e] = 0;
-    for (int64_t f = 0; f < R; ++f) {
-        if (ids[f] < 0 || ids[f] >= E) {
-            free(off);
-            return -2;
-        }
-        cnt[ids[f]]++;
-    }
+    /* a pair whose expert id lies outside [0, E) is dropped: it is not counted, its row is not written and its
+     * destination is R, one past the last row (an index the combine skips) */
+    for (int64_t f = 0; f < R; ++f)
+        if (ids[f] >= 0 && ids[f] < E) cnt[ids[f]]++;
     for (int e = 0; e < E; ++e) off[e + 1] = off[e] + cnt[e];
-    for (int64_t f = 0; f < R; ++f) dst[f] = (int32_t)(off[ids[f]]++);
+    for (int64_t f = 0; f < R; ++f) dst[f] = (ids[f] >= 0 && ids[f] < E) ? (int32_t)(off[ids[f]]++) : (int32_t)R;
     free(off);
     if (xs && x) {
         float *tmp = (float *)malloc(sizeof(float) * (size_t)H);
@@ -375,6 +385,7 @@ ORC_API int orc_init_routing(const int32_t *ids, int64_t T, int k, int E, const 
             quant_row_f32(tmp, H, qrow, &s);
             for (int j = 0; j < k; ++j) {
                 int64_t d = dst[t * k + j];
+                if (d >= R) continue;
                 memcpy(xs + d * H, qrow, (size_t)H);
                 sx[d] = s;
             }
@@ -389,7 +400,8 @@ ORC_API int orc_init_routing(const int32_t *ids, int64_t T, int k, int E, const 
 ORC_API int orc_permute_rows_bf16(const int32_t *dst, int64_t T, int k, const uint16_t *x, int64_t H, uint16_t *xp)
 {
     for (int64_t t = 0; t < T; ++t)
-        for (int j = 0; j < k; ++j) memcpy(xp + (int64_t)dst[t * k + j] * H, x + t * H, (size_t)H * 2);
+        for (int j = 0; j < k; ++j)
+            if ((int64_t)dst[t * k + j] < T * k) memcpy(xp + (int64_t)dst[t * k + j] * H, x + t * H, (size_t)H * 2);
     return 0;
 }
 
@@ -586,9 +598,11 @@ ORC_API int orc_gmm2_dequant(const int32_t *acc, const float *s1, const float *s
  * call site vllm_ascend/ops/fused_moe/token_dispatcher.py:451-461.  [accumulation
  * order inside torch_npu.npu_moe_token_unpermute is not visible -- PARITY UNPINNED]
  * add (optional, [T,H] bf16) is added last in fp32 (shared-expert output).
+ * o has `rows` rows; an index whose magnitude is not below `rows` is skipped, as the reference kernel skips
+ * indices >= num_out_tokens (moe_token_unpermute.h:250-275): that is how dropped pairs leave the sum.
  */
-ORC_API int orc_unpermute(const uint16_t *o, const int32_t *dst, const uint16_t *w, int64_t T, int k, int64_t H,
-                          const uint16_t *add, uint16_t *out)
+ORC_API int orc_unpermute(const uint16_t *o, int64_t rows, const int32_t *dst, const uint16_t *w, int64_t T, int k,
+                          int64_t H, const uint16_t *add, uint16_t *out)
 {
 #pragma omp parallel for
     for (int64_t t = 0; t < T; ++t) {
@@ -597,6 +611,7 @@ ORC_API int orc_unpermute(const uint16_t *o, const int32_t *dst, const uint16_t 
             for (int j = 0; j < k; ++j) {
                 int64_t d = dst[t * k + j];
                 d = d < 0 ? -d : d;
+                if (d >= rows) continue;
                 float p = h2f(w[t * k + j]) * h2f(o[d * H + h]);
                 acc = acc + p;
             }

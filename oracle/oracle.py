@@ -187,7 +187,9 @@ def dynamic_quant(x_bf16: np.ndarray):
 
 
 def init_routing(x_bf16, topk_ids, num_experts, quant=True):
-    """Returns (expanded_x, expanded_row_idx[R] int32, expert_tokens[E] int64 counts, dynamic_scale[R]|None)."""
+    """Returns (expanded_x, expanded_row_idx[R] int32, expert_tokens[E] int64 counts, dynamic_scale[R]|None).
+    Pairs whose expert id lies outside [0, num_experts) are dropped: destination R, rows past the last valid one
+    are left zero."""
     ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
     T, k = ids.shape
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
@@ -196,18 +198,18 @@ def init_routing(x_bf16, topk_ids, num_experts, quant=True):
     dst = np.empty((R,), dtype=np.int32)
     cnt = np.empty((num_experts,), dtype=np.int64)
     if quant:
-        xs = np.empty((R, H), dtype=np.int8)
-        sx = np.empty((R,), dtype=np.float32)
+        xs = np.zeros((R, H), dtype=np.int8)
+        sx = np.zeros((R,), dtype=np.float32)
         rc = lib().orc_init_routing(_p(ids), _i64(T), _i32(k), _i32(num_experts), _p(x), _i64(H), _p(dst), _p(cnt),
                                     _p(xs), _p(sx))
         if rc != 0:
-            raise ValueError(f"orc_init_routing failed (rc={rc}): expert id out of range")
+            raise ValueError(f"orc_init_routing failed (rc={rc})")
         return xs, dst, cnt, sx
     rc = lib().orc_init_routing(_p(ids), _i64(T), _i32(k), _i32(num_experts), None, _i64(H), _p(dst), _p(cnt), None,
                                 None)
     if rc != 0:
-        raise ValueError(f"orc_init_routing failed (rc={rc}): expert id out of range")
-    xp = np.empty((R, H), dtype=np.uint16)
+        raise ValueError(f"orc_init_routing failed (rc={rc})")
+    xp = np.zeros((R, H), dtype=np.uint16)
     lib().orc_permute_rows_bf16(_p(dst), _i64(T), _i32(k), _p(x), _i64(H), _p(xp))
     return xp, dst, cnt, None
 
@@ -310,7 +312,7 @@ def unpermute(o_bf16, dst, w_bf16, add_bf16=None):
     H = o.shape[1]
     add = np.ascontiguousarray(add_bf16, dtype=np.uint16) if add_bf16 is not None else None
     out = np.empty((T, H), dtype=np.uint16)
-    lib().orc_unpermute(_p(o), _p(dst), _p(w), _i64(T), _i32(k), _i64(H), _p(add), _p(out))
+    lib().orc_unpermute(_p(o), _i64(o.shape[0]), _p(dst), _p(w), _i64(T), _i32(k), _i64(H), _p(add), _p(out))
     return out
 
 

@@ -63,8 +63,38 @@ def test_permutation_is_the_inverse_of_a_stable_argsort(T, k, E):
     assert np.array_equal(dst[order], np.arange(T * k))
     assert np.array_equal(cnt, np.bincount(ids.reshape(-1), minlength=E))
     assert np.array_equal(xp, x[order // k])  # sorted row i holds the token of flat pair order[i]
-    with pytest.raises(ValueError):
-        orc.init_routing(x, ids + E, E)
+
+
+def test_pairs_with_out_of_range_experts_are_dropped():
+    """Ids outside [0, E) take no row: the other pairs keep the stable order among themselves, the histogram
+    only counts them, and the dropped pairs point one past the last row (the index the combine skips, as the
+    reference kernel skips indices >= num_out_tokens, moe_token_unpermute.h:250-275)."""
+    rng = np.random.RandomState(77)
+    T, k, E, H = 50, 4, 16, 32
+    ids = rng.randint(0, E, size=(T, k)).astype(np.int32)
+    flat = ids.reshape(-1)
+    bad = rng.choice(T * k, size=23, replace=False)
+    flat[bad[:10]] = E + rng.randint(0, 5, size=10)
+    flat[bad[10:]] = -1 - rng.randint(0, 5, size=13)
+    x = orc.f32_to_bf16(rng.normal(size=(T, H)).astype(np.float32))
+    xs, dst, cnt, sx = orc.init_routing(x, ids, E)
+    R = T * k
+    valid = (flat >= 0) & (flat < E)
+    assert np.all(dst[~valid] == R)
+    keep = np.nonzero(valid)[0]
+    order = keep[np.argsort(flat[keep], kind="stable")]  # sorted position -> flat index, valid pairs only
+    assert np.array_equal(dst[order], np.arange(order.size))
+    assert np.array_equal(cnt, np.bincount(flat[keep], minlength=E))
+    q, s = orc.dynamic_quant(x)
+    assert np.array_equal(xs[: order.size], q[order // k]) and np.array_equal(sx[: order.size], s[order // k])
+    assert not xs[order.size:].any()  # rows past the last valid pair are not written
+    # ... and the combine leaves them out: the same result as a combine over the valid pairs with the others' weights at 0
+    o = bf16(rng.normal(size=(R, H)).astype(np.float32))
+    w = bf16(rng.rand(T, k).astype(np.float32))
+    w0 = w.copy().reshape(-1)
+    w0[~valid] = 0
+    dst0 = np.where(valid, dst, 0).astype(np.int32)
+    assert np.array_equal(orc.unpermute(o, dst, w), orc.unpermute(o, dst0, w0.reshape(T, k)))
 
 
 def test_cumsum_group_list_vectors():
@@ -236,6 +266,85 @@ def test_unpermute_against_a_dense_reference():
     w2 = bf16(np.ones((1, 3), np.float32))
     assert orc.bf16_to_f32(orc.unpermute(o2, np.array([0, 1, 2], np.int32), w2))[0, 0] == 0.0  # (2^24+1)-2^24 -> 0
     assert orc.bf16_to_f32(orc.unpermute(o2, np.array([0, 2, 1], np.int32), w2))[0, 0] == 1.0
+
+
+def test_unpermute_residual_is_added_last_in_fp32():
+    """The shared-expert output joins the sum after the k routed rows and before the one rounding to bf16."""
+    one = bf16(np.ones((1, 2), np.float32))
+    idx = np.array([0, 1], np.int32)
+
+    def run(o_vals, add_val, w=one, index=idx):
+        o = bf16(np.array(o_vals, np.float32).reshape(-1, 1))
+        add = bf16(np.array([[add_val]], np.float32))
+        return float(orc.bf16_to_f32(orc.unpermute(o, index, w, add))[0, 0])
+
+    # exact small integers
+    assert run([3.0, 4.0], 5.0) == 12.0
+    # one rounding at the end: 1 + 2^-8 is a bf16 tie (-> 1.0); with the residual 2^-8 the fp32 sum 1 + 2^-7 is
+    # representable.  Rounding before the add would give bf16(1 + 2^-8) + 2^-8 -> 1.0
+    assert run([1.0, 2.0 ** -8], 2.0 ** -8) == 1.0 + 2.0 ** -7
+    # added last: (2^24 - 2^24) + 1 = 1; added first, 1 + 2^24 rounds to 2^24 in fp32 and the result is 0
+    assert run([2.0 ** 24, -(2.0 ** 24)], 1.0) == 1.0
+    # the residual is not scaled by a routing weight
+    half = bf16(np.full((1, 2), 0.5, np.float32))
+    assert run([2.0, 4.0], 7.0, w=half) == 10.0
+    # a skipped row (index one past the end) leaves only the others and the residual
+    assert run([2.0, 4.0], 7.0, index=np.array([1, 2], np.int32)) == 11.0
+
+
+def test_dequant_swiglu_quant_activates_the_right_half_when_asked():
+    """activate_left = False: the SiLU goes on the right half, the left half is the linear factor
+    (csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant_dynamic_base.hpp:86-91 swaps the two offsets)."""
+    rng = np.random.RandomState(8)
+    rows, n = 7, 192
+    x = rng.randint(-100, 100, size=(rows, n)).astype(np.int32)
+    ws = (rng.normal(size=n) * 0.1).astype(np.float32)
+    a = (rng.normal(size=rows) * 0.5).astype(np.float32)
+    q, s = orc.dequant_swiglu_quant(x, ws, a, activate_left=False)
+    # numpy rendering of the golden with the halves exchanged
+    gu = x.astype(np.float32) * ws[None, :] * a[:, None]
+    u, g = gu[:, : n // 2].astype(np.float64), gu[:, n // 2:].astype(np.float64)
+    y = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+    assert np.allclose(s, np.abs(y).max(axis=1) / 127.0, rtol=1e-5)
+    assert np.max(np.abs(q - np.round(y / s[:, None]))) <= 1
+    # identity: exchanging the halves of x and of the weight scale turns it into the default op, bit for bit
+    swap = np.concatenate([np.arange(n // 2, n), np.arange(n // 2)])
+    q2, s2 = orc.dequant_swiglu_quant(np.ascontiguousarray(x[:, swap]), ws[swap], a, activate_left=True)
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+    # and it is not the default op
+    q3, _ = orc.dequant_swiglu_quant(x, ws, a, activate_left=True)
+    assert not np.array_equal(q, q3)
+
+
+def test_shared_expert_against_a_dense_float64_mlp():
+    """The dense W8A8 MLP of the shared expert (op order of vllm_ascend/ops/fused_moe/shared_experts.py:254-301)
+    against silu(x W1^T) * (x W3^T) W2^T on the dequantised weights in float64: they differ by the noise of the two
+    activation quantisations only.  With power-of-two weight scales the order of the two scale multiplications
+    cannot matter, and the result must equal the routed path run with one expert that owns every token."""
+    rng = np.random.RandomState(21)
+    T, H, I = 24, 256, 128
+    x = bf16(rng.normal(size=(T, H)).astype(np.float32))
+    w13 = rng.randint(-127, 128, size=(2 * I, H)).astype(np.int8)
+    w2 = rng.randint(-127, 128, size=(H, I)).astype(np.int8)
+    s13 = (rng.rand(2 * I) * 0.009 + 0.001).astype(np.float32)
+    s2 = (rng.rand(H) * 0.009 + 0.001).astype(np.float32)
+    got = orc.bf16_to_f32(orc.shared_expert_forward(x, w13, s13, w2, s2)).astype(np.float64)
+    xf = orc.bf16_to_f32(x).astype(np.float64)
+    gu = xf @ (w13.astype(np.float64) * s13[:, None].astype(np.float64)).T
+    g, u = gu[:, :I], gu[:, I:]
+    ref = (g / (1 + np.exp(-g)) * u) @ (w2.astype(np.float64) * s2[:, None].astype(np.float64)).T
+    err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert err <= 5e-2, err
+    # a dropped term, a transposed weight or a missing scale is far outside that: e.g. without the SiLU
+    wrong = (g * u) @ (w2.astype(np.float64) * s2[:, None].astype(np.float64)).T
+    assert np.linalg.norm(got - wrong) / np.linalg.norm(wrong) > 0.3
+    # one expert, top-1, weight 1: the routed path is the same MLP
+    p13 = (2.0 ** rng.randint(-10, -6, size=2 * I)).astype(np.float32)
+    p2 = (2.0 ** rng.randint(-10, -6, size=H)).astype(np.float32)
+    sh = orc.shared_expert_forward(x, w13, p13, w2, p2)
+    ids = np.zeros((T, 1), np.int32)
+    tr = orc.experts_forward(x, bf16(np.ones((T, 1), np.float32)), ids, w13[None], p13[None], w2[None], p2[None])
+    assert np.array_equal(tr.o, sh) and np.array_equal(tr.out, sh)
 
 
 def golden_dequant_swiglu_quant(x, w_scale, a_scale):
