@@ -1,22 +1,32 @@
 #!/usr/bin/env python3
 """Benchmark of the W8A8-dynamic fused-MoE layer on one MI355X.
 
-One step = one pass of the whole routed-experts layer (router logits -> final bf16)
-over one batch of synthetic tokens, through the plugin interface
+One step = one pass of the whole routed-experts layer (router logits -> final bf16, shared expert included where
+the configuration has one) over one batch of synthetic tokens, through the plugin interface
 (router.select_experts -> quant_method.apply).  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--mode graph|eager]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME[,NAME...]] [--mode graph|eager]
 
-The default workload is the Qwen3-30B-A3B-shaped decode batch (64 tokens), the
-configuration the headline metric is quoted on.  Inputs are resident in HBM before the
-timed region.  `roofline` describes the dominant kernel (the gate_up grouped GEMM), timed
-with HIP events that bracket exactly that kernel in every step of a second, eager pass.
-`cpu_baseline` is the CPU checker (a C port, OpenMP) timed on this host on the same batch.
+Without --workload every configured workload runs in this one process: the DeepSeek-V3-shaped 4096-token prefill
+(the largest single-GPU configuration and the shape the target is stated on: the top-level `value`, `ms_per_step`,
+`roofline` and `cpu_baseline` are its figures), the Qwen3-30B-A3B-shaped decode and prefill batches, the W4A8
+Zipf-routed batch and the DeepSeek-V3-shaped 64-token decode batch; `workloads` carries the same figures for each.
+Inputs are resident in HBM before the timed region (they are drawn on the GPU by a seeded generator).
+Per workload:
+  ms_per_step   K timed steps (one HIP-graph replay per step) after W warm-up steps
+  roofline      the dominant kernel (the gate_up grouped GEMM), timed with HIP events that bracket exactly that kernel
+                in every step of a second, eager pass; its name comes from the library
+  parity        the bit-exact gates of the layer against the CPU checker (routing ids and weights, permutation,
+                histogram and the first int8 quantisation on the whole batch; both int32 accumulators, the int8 SwiGLU
+                output, the expert output and the final output on sampled rows / tokens) and the relative error of
+                the 16-bit output against a reference without activation quantisation
+  cpu_baseline  the CPU checker (a C port with OpenMP) timed on this host on a bounded sample of the same batch
 """
 from __future__ import annotations
 
 import argparse
 import ctypes
+import dataclasses
 import json
 import os
 import sys
@@ -29,17 +39,16 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
-# scaled by a copy kernel of known size); filled in from the summaries under profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/moe_layer_qwen3_decode_hbm_traffic.md: 194220.8 KiB x 2.00 fetched + 1536.0 KiB x 1.00 written
-    "c2_qwen3_decode": 399_300_000,
-    # profiles/moe_layer_qwen3_prefill_kernel_trace.md: 384107.5 KiB x 2.00 + 196608.0 KiB
-    "c3_qwen3_prefill": 988_000_000,
-    # profiles/moe_layer_dsv3_prefill_kernel_trace.md: 3842493.7 KiB x 2.00 + 262144.0 KiB
-    "c4_dsv3_prefill": 8_137_900_000,
-    # profiles/moe_layer_w4a8_zipf_kernel_trace.md: 900832.3 KiB x 2.00 + 32921.8 KiB
-    "c5_w4a8_zipf": 1_878_600_000,
+HEADLINE = "c4_dsv3_prefill"
+WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode"]
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE / WRITE_SIZE scaled by a copy
+# kernel of known size), taken from the committed summaries: NOT measured in this run.
+TRAFFIC_FROM_PROFILES = {
+    "c2_qwen3_decode": (399_300_000, "profiles/moe_layer_qwen3_decode_hbm_traffic.md"),
+    "c3_qwen3_prefill": (988_000_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
+    "c4_dsv3_prefill": (8_137_900_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
+    "c5_w4a8_zipf": (1_878_600_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
 }
 
 
@@ -82,42 +91,81 @@ def layer_bytes(cfg, counts) -> int:
     return w + act
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2_qwen3_decode")
-    ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
-    ap.add_argument("--with-gate", action="store_true",
-                    help="start the step one operator earlier: the fp32 router gate GEMM (hidden states -> logits, "
-                         "random fp32 weight) runs inside every step; the headline metric starts at the logits")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-roofline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs the whole MoE layer on ONE GPU (no expert parallelism, no collectives); "
-              "--gpus must be 1", file=sys.stderr)
-        return 2
+def log(msg: str) -> None:
+    print(f"bench.py: {msg}", file=sys.stderr, flush=True)
 
-    import numpy as np
-    import torch
 
-    from _inputs import CONFIGS, bits, make_layer
+def capture(step, torch):
+    """HIP graph of one step, checked against the eager result; None when capture is not possible."""
+    want = step().routed_out
+    torch.cuda.synchronize()
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            gres = step()
+        # several replays with the program's own work between them, each checked against the eager result
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            if not torch.equal(gres.routed_out, want):
+                raise RuntimeError("graph replay differs from the eager result")
+        return graph
+    except Exception as exc:  # capture not possible: measure eager and say so
+        log(f"HIP graph capture failed ({exc}); timing eager launches")
+        return None
+
+
+def time_steps(run, steps, warmup, torch) -> float:
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def single_steps_us(run, n, torch, before=None):
+    """n steps, each between its own pair of events; `before` runs (untimed) in front of every step."""
+    pev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for s, e in pev:
+        if before is not None:
+            before()
+        s.record()
+        run()
+        e.record()
+    torch.cuda.synchronize()
+    us = sorted(s.elapsed_time(e) * 1e3 for s, e in pev)
+
+    def pct(p):
+        return round(us[min(len(us) - 1, int(p * len(us)))], 2)
+
+    return {"p10": pct(0.10), "p50": pct(0.50), "p90": pct(0.90), "n": n}
+
+
+def run_workload(name, args, lib, torch, np):
+    from _inputs import CONFIGS, make_layer
     from _layer_utils import build_layer, oracle_layer
+    from _parity import layer_parity, staged_run, to_cpu
 
-    from vllm_ascend_amd import _lib
+    from vllm_ascend_amd import kernels as K
 
-    lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        return 2
     dev = "cuda:0"
-    cfg = CONFIGS[args.workload]
-    d = make_layer(cfg, seed=0)
-    layer = build_layer(cfg, d, dev, shared=cfg.shared)
-    x, logits = d["x"].to(dev), d["logits"].to(dev)
-    del d["w13"], d["w2"]  # the host copies are only needed again for the CPU baseline
+    cfg = CONFIGS[name]
+    t_start = time.perf_counter()
+    dg = make_layer(cfg, seed=0, gen_device=dev)
+    layer = build_layer(cfg, dg, dev, shared=cfg.shared, overlap=False)
+    x, logits = dg["x"], dg["logits"]
+    torch.cuda.synchronize()
+    log(f"{name}: layer built in {time.perf_counter() - t_start:.1f} s")
 
     gate = None
     if args.with_gate:
@@ -136,77 +184,71 @@ def main() -> int:
     counts = res.expert_tokens.cpu().numpy()
     R = int(counts.sum())
 
-    # ---------------- headline: K steps of the whole layer
-    graph = None
+    # ---------------- K steps of the whole layer
     mode = args.mode
-    if mode == "graph":
-        try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for _ in range(3):
-                    step()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                gres = step()
-            graph.replay()
-            torch.cuda.synchronize()
-            if not torch.equal(gres.routed_out, res.routed_out):
-                raise RuntimeError("graph replay differs from the eager result")
-        except Exception as exc:  # capture not possible: measure eager and say so
-            print(f"bench.py: HIP graph capture failed ({exc}); timing eager launches", file=sys.stderr)
-            graph = None
-            mode = "eager"
+    graph = capture(step, torch) if mode == "graph" else None
+    if graph is None:
+        mode = "eager"
     run = graph.replay if graph is not None else step
-    for _ in range(args.warmup):
-        run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = time_steps(run, args.steps, args.warmup, torch)
     tokens_per_s = cfg.T / (ms_per_step * 1e-3)
-
-    # ---------------- spread of single steps: each of up to 100 steps between its own pair of events
     n_pct = min(args.steps, 100)
-    pev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_pct)]
-    for s, e in pev:
-        s.record()
-        run()
-        e.record()
-    torch.cuda.synchronize()
-    step_us = sorted(s.elapsed_time(e) * 1e3 for s, e in pev)
-
-    def pct(p):
-        return round(step_us[min(len(step_us) - 1, int(p * len(step_us)))], 2)
+    spread = single_steps_us(run, n_pct, torch)
+    out = {
+        "tokens_per_s": round(tokens_per_s, 1),
+        "ms_per_step": round(ms_per_step, 5),
+        "us_per_layer": round(ms_per_step * 1e3, 2),
+        "us_per_layer_single_steps": spread,
+        "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E, "top_k": cfg.k,
+                   "moe_intermediate": cfg.I, "scoring": cfg.scoring, "shared_expert": bool(cfg.shared),
+                   "weights": "int4 group %d" % cfg.w4_group if cfg.w4_group >= 0 else "int8 per channel",
+                   "launch": mode, "router_gate": gate is not None, "experts_touched": int((counts > 0).sum()),
+                   "rows": R},
+    }
+    lbytes, lops = layer_bytes(cfg, counts), algorithmic_ops(cfg, R)
+    out["layer_frac_of_peak"] = {"hbm": round(lbytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                 "mfma": round(lops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                                 "layer_algorithmic_bytes": lbytes, "layer_algorithmic_ops": lops}
+    if cfg.T <= 64:
+        # decode: the same steps with the caches emptied in front of each (a 1 GiB fill: four times the 256 MB of
+        # the Infinity Cache); only the step itself is between the events
+        flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        out["us_per_layer_single_steps_after_cache_flush"] = single_steps_us(run, min(n_pct, 50), torch,
+                                                                              before=flush.zero_)
+        del flush
+    if cfg.shared:
+        # the shared expert on the side stream, next to the routed experts
+        layer.shared_experts.multistream_overlap = True
+        g2 = capture(step, torch) if mode == "graph" else None
+        ms2 = time_steps(g2.replay if g2 is not None else step, args.steps, args.warmup, torch)
+        out["shared_expert_on_side_stream"] = {"ms_per_step": round(ms2, 5), "launch": "graph" if g2 else "eager"}
+        layer.shared_experts.multistream_overlap = False
+        del g2
 
     # ---------------- eager pass with events around the dominant kernel only
     roofline = None
-    eager_ms = None
     if not args.no_roofline:
         n = min(args.steps, 100)
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
         for _ in range(min(args.warmup, 10)):
             step()
         torch.cuda.synchronize()
-        hooked = {"i": 0}
-        from vllm_ascend_amd import kernels as K
-
+        hooked = {"i": 0, "fired": 0}
         hook_name = "gmm1_swiglu_quant_w4" if cfg.w4_group >= 0 else "gmm1_swiglu_quant"
         orig = getattr(K, hook_name)
+        rows_seen = {}
 
-        def timed_gmm1(*a, **kw):
+        def timed_gmm1(x_, *a, **kw):
+            if x_.shape[0] != R:  # the shared expert's dense GEMMs go through the same launcher
+                return orig(x_, *a, **kw)
             s, e = evs[hooked["i"]]
-            hooked["fired"] = hooked.get("fired", 0) + 1
+            hooked["fired"] += 1
+            rows_seen["rows"] = x_.shape[0]
             # create the underlying hipEvent handles, then let the library record them around the GEMM kernel
             s.record()
             e.record()
             lib.moe355_profile_next_gemm(ctypes.c_void_p(s.cuda_event), ctypes.c_void_p(e.cuda_event))
-            return orig(*a, **kw)
+            return orig(x_, *a, **kw)
 
         setattr(K, hook_name, timed_gmm1)
         try:
@@ -216,103 +258,158 @@ def main() -> int:
                 hooked["i"] = i
                 step()
             torch.cuda.synchronize()
-            te1 = time.perf_counter()
+            out["eager_ms_per_step"] = round((time.perf_counter() - te0) * 1e3 / n, 5)
         finally:
             setattr(K, hook_name, orig)
-        eager_ms = (te1 - te0) * 1e3 / n
-        fired = hooked.get("fired", 0) > 0
-        durs = sorted(s.elapsed_time(e) for s, e in evs) if fired else [1.0]  # ms
-        avg_ms = sum(durs) / len(durs)
-        abytes = algorithmic_bytes_gmm1(cfg, counts)
-        ops1 = 2 * R * cfg.H * 2 * cfg.I
-        achieved_gbs = abytes / (avg_ms * 1e-3) / 1e9
-        achieved_tops = ops1 / (avg_ms * 1e-3) / 1e12
-        # the binding roofline of this kernel: HBM when the weight stream outweighs the MFMA time
-        hbm_bound = abytes / (HBM_PEAK_GBS * 1e9) >= ops1 / (INT8_PEAK_TOPS * 1e12)
-        if not fired:
-            roofline = None
-        elif hbm_bound:
-            roofline = {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": round(achieved_gbs / HBM_PEAK_GBS, 4)}
-        else:
-            roofline = {"bound": "mfma", "achieved": round(achieved_tops, 1), "peak": INT8_PEAK_TOPS,
-                        "unit": "TOP/s", "frac": round(achieved_tops / INT8_PEAK_TOPS, 4)}
-        if roofline is not None:
+        if hooked["fired"] == n:
+            durs = sorted(s.elapsed_time(e) for s, e in evs)  # ms
+            avg_ms = sum(durs) / len(durs)
+            abytes = algorithmic_bytes_gmm1(cfg, counts)
+            ops1 = 2 * R * cfg.H * 2 * cfg.I
+            gbs = abytes / (avg_ms * 1e-3) / 1e9
+            tops = ops1 / (avg_ms * 1e-3) / 1e12
+            # the binding roofline of this kernel: HBM when the weight stream outweighs the MFMA time
+            hbm_bound = abytes / (HBM_PEAK_GBS * 1e9) >= ops1 / (INT8_PEAK_TOPS * 1e12)
+            if hbm_bound:
+                roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": round(gbs / HBM_PEAK_GBS, 4)}
+            else:
+                roofline = {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                            "frac": round(tops / INT8_PEAK_TOPS, 4)}
+            if cfg.w4_group >= 0:
+                kernel = "gmm_w4_stream_kernel"
+            else:
+                kernel = lib.moe355_gmm_kernel_name(1, R, cfg.H, 2 * cfg.I, cfg.E).decode()
+            traffic = TRAFFIC_FROM_PROFILES.get(name)
             roofline.update({
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                # the same rule as the library's choice of GEMM kernel (rows per expert and K)
-                "kernel": ("gmm_w4_stream_kernel<EPI_SWIGLU>" if cfg.w4_group >= 0 else
-                           "gmm_stream_kernel<EPI_SWIGLU>" if (R // cfg.E < 48 or cfg.H % 64 != 0) else
-                           "gmm_wide_kernel<EPI_SWIGLU>" if ((R // cfg.E <= 256 and cfg.H >= 4096) or
-                                                             (96 <= R // cfg.E <= 192 and cfg.H >= 1024)) else
-                           "gmm_tiled_kernel<EPI_SWIGLU>") + " (gate_up grouped GEMM + dequant + SwiGLU)",
+                "traffic": traffic[0] if traffic else None,
+                "traffic_source": (traffic[1] + " (rocprofv3 --pmc of an earlier run of this command, not measured "
+                                                "in this run)") if traffic else None,
+                "kernel": kernel + "<EPI_SWIGLU> (gate_up grouped GEMM + dequant + SwiGLU)",
                 "kernel_avg_us": round(avg_ms * 1e3, 2),
                 "kernel_p50_us": round(durs[len(durs) // 2] * 1e3, 2),
                 "algorithmic_bytes": abytes,
                 "algorithmic_ops": ops1,
-                "other_frac": {"hbm": round(achieved_gbs / HBM_PEAK_GBS, 4),
-                               "mfma": round(achieved_tops / INT8_PEAK_TOPS, 4)},
+                "other_frac": {"hbm": round(gbs / HBM_PEAK_GBS, 4), "mfma": round(tops / INT8_PEAK_TOPS, 4)},
             })
+    out["roofline"] = roofline
 
-    # ---------------- CPU baseline: the C checker on this host, same batch
-    cpu = None
-    if not args.no_cpu_baseline and gate is None:  # the CPU baseline covers the path from the logits on
+    # ---------------- parity gates against the CPU checker
+    dc = None
+    if not args.no_parity or not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        dc = to_cpu(dg)
+        log(f"{name}: host copies of the tensors in {time.perf_counter() - t0:.1f} s")
+    if not args.no_parity and gate is None:
         from oracle import oracle as orc
 
-        d2 = make_layer(cfg, seed=0)
+        t0 = time.perf_counter()
+        r = staged_run(K, cfg, dg)
+        big = cfg.H * cfg.I >= 4096 * 2048
+        parity = layer_parity(orc, cfg, dc, r, n_tokens=4 if big else 16, layer_out=res.routed_out,
+                              shared=cfg.shared)
+        parity["seconds"] = round(time.perf_counter() - t0, 1)
+        out["parity"] = parity
+        del r
+        log(f"{name}: parity {'FAILED ' + str(parity['failed']) if parity['failed'] else 'ok'} "
+            f"in {parity['seconds']} s")
+
+    # ---------------- CPU baseline: the C checker on this host, a bounded sample of the same batch
+    if not args.no_cpu_baseline and gate is None:
+        from oracle import oracle as orc
+
         sample_T = cfg.T
-        # bound the CPU work to roughly 10-30 s: shrink the batch for the prefill shapes
-        budget_ops = 4.0e11
+        budget_ops = 1.5e11  # per pass: a few seconds of the C port on 16 cores
         if algorithmic_ops(cfg, cfg.T * cfg.k) > budget_ops:
             sample_T = max(cfg.k, int(cfg.T * budget_ops / algorithmic_ops(cfg, cfg.T * cfg.k)))
-            d2["x"] = d2["x"][:sample_T].contiguous()
-            d2["logits"] = d2["logits"][:sample_T].contiguous()
-        import dataclasses
-
+        d2 = dict(dc)
+        d2["x"] = dc["x"][:sample_T].contiguous()
+        d2["logits"] = dc["logits"][:sample_T].contiguous()
         scfg = dataclasses.replace(cfg, T=sample_T)
         passes, elapsed, tr = 0, 0.0, None
-        while passes < 3 or (elapsed < 10.0 and passes < 1000):
+        while passes < 1 or (elapsed < args.cpu_seconds and passes < 1000):
             tc0 = time.perf_counter()
             tr = oracle_layer(scfg, d2, keep_acc=False, shared=cfg.shared)
             elapsed += time.perf_counter() - tc0
             passes += 1
-        if sample_T == cfg.T:
-            ok = bool(np.array_equal(bits(res.routed_out), tr.out))
-        else:
-            ok = None
-        cpu = {"value": round(sample_T * passes / elapsed, 2), "unit": "tokens/s", "cores": orc.num_threads(),
-               "kind": "port",
-               "sample": f"{sample_T} of {cfg.T} tokens of the same workload, {passes} passes of the whole layer "
-                         f"in {elapsed:.2f} s",
-               "gpu_output_bit_exact_vs_cpu": ok}
+        from _inputs import bits
 
-    lbytes = layer_bytes(cfg, counts)
-    lops = algorithmic_ops(cfg, R)
+        ok = bool(np.array_equal(bits(res.routed_out[:sample_T]), tr.out))
+        out["cpu_baseline"] = {
+            "value": round(sample_T * passes / elapsed, 2), "unit": "tokens/s", "cores": orc.num_threads(),
+            "kind": "port",
+            "sample": f"the first {sample_T} of {cfg.T} tokens of the same workload, {passes} pass(es) of the whole "
+                      f"layer in {elapsed:.2f} s",
+            "gpu_output_bit_exact_vs_cpu_on_sample": ok}
+        log(f"{name}: CPU baseline {out['cpu_baseline']['value']} tokens/s ({passes} passes, {elapsed:.1f} s)")
+    else:
+        out["cpu_baseline"] = None
+    del layer, dg, dc, graph
+    torch.cuda.empty_cache()
+    log(f"{name}: {out['us_per_layer']} us per layer, done in {time.perf_counter() - t_start:.1f} s")
+    return out
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=None,
+                    help="one workload or a comma-separated list; default: all of " + ", ".join(WORKLOADS))
+    ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
+    ap.add_argument("--with-gate", action="store_true",
+                    help="start the step one operator earlier: the fp32 router gate GEMM (hidden states -> logits, "
+                         "random fp32 weight) runs inside every step; the headline metric starts at the logits")
+    ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU-baseline time per workload")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the whole MoE layer on ONE GPU (no expert parallelism, no collectives); "
+              "--gpus must be 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from vllm_ascend_amd import _lib
+
+    lib = _lib.load()  # raises if the HIP library is missing: there is no fallback
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    names = args.workload.split(",") if args.workload else list(WORKLOADS)
+    head_name = HEADLINE if HEADLINE in names else names[0]
+    results = {}
+    for name in names:
+        results[name] = run_workload(name, args, lib, torch, np)
+    head = results[head_name]
+    all_ok = all(not w.get("parity", {}).get("failed") for w in results.values())
     out = {
         "metric": "W8A8 MoE-layer tokens/sec at 1 GPU",
-        "value": round(tokens_per_s, 1),
+        "value": head["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
-        "us_per_layer": round(ms_per_step * 1e3, 2),
+        "ms_per_step": head["ms_per_step"],
+        "us_per_layer": head["us_per_layer"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "int8",
-        "data": "synthetic (seed 0: bf16 N(0,1) activations, N(0,1) router logits, int8 U[-127,127] weights, "
-                "fp32 U(0.001,0.01) channel scales)",
-        "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E, "top_k": cfg.k,
-                   "moe_intermediate": cfg.I, "scoring": cfg.scoring, "launch": mode, "router_gate": gate is not None,
-                   "experts_touched": int((counts > 0).sum()), "rows": R},
-        "layer_frac_of_peak": {"hbm": round(lbytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                               "mfma": round(lops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
-                               "layer_algorithmic_bytes": lbytes, "layer_algorithmic_ops": lops},
-        "us_per_layer_single_steps": {"p10": pct(0.10), "p50": pct(0.50), "p90": pct(0.90), "n": n_pct},
-        "eager_ms_per_step": None if eager_ms is None else round(eager_ms, 5),
-        "roofline": roofline,
-        "cpu_baseline": cpu,
+        "data": "synthetic (seed 0, drawn on the GPU: bf16 N(0,1) activations, N(0,1) router logits, int8 U[-127,127] "
+                "weights, fp32 U(0.001,0.01) channel scales; int4 U[-8,7] weights with group-256 scales and "
+                "Zipf(1.1) routing for the W4A8 workload)",
+        "config": head["config"],
+        "layer_frac_of_peak": head["layer_frac_of_peak"],
+        "roofline": head["roofline"],
+        "cpu_baseline": head["cpu_baseline"],
+        "parity": head.get("parity"),
+        "parity_gates_hold_on_every_workload": all_ok,
+        "workloads": results,
     }
     print(json.dumps(out))
     return 0

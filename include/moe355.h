@@ -7,7 +7,9 @@
  *   - every call only enqueues work on `stream` (a hipStream_t passed as void*)
  *     and returns; it never synchronises, allocates or frees;
  *   - scratch memory comes from the caller: ask moe355_*_workspace() for the
- *     byte count, pass a 256-byte aligned buffer of at least that size;
+ *     byte count, pass a 256-byte aligned buffer of at least that size
+ *     (one entry point keeps its scratch in a fixed device array instead and says so:
+ *     moe355_init_routing_static);
  *   - return value 0 = enqueued; negative = rejected, nothing was enqueued
  *     (see MOE355_E_*; moe355_strerror() gives the text);
  *   - tensors are dense row-major; "bf16" means raw bfloat16 bits.  Wherever hidden states are bf16 they may
@@ -112,8 +114,11 @@ int moe355_gating_top_k(const void *x, int x_dtype, const void *bias, int64_t ro
  * quant_mode -1: expanded_x is a [R, H] copy in x's dtype and dynamic_scale is ignored.
  * expert_tokens [E] int64: per-expert counts (tokens_num_type 1) or their
  * running sum (tokens_num_type 0).
- * x [T, H] bf16 / fp16, expert_idx [T, k] int32 in [0, E).  Ids outside the range are
- * dropped (their expanded_row_idx is -1).  R = T*k must be < 2^31.
+ * x [T, H] bf16 / fp16, expert_idx [T, k] int32 in [0, E).  A pair whose id lies outside the range is
+ * dropped: it is not counted, takes no row, and its expanded_row_idx is R = T*k, one past the last row --
+ * an index that moe355_token_unpermute skips (and that survives the abs() the reference's caller applies,
+ * vllm_ascend/device/device_op.py:950-954).  Rows of expanded_x past the last valid pair are left untouched.
+ * R must be < 2^31.
  */
 size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, int num_experts);
 int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t hidden, const int32_t *expert_idx,
@@ -121,7 +126,19 @@ int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t 
                         int32_t *expanded_row_idx, int64_t *expert_tokens, float *dynamic_scale, void *workspace,
                         size_t workspace_bytes, void *stream);
 
-/* The same operation without a workspace argument: for callers that cannot allocate device memory (code under
+/* The same permutation for activations that are already quantised: x int8 [T, H] with one fp32 scale per
+ * token; rows and scales are only moved (expanded_x[row] = x[t], expanded_scale[row] = x_scale[t]).
+ * Stands in for torch_npu.npu_moe_init_routing_v2(x, ids, scale=pertoken_scale, quant_mode=-1), the call the
+ * dispatcher makes when the layer was handed pre-quantised hidden states
+ * (vllm_ascend/ops/fused_moe/token_dispatcher.py:399-435 with routing.pertoken_scale set; the expert MLP then
+ * skips its own quantisation, vllm_ascend/ops/fused_moe/moe_mlp.py:226-242).  H % 16 == 0; the workspace is
+ * the one of moe355_init_routing_workspace. */
+int moe355_init_routing_prequant(const int8_t *x, const float *x_scale, int64_t num_tokens, int64_t hidden,
+                                 const int32_t *expert_idx, int top_k, int num_experts, int tokens_num_type,
+                                 int8_t *expanded_x, int32_t *expanded_row_idx, int64_t *expert_tokens,
+                                 float *expanded_scale, void *workspace, size_t workspace_bytes, void *stream);
+
+/* moe355_init_routing without a workspace argument: for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the reference.
  * The scratch of the routing kernels (chunk histograms, expert offsets, partition bases) lives in a fixed
  * device array of MOE355_INIT_ROUTING_STATIC_BYTES that every GPU the library runs on holds until the process
@@ -268,6 +285,8 @@ int moe355_dequant_swiglu_quant(const int32_t *x, const float *weight_scale, con
  * vllm_ascend/device/device_op.py:950-954 (token_dispatcher.py:451-461; math
  * csrc/mc2/dispatch_ffn_combine/op_kernel/unpermute/moe_token_unpermute.h:241-372):
  *   out[t, :] = bf16( sum_{j=0..k-1, slot order} float(probs[t, j]) * float(permuted[|idx[t*k+j]|, :]) )
+ * Slots whose |idx| is not below permuted_rows are skipped, as the reference kernel skips indices >=
+ * num_out_tokens (moe_token_unpermute.h:250-275): dropped pairs leave the sum that way.
  * permuted [R, H] bf16 / fp16 (dtype); sorted_indices [T*k] int32; probs [T, k] in the same dtype or NULL
  * (NULL = weight 1); residual [T, H] in the same dtype or NULL is added last in fp32
  * (the shared-expert output; the reference adds it in upstream vLLM).
@@ -277,7 +296,9 @@ int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorte
                            const void *residual, void *out, void *stream);
 
 /* ---------------------------------------------------------------------------
- * Measurement hook (no counterpart in the reference; for benchmarks).
+ * Measurement hook (no counterpart in the reference; for benchmarks).  The one piece of per-thread host
+ * state in the library: the armed pair of events is kept in thread-local storage until the next GEMM launch
+ * of the same thread takes it.
  * The next grouped-GEMM kernel launched from the calling thread by
  * moe355_gmm1_swiglu_quant / moe355_gmm2_dequant / moe355_gmm_i32 is bracketed
  * by the two hipEvent_t handles (recorded immediately before and after that
@@ -285,6 +306,13 @@ int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorte
  * consumed by that launch.  Pass two NULLs to cancel.
  */
 int moe355_profile_next_gemm(void *start_event, void *stop_event);
+
+/* Which kernel family the int8 grouped GEMMs above launch for a shape, given a workspace of the size their
+ * moe355_*_workspace() asks for: "gmm_stream_kernel" (few rows per expert), "gmm_tiled_kernel" (128-row
+ * LDS-tiled) or "gmm_wide_kernel" (weight-streaming tiles of up to 256 rows); "" for arguments no GEMM accepts.
+ * epilogue: 0 raw int32 (moe355_gmm_i32), 1 SwiGLU (moe355_gmm1_swiglu_quant), 2 dequant (moe355_gmm2_dequant).
+ * A pure function of its arguments, for benchmarks and profiles (no counterpart in the reference). */
+const char *moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_t k, int64_t n, int num_experts);
 
 #ifdef __cplusplus
 }

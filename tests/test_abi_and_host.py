@@ -169,11 +169,15 @@ def test_unsupported_options_raise_by_name():
     disp = TokenDispatcherWithAllGather(top_k=2, num_experts=8, num_local_experts=8)
     base = dict(hidden_states=torch.zeros(4, 64, dtype=torch.bfloat16), topk_weights=torch.zeros(4, 2),
                 topk_ids=torch.zeros(4, 2, dtype=torch.int32), w1=[None], w2=[None], quant_type=QuantType.W8A8)
-    for kw, pat in ((dict(expert_map=torch.arange(8)), "expert_map"), (dict(mc2_mask=torch.ones(4)), "mc2_mask"),
-                    (dict(pertoken_scale=torch.ones(4)), "pertoken_scale")):
+    for kw, pat in ((dict(expert_map=torch.arange(8)), "expert_map"), (dict(mc2_mask=torch.ones(4)), "mc2_mask")):
         inp = build_token_dispatch_input(fused_experts_input=build_fused_experts_input(**base, **kw))
         with pytest.raises(NotImplementedError, match=pat):
             disp.token_dispatch(inp)
+    # pertoken_scale is honoured, for the int8 hidden states it belongs to (moe_mlp.py:226-242)
+    inp = build_token_dispatch_input(fused_experts_input=build_fused_experts_input(
+        **base, pertoken_scale=torch.ones(4)))
+    with pytest.raises(ValueError, match="int8 hidden states"):
+        disp.token_dispatch(inp)
     from vllm_ascend_amd.fused_moe.moe_mlp import quant_apply_mlp
 
     with pytest.raises(NotImplementedError, match="gelu"):
@@ -227,3 +231,102 @@ def test_dense_quant_matmul_argument_checks():
         npu_ops.npu_quant_matmul(x, w, s, pertoken_scale=torch.ones(2), output_dtype=torch.float32)
     with pytest.raises(RuntimeError):   # CPU tensors never reach a kernel: there is no host fallback
         npu_ops.npu_quant_matmul(x, w, s, output_dtype=torch.int32)
+
+
+def test_grouped_gemm_launchers_check_their_operands_on_the_host():
+    """The C ABI takes raw pointers: a scale in the model dtype, a short group list or a mis-shaped x must raise
+    in Python instead of being read out of bounds on the device.  (The checks run before the device test, so
+    CPU tensors reach them.)"""
+    from vllm_ascend_amd import kernels as K
+
+    E, n, k, rows = 4, 128, 64, 8
+    x = torch.zeros(rows, k, dtype=torch.int8)
+    w = torch.zeros(E, k, n, dtype=torch.int8)
+    s = torch.ones(E, n)
+    xs = torch.ones(rows)
+    gl = torch.tensor([2, 2, 2, 2])
+    good = dict(x=x, weight_nz=w, weight_scale=s, x_scale=xs, group_list=gl)
+
+    def gmm1(**kw):
+        a = {**good, **kw}
+        return K.gmm1_swiglu_quant(a["x"], a["weight_nz"], a["weight_scale"], a["x_scale"], a["group_list"], 1, n, k)
+
+    with pytest.raises(TypeError, match="x must be int8"):
+        gmm1(x=x.to(torch.bfloat16))
+    with pytest.raises(ValueError, match=r"x must be \[rows, K"):
+        gmm1(x=torch.zeros(rows, k + 32, dtype=torch.int8))
+    with pytest.raises(ValueError, match="one entry per expert"):
+        gmm1(group_list=gl[:3])
+    with pytest.raises(TypeError, match="x_scale must be float32"):
+        gmm1(x_scale=xs.to(torch.bfloat16))
+    with pytest.raises(ValueError, match="one scale per row"):
+        gmm1(x_scale=torch.ones(rows - 1))
+    with pytest.raises(TypeError, match="weight scale must be float32"):
+        gmm1(weight_scale=s.to(torch.bfloat16))
+    with pytest.raises(ValueError, match="weight scale holds"):
+        gmm1(weight_scale=torch.ones(E, n // 2))
+    with pytest.raises(ValueError, match="weight holds"):
+        gmm1(weight_nz=torch.zeros(E, k, n // 2, dtype=torch.int8))
+    with pytest.raises(RuntimeError, match="no CPU implementation"):  # everything else right: refused as a CPU tensor
+        gmm1()
+    w2 = torch.zeros(E, n // 2, 64, dtype=torch.int8)
+    q1 = torch.zeros(rows, n // 2, dtype=torch.int8)
+    with pytest.raises(TypeError, match="per_token_scale must be float32"):
+        K.gmm2_dequant(q1, w2, torch.ones(E, 64), xs.double(), gl, 1, 64, n // 2)
+    with pytest.raises(ValueError, match="one entry per expert"):
+        K.gmm2_dequant(q1, w2, torch.ones(E, 64), xs, gl[:2], 1, 64, n // 2)
+    with pytest.raises(TypeError, match="weight scale must be float32"):
+        K.gmm2_dequant(q1, w2, torch.ones(E, 64, dtype=torch.bfloat16), xs, gl, 1, 64, n // 2)
+    w4 = torch.zeros(E, n * k // 2, dtype=torch.uint8)
+    with pytest.raises(ValueError, match="weight scale holds"):
+        K.gmm1_swiglu_quant_w4(x, w4, torch.ones(E, 1, n), 32, xs, gl, 1, n, k)  # group 32: two groups expected
+
+
+def test_expert_tensor_lists_keep_their_address_tables():
+    """One table per list, built when the list is created and kept for its lifetime (a captured HIP graph holds the
+    table's address): many layers, and many lookups, never rebuild or evict a table; replacing an expert rewrites
+    one entry of the same table."""
+    from vllm_ascend_amd.kernels import ExpertTensorList, _as_expert_list
+
+    layers = []
+    for layer in range(40):  # more per-expert-list layers than Qwen3-30B-A3B or DeepSeek-V3 ever evicted before
+        lists = [ExpertTensorList([torch.zeros(8, 16, dtype=torch.int8) for _ in range(6)], "w") for _ in range(4)]
+        layers.append((lists, [lst.table for lst in lists]))
+    for _ in range(3):
+        for lists, tables in layers:
+            for lst, tab in zip(lists, tables):
+                assert _as_expert_list(lst, "w", torch.int8) is lst and lst.table is tab
+                assert tab.tolist() == [t.data_ptr() for t in lst]
+    lst, tab = layers[0][0][0], layers[0][1][0]
+    new = torch.ones(8, 16, dtype=torch.int8)
+    lst[2] = new
+    assert lst.table is tab and tab[2].item() == new.data_ptr() and lst[2] is new
+    with pytest.raises(RuntimeError, match=r"one\s+shape"):
+        lst[1] = torch.ones(8, 8, dtype=torch.int8)
+    with pytest.raises(TypeError, match="fixed"):
+        lst.append(new)
+    # a plain list gets a table of its own, for the one call
+    plain = [torch.zeros(8, 16, dtype=torch.int8) for _ in range(3)]
+    assert isinstance(_as_expert_list(plain, "w", torch.int8), ExpertTensorList)
+    with pytest.raises(RuntimeError, match="must be torch.float32"):
+        _as_expert_list(lst, "w", torch.float32)
+
+
+def test_force_load_balance_replaces_the_ids_only():
+    """Profile-run routing (vllm_ascend/ops/fused_moe/routed_experts.py:484-492): k distinct random experts per
+    token; exercised here on the replacement step itself (the gating kernel needs the GPU)."""
+    from vllm_ascend_amd.fused_moe.router import AscendFusedTopKRouter
+
+    r = AscendFusedTopKRouter(4, 32)
+    w = torch.rand(10, 4).to(torch.bfloat16)
+    ids = torch.zeros(10, 4, dtype=torch.int32)
+    r._compute_routing = lambda *a, **k: (w, ids)
+    torch.manual_seed(0)
+    w2, ids2 = r.select_experts(torch.zeros(10, 8, dtype=torch.bfloat16), torch.zeros(10, 32),
+                                enable_force_load_balance=True)
+    assert torch.equal(w2, w) and ids2.dtype == ids.dtype and ids2.shape == ids.shape
+    assert int(ids2.min()) >= 0 and int(ids2.max()) < 32
+    assert all(len(set(row.tolist())) == 4 for row in ids2)          # distinct experts per token
+    assert len(set(ids2.reshape(-1).tolist())) > 8                    # spread over the experts
+    w3, ids3 = r.select_experts(torch.zeros(10, 8, dtype=torch.bfloat16), torch.zeros(10, 32))
+    assert ids3 is ids

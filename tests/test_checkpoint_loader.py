@@ -225,7 +225,7 @@ def test_loader_refuses_incomplete_or_foreign_checkpoints(tmp_path):
 
 
 # ------------------------------------------------------------------ on the GPU: the loaded layer computes what the
-# directly built layer computes
+# directly built layer computes, and what the CPU checker computes
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["c1_tiny", "w4a8_small"])
 def test_layer_from_checkpoint_matches_layer_from_tensors(tmp_path, name):
@@ -260,3 +260,8 @@ def test_layer_from_checkpoint_matches_layer_from_tensors(tmp_path, name):
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     assert np.isfinite(got.float().cpu().numpy()).all()
+    # ... and both compute what the CPU checker computes from the tensors that were written to disk
+    from _inputs import bits
+    from _layer_utils import oracle_layer
+
+    assert np.array_equal(bits(got), oracle_layer(cfg, d, keep_acc=False).out)

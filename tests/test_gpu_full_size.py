@@ -27,68 +27,28 @@ def orc():
     return oracle
 
 
-def _sample_rows(counts: np.ndarray, rng, per_expert=3):
-    """Rows at the start, the end and inside of every non-empty expert's range, plus the 128- and 64-row tile
-    borders of the first experts."""
-    cum = np.cumsum(counts)
-    rows = []
-    for e, m in enumerate(counts):
-        if m == 0:
-            continue
-        lo = cum[e] - m
-        pick = {lo, cum[e] - 1, lo + int(rng.integers(0, m))}
-        if e < 8:
-            pick |= {lo + b for b in (63, 64, 127, 128) if b < m}
-        rows += sorted(pick)[: per_expert + 4]
-    return np.array(sorted(set(rows)), dtype=np.int64)
+def _make(cfg, seed=0):
+    """The configuration's tensors, drawn on the GPU (seconds for the 11 GB of the DeepSeek-V3 shapes), and CPU
+    copies of them for the checker."""
+    from _parity import to_cpu
 
-
-def _run_full(K, orc, cfg, seed=0):
-    d = make_layer(cfg, seed=seed)
-    from vllm_ascend_amd._lib import W_ENK
-
-    kw = gating_kwargs(cfg)
-    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
-    y, ids, _ = K.gating_top_k(logits, kw["k"], kw["k_group"], kw["group_count"], 1, kw["renorm"], kw["norm_type"],
-                               False, kw["routed_scaling_factor"], kw["eps"],
-                               d["bias"].to(DEV) if cfg.bias else None)
-    w_bf16 = y.to(torch.bfloat16)
-    xs, dst, cnt, sx = K.init_routing(x, ids, cfg.E, 1, 1)
-    if cfg.w4_group >= 0:
-        g = cfg.w4_group
-        w13 = K.format_cast_nz_int4(d["w13"].to(DEV), 0, 2 * cfg.I, cfg.H)
-        w2 = K.format_cast_nz_int4(d["w2"].to(DEV), 0, cfg.H, cfg.I)
-        sg13 = d["s13"].transpose(1, 2).contiguous().to(DEV)   # [E, N, G] -> [E, G, N]
-        sg2 = d["s2"].transpose(1, 2).contiguous().to(DEV)
-        q1, s1 = K.gmm1_swiglu_quant_w4(xs, w13, sg13, g, sx, cnt, 1, 2 * cfg.I, cfg.H)
-        o = K.gmm2_dequant_w4(q1, w2, sg2, g, s1, cnt, 1, cfg.H, cfg.I)
-    else:
-        w13 = K.format_cast_nz(d["w13"].to(DEV), W_ENK)
-        w2 = K.format_cast_nz(d["w2"].to(DEV), W_ENK)
-        s13, s2 = d["s13"].to(DEV), d["s2"].to(DEV)
-        q1, s1 = K.gmm1_swiglu_quant(xs, w13, s13, sx, cnt, 1, 2 * cfg.I, cfg.H)
-        o = K.gmm2_dequant(q1, w2, s2, s1, cnt, 1, cfg.H, cfg.I)
-    out = K.token_unpermute(o, dst, w_bf16)
+    dg = make_layer(cfg, seed=seed, gen_device=DEV)
     torch.cuda.synchronize()
-    return d, dict(x=x, ids=ids, w=w_bf16, xs=xs, dst=dst, cnt=cnt, sx=sx, q1=q1, s1=s1, o=o, out=out)
+    return dg, to_cpu(dg)
 
 
-@pytest.mark.parametrize("name", ["c3_qwen3_prefill", "c4_dsv3_reduced", "c5_w4a8_reduced"])
+@pytest.mark.parametrize("name", ["c3_qwen3_prefill", "c4_dsv3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode"])
 def test_full_size_properties_and_sampled_rows(K, orc, name):
-    import dataclasses
+    """The benchmark configurations at their full sizes (all 256 experts of the DeepSeek-V3 shapes, 4096 / 512 / 64
+    tokens), stage by stage."""
+    from _parity import layer_parity, staged_run
 
-    if name == "c4_dsv3_reduced":
-        # DeepSeek-V3's real K and N (7168 / 2 x 2048) and its rows per expert (about 128), with 16 of the 256
-        # experts so that the weights fit a test (0.7 GB instead of 11 GB)
-        cfg = dataclasses.replace(CONFIGS["c4_dsv3_prefill"], name=name, T=256, E=16, n_group=4, topk_group=2,
-                                  shared=False)
-    elif name == "c5_w4a8_reduced":
-        # the W4A8 configuration's real K, N, group size and Zipf skew with 16 of its 256 experts
-        cfg = dataclasses.replace(CONFIGS["c5_w4a8_zipf"], name=name, E=16, n_group=4, topk_group=2)
-    else:
-        cfg = CONFIGS[name]
+    cfg = CONFIGS[name]
     print(f"full size {name}: T={cfg.T} E={cfg.E} H={cfg.H} I={cfg.I}", flush=True)
-    d, r = _run_full(K, orc, cfg)
+    dg, dc = _make(cfg)
+    print("  tensors ready", flush=True)
+    r = staged_run(K, cfg, dg)
+    print("  GPU pass done", flush=True)
     R = cfg.T * cfg.k
     ids = r["ids"].cpu().numpy()
     dst = r["dst"].cpu().numpy().astype(np.int64)
@@ -117,42 +77,49 @@ def test_full_size_properties_and_sampled_rows(K, orc, name):
     assert bool((err <= sx[:, None] * 0.50001).all())
     del xf, err
 
-    # ---- sampled rows, bit for bit, through the checker (a miniature grouped problem with the same experts)
-    rng = np.random.default_rng(1)
-    rows = _sample_rows(cnt, rng)
-    e_rows = expert_of_row[rows]
-    cum_s = np.cumsum(np.bincount(e_rows, minlength=cfg.E)).astype(np.int64)
-    rows_t = torch.from_numpy(rows).to(DEV)
-    xs_s = xs[rows_t].cpu().numpy()
-    sx_s = sx[rows_t].cpu().numpy()
-    if cfg.w4_group >= 0:
-        sg13 = np.ascontiguousarray(d["s13"].numpy().transpose(0, 2, 1))
-        sg2 = np.ascontiguousarray(d["s2"].numpy().transpose(0, 2, 1))
-        f1 = orc.scale_rows(orc.gmm_w4_grouped(xs_s, d["w13"].numpy(), sg13, cum_s, cfg.w4_group), sx_s)
-        q_want, s_want = orc.swiglu_quant(f1)
-        o_want = orc.w4_rows_to_bf16(orc.gmm_w4_grouped(q_want, d["w2"].numpy(), sg2, cum_s, cfg.w4_group), s_want)
-    else:
-        acc1 = orc.gmm_i32(xs_s, d["w13"].numpy(), cum_s)
-        q_want, s_want = orc.swiglu_quant(orc.dequant_acc(acc1, sx_s, d["s13"].numpy(), cum_s))
-        o_want = orc.gmm2_dequant(orc.gmm_i32(q_want, d["w2"].numpy(), cum_s), s_want, d["s2"].numpy(), cum_s)
-    assert np.array_equal(r["q1"][rows_t].cpu().numpy(), q_want)
-    assert np.array_equal(r["s1"][rows_t].cpu().numpy().view(np.uint32), s_want.view(np.uint32))
-    assert np.array_equal(bits(r["o"][rows_t]), o_want)
+    # ---- every gate of the layer against the checker: routing, permutation and the first quantisation on the
+    # whole batch; int32 accumulators, int8 SwiGLU output, expert output and the combine on sampled rows / tokens
+    p = layer_parity(orc, cfg, dc, r, n_tokens=12)
+    print(f"  parity {p}", flush=True)
+    assert not p["failed"], p
+    assert p["rel_err_vs_fp32_dequant_reference"] <= 5e-2
+    if "rel_err_vs_quantized_fp64_reference" in p:
+        assert p["rel_err_vs_quantized_fp64_reference"] <= 1e-2
 
-    # ---- combine: sampled tokens recomputed from their k expert rows; linear in the routing weights
-    toks = np.unique(rng.integers(0, cfg.T, size=48))
-    o_cpu = {}
-    for t in toks:
-        rr = dst[t * cfg.k:(t + 1) * cfg.k]
-        o_cpu[t] = bits(r["o"][torch.from_numpy(rr).to(DEV)])
-    w_bits = bits(r["w"])
-    for t in toks:
-        want = orc.unpermute(o_cpu[t], np.arange(cfg.k, dtype=np.int32), w_bits[t:t + 1])
-        assert np.array_equal(bits(r["out"][int(t):int(t) + 1]), want)
+    # ---- the combine is linear in the routing weights
     out2 = K.token_unpermute(r["o"], r["dst"], (r["w"].float() * 2).to(torch.bfloat16))
     assert torch.equal(out2.float(), r["out"].float() * 2)
 
     # ---- a second run gives the same bits
-    _, r2 = _run_full(K, orc, cfg)
+    r2 = staged_run(K, cfg, dg, want_acc=False)
     for key in ("dst", "xs", "q1", "s1", "o", "out"):
         assert torch.equal(r[key], r2[key]), key
+
+
+@pytest.mark.parametrize("name", ["c4_dsv3_prefill", "c6_dsv3_decode"])
+def test_full_size_layer_with_shared_expert(K, orc, name):
+    """The DeepSeek-V3-shaped layer at full size through the plugin interface, with its shared expert on the main
+    stream and on the side stream: histogram on the whole batch, final output of sampled tokens recomputed by the
+    checker (routed rows, shared expert and the fused add)."""
+    from _layer_utils import build_layer
+    from _parity import layer_parity, staged_run
+
+    cfg = CONFIGS[name]
+    print(f"full size layer {name} with shared expert", flush=True)
+    dg, dc = _make(cfg)
+    r = staged_run(K, cfg, dg, want_acc=False)
+    layer = build_layer(cfg, dg, DEV, shared=True, overlap=False)
+    print("  layer built", flush=True)
+    outs = {}
+    for overlap in (False, True):
+        layer.shared_experts.multistream_overlap = overlap
+        for _ in range(2):
+            res = layer.forward_impl(dg["x"], dg["logits"])
+        torch.cuda.synchronize()
+        outs[overlap] = res.routed_out
+        assert torch.equal(res.expert_tokens, r["cnt"])
+        p = layer_parity(orc, cfg, dc, r, n_tokens=6, layer_out=res.routed_out, shared=True, full_dispatch=False)
+        print(f"  overlap={overlap} parity {p}", flush=True)
+        assert not p["failed"], p
+        assert p["rel_err_vs_fp32_dequant_reference"] <= 5e-2
+    assert torch.equal(outs[False], outs[True])

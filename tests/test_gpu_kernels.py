@@ -100,6 +100,57 @@ def test_init_routing(K, orc, T, k, E, H, quant):
     assert np.array_equal(cum.cpu().numpy(), np.cumsum(co))
 
 
+@pytest.mark.parametrize("T,k,E,H", [(60, 4, 16, 64), (900, 6, 100, 64), (3, 2, 8, 128)])
+@pytest.mark.parametrize("quant", [True, False])
+def test_init_routing_drops_out_of_range_experts(K, orc, T, k, E, H, quant):
+    """Ids outside [0, E) take no row; their destination is one past the last row, which the combine skips (both the
+    single-launch and the chunked form)."""
+    print(f"init_routing with dropped pairs T={T} k={k} E={E} quant={quant}", flush=True)
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    bad = torch.rand(T, k, generator=g) < 0.15
+    bad[0, 0] = True
+    ids[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, E + 3, -2).to(torch.int32)
+    R = T * k
+    xs = torch.zeros(R, H, dtype=torch.int8 if quant else torch.bfloat16, device=DEV)
+    xs_got, dst, cnt, sx = K.init_routing(x.to(DEV), ids.to(DEV), E, 1 if quant else -1, 1)
+    torch.cuda.synchronize()
+    xo, do, co, so = orc.init_routing(bits(x), ids.numpy(), E, quant=quant)
+    valid = int(co.sum())
+    assert valid < R and np.all(do[bad.reshape(-1).numpy()] == R)
+    assert np.array_equal(dst.cpu().numpy(), do)
+    assert np.array_equal(cnt.cpu().numpy(), co)
+    assert np.array_equal(bits(xs_got[:valid]), xo[:valid])      # rows past the last valid pair are not written
+    if quant:
+        assert np.array_equal(sx[:valid].cpu().numpy().view(np.uint32), so[:valid].view(np.uint32))
+    # the combine leaves the dropped pairs out (k rows of bf16 expert outputs per token, weights all non-zero)
+    o = torch.randn(R, H, generator=g).to(torch.bfloat16)
+    p = (torch.rand(T, k, generator=g) + 0.5).to(torch.bfloat16)
+    out = K.token_unpermute(o.to(DEV), dst, p.to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out), orc.unpermute(bits(o), do, bits(p)))
+    # ... also when the caller has taken abs() of the indices first, as the reference's caller does
+    out_abs = K.token_unpermute(o.to(DEV), dst.abs(), p.to(DEV))
+    assert torch.equal(out_abs, out)
+
+
+@pytest.mark.parametrize("T,k,E,H", [(64, 8, 128, 2048), (700, 8, 256, 512), (1, 1, 8, 64)])
+def test_init_routing_of_prequantised_activations(K, orc, T, k, E, H):
+    """int8 rows with their per-token scales are only moved: the result is what the quantising gather produces
+    from the unquantised rows (the identity the checker's tests pin on the CPU)."""
+    g = torch.Generator().manual_seed(T + E + 5)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    xq, s = K.dynamic_quant(x.to(DEV))
+    xs, dst, cnt, sx = K.init_routing_prequant(xq, s, ids.to(DEV), E, 1)
+    torch.cuda.synchronize()
+    xo, do, co, so = orc.init_routing(bits(x), ids.numpy(), E, quant=True)
+    assert np.array_equal(dst.cpu().numpy(), do) and np.array_equal(cnt.cpu().numpy(), co)
+    assert np.array_equal(xs.cpu().numpy(), xo)
+    assert np.array_equal(sx.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
 def test_init_routing_known_answer(K):
     """Permutation known-answer vector of the reference (tests/ut/lora/test_lora.py:151-165)."""
     ids = torch.tensor([[1, 0], [0, 1], [1, 1]], dtype=torch.int32)
@@ -124,7 +175,11 @@ GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100
              (1, 4, 32, 64), (300, 3, 7168, 256), (2100, 8, 256, 256), (3000, 4, 768, 2048),
              (1000, 16, 2048, 1536), (700, 2, 128, 320), (900, 3, 96, 192), (4100, 16, 512, 4096),
              # long rows of the SwiGLU re-quantisation: 2112 values (held in registers), 4160 (two passes)
-             (40, 4, 64, 4224), (24, 2, 64, 8320)]
+             (40, 4, 64, 4224), (24, 2, 64, 8320),
+             # many experts (a lane of the tile map / a thread of the scans owns more than one expert from 257
+             # on): weight streaming, 128-row tiles and the weight-streaming tiles, each with 256 and with more
+             (2000, 256, 128, 128), (1500, 320, 64, 64), (16000, 256, 128, 256), (20000, 320, 192, 128),
+             (32000, 256, 1024, 128), (40000, 320, 1024, 64)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)

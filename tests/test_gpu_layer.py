@@ -129,6 +129,81 @@ def test_layer_with_shared_expert(overlap):
     assert np.array_equal(bits(res.routed_out), tr.out)
 
 
+def test_layer_with_prequantised_hidden_states():
+    """ascend_pertoken_scale + int8 hidden states (vllm_ascend/ops/fused_moe/moe_mlp.py:226-242,
+    token_dispatcher.py:399-435): the dispatcher moves rows and scales, the MLP does not quantise again.  Handing
+    the layer the quantiser's own output must give the bits of the ordinary path."""
+    from vllm_ascend_amd import kernels as K
+
+    for name in ("c2_small", "c4_small"):
+        cfg = CONFIGS[name]
+        d = make_layer(cfg, seed=0)
+        layer = build_layer(cfg, d, DEV)
+        x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+        xq, s = K.dynamic_quant(x)
+        layer.ascend_pertoken_scale = s
+        res = layer.forward_impl(xq, logits)
+        torch.cuda.synchronize()
+        layer.ascend_pertoken_scale = None
+        tr = oracle_layer(cfg, d, keep_acc=False)
+        assert res.routed_out.dtype == torch.bfloat16
+        assert np.array_equal(bits(res.routed_out), tr.out), name
+        with pytest.raises(ValueError, match="int8 hidden states"):
+            layer.ascend_pertoken_scale = s
+            try:
+                layer.forward_impl(x, logits)
+            finally:
+                layer.ascend_pertoken_scale = None
+
+
+def test_apply_router_weight_on_input():
+    """top-1 routing with the weight applied to the expert's INPUT (token_dispatcher.py:409-413):
+    x' = x * w in the model dtype before the dispatch; the combine still multiplies by w, as the reference's
+    does (the metadata keeps topk_weights).  Checked against the checker fed with x'."""
+    import dataclasses
+
+    from oracle import oracle as orc
+
+    cfg = dataclasses.replace(CONFIGS["c2_small"], name="top1", k=1, renorm=0)
+    d = make_layer(cfg, seed=3)
+    layer = build_layer(cfg, d, DEV)
+    layer.apply_router_weight_on_input = True
+    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+    res = layer.forward_impl(x, logits)
+    torch.cuda.synchronize()
+    kw = dict(k_group=1, group_count=1, group_select_mode=1, renorm=0, norm_type=0, routed_scaling_factor=1.0)
+    y, ids, _ = orc.gating_top_k(d["logits"].numpy(), 1, x_dtype="f32", **kw)
+    w_bf16 = orc.f32_to_bf16(y)
+    # bf16 * bf16 -> bf16 on the GPU (torch): one fp32 product, one rounding
+    x_scaled = orc.f32_to_bf16(orc.bf16_to_f32(bits(d["x"])) * orc.bf16_to_f32(w_bf16))
+    tr = orc.experts_forward(x_scaled, w_bf16, ids, d["w13"].numpy(), d["s13"].numpy(), d["w2"].numpy(),
+                             d["s2"].numpy(), keep_acc=False)
+    assert np.array_equal(bits(res.routed_out), tr.out)
+    layer.apply_router_weight_on_input = False
+    res_plain = layer.forward_impl(x, logits)
+    assert not torch.equal(res_plain.routed_out, res.routed_out)
+    # top-k > 1 is refused, as in the reference
+    cfg2 = CONFIGS["c2_small"]
+    d2 = make_layer(cfg2, seed=0)
+    layer2 = build_layer(cfg2, d2, DEV)
+    layer2.apply_router_weight_on_input = True
+    with pytest.raises(AssertionError, match="topk=1"):
+        layer2.forward_impl(d2["x"].to(DEV), d2["logits"].to(DEV))
+
+
+def test_force_load_balance_routes_every_token_to_k_distinct_experts():
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV)
+    layer.enable_force_load_balance = True
+    res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
+    torch.cuda.synchronize()
+    assert int(res.expert_tokens.sum()) == cfg.T * cfg.k
+    assert torch.isfinite(res.routed_out.float()).all()
+    w, ids = layer.router.select_experts(d["x"].to(DEV), d["logits"].to(DEV), enable_force_load_balance=True)
+    assert all(len(set(r)) == cfg.k for r in ids.cpu().tolist())
+
+
 def test_layer_with_per_expert_weight_lists():
     """dynamic-EPLB form: every expert's weights and scales are separate tensors; swapping two experts'
     tensors in place must swap what they compute."""

@@ -32,6 +32,8 @@ PROTOTYPES = {
     "moe355_init_routing_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "moe355_init_routing": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "moe355_init_routing_prequant": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_int, c_int,
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe355_init_routing_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int, c_int, c_int,
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe355_format_cast_nz": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
@@ -58,6 +60,7 @@ PROTOTYPES = {
     "moe355_dequant_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p,
                                             c_void_p, c_void_p]),
     "moe355_profile_next_gemm": (c_int, [c_void_p, c_void_p]),
+    "moe355_gmm_kernel_name": (c_char_p, [c_int, c_int64, c_int64, c_int64, c_int]),
     "moe355_token_unpermute": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p,
                                        c_void_p, c_void_p]),
 }

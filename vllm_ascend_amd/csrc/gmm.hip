@@ -306,13 +306,14 @@ static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs
 // weight-streaming tiles (up to 256 rows) that fetch an expert's weights once.
 static int tiled_bm(const GmmArgs& a)
 {
-    // development knob: 's' stream, 't' 128-row tiles, 'T' 256-row weight-streaming tiles, 'u' 64-row tiles
-    static const char* force = getenv("MOE355_GEMM");
     if (a.K % 64 != 0) return 0;
+#ifdef MOE355_DEV_KNOBS  // experiments only (never defined for the shipped library): force one kernel family
+    static const char* force = getenv("MOE355_GEMM");
     if (force && force[0] == 's') return 0;
     if (force && force[0] == 't') return 128;
     if (force && force[0] == 'T') return 256;
     if (force && force[0] == 'u') return 64;
+#endif
     const int64_t avg = a.R / a.E;
     if (avg < 48) return 0;
     if (avg <= 256 && a.K >= 4096) return 256;
@@ -358,6 +359,20 @@ extern "C" int moe355_profile_next_gemm(void* start_event, void* stop_event)
     t_ev_start = (hipEvent_t)start_event;
     t_ev_stop = (hipEvent_t)stop_event;
     return MOE355_OK;
+}
+
+extern "C" const char* moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_t k, int64_t n, int num_experts)
+{
+    if (rows <= 0 || k <= 0 || n <= 0 || num_experts <= 0 || epilogue < 0 || epilogue > 2) return "";
+    GmmArgs a = {};
+    a.R = rows;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    const int bm = tiled_bm(a);
+    if (bm == 256) return "gmm_wide_kernel";
+    if (bm != 0) return "gmm_tiled_kernel";
+    return "gmm_stream_kernel";
 }
 
 extern "C" int moe355_format_cast_nz(const int8_t* w, int layout, int64_t num_experts, int64_t n, int64_t k,

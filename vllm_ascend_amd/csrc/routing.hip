@@ -149,7 +149,7 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
             start = __shfl(start, leader, 64);
             dst[f] = start + rank;
         } else if (f < R) {
-            dst[f] = -1;
+            dst[f] = (int32_t)R;  // dropped pair: one past the last row
         }
         __syncthreads();
     }
@@ -196,7 +196,7 @@ __device__ __forceinline__ void small_hist_scan(const int32_t* __restrict__ ids,
     }
 }
 
-// The token's row to its k destinations drow[0..k) (LDS, written before the call; -1 = dropped), quantised
+// The token's row to its k destinations drow[0..k) (LDS, written before the call; negative = dropped), quantised
 // per row when QUANT.  DT: bf16 or fp16 rows (the copy without quantisation moves 16-bit patterns).
 // held: the thread's first 16-byte piece of the row (first_piece()), requested by the caller before it worked
 // out the destinations; rows of up to 2048 values are then read from memory once.
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* 
         const int ej = ids[t * top_k + tid];
         const bool valid = ej >= 0 && ej < E;
         const int d = valid ? wsum[0][tid] + wsum[1][tid] + wsum[2][tid] + wsum[3][tid] : -1;
-        dst[t * top_k + tid] = d;
+        dst[t * top_k + tid] = valid ? d : R;  // a dropped pair points one past the last row
         drow[tid] = d;
     }
     gather_token_row<QUANT, DT>(x + (int64_t)t * H, H, top_k, drow, lds4, xs, sx, held);
@@ -323,8 +323,22 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __rest
     __shared__ int32_t drow[64];
     const int64_t t = blockIdx.x;
     const v8u16 held = first_piece(x + t * H, H);
-    if (threadIdx.x < top_k) drow[threadIdx.x] = dst[t * top_k + threadIdx.x];
+    if (threadIdx.x < top_k) {
+        const int32_t d = dst[t * top_k + threadIdx.x];
+        drow[threadIdx.x] = (int64_t)d < (int64_t)gridDim.x * top_k ? d : -1;  // R = tokens * top_k: dropped
+    }
     gather_token_row<QUANT, DT>(x + t * H, H, top_k, drow, lds4, xs, sx, held);
+}
+
+// expanded_scale[dst[f]] = scale[f / top_k] for every pair that has a row
+__global__ __launch_bounds__(256) void gather_scale_kernel(const int32_t* __restrict__ dst,
+                                                           const float* __restrict__ scale, int64_t R, int top_k,
+                                                           float* __restrict__ expanded_scale)
+{
+    const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (f >= R) return;
+    const int32_t d = dst[f];
+    if (d >= 0 && (int64_t)d < R) expanded_scale[d] = scale[f / top_k];
 }
 
 }  // namespace moe355
@@ -421,6 +435,25 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     return init_routing_impl(x, x_dtype, num_tokens, hidden, expert_idx, top_k, num_experts, quant_mode,
                              tokens_num_type, expanded_x, expanded_row_idx, expert_tokens, dynamic_scale, workspace,
                              workspace_bytes, stream);
+}
+
+extern "C" int moe355_init_routing_prequant(const int8_t* x, const float* x_scale, int64_t num_tokens, int64_t hidden,
+                                            const int32_t* expert_idx, int top_k, int num_experts,
+                                            int tokens_num_type, int8_t* expanded_x, int32_t* expanded_row_idx,
+                                            int64_t* expert_tokens, float* expanded_scale, void* workspace,
+                                            size_t workspace_bytes, void* stream)
+{
+    if (hidden <= 0 || hidden % 16 != 0) return hidden <= 0 ? MOE355_E_ARG : MOE355_E_SHAPE;
+    const int64_t R = num_tokens * (int64_t)top_k;
+    if (R > 0 && (!x_scale || !expanded_scale)) return MOE355_E_ARG;
+    // an int8 row of `hidden` bytes moves as hidden / 2 16-bit patterns through the copy form of the gather
+    const int rc = init_routing_impl(x, MOE355_DT_BF16, num_tokens, hidden / 2, expert_idx, top_k, num_experts, -1,
+                                     tokens_num_type, expanded_x, expanded_row_idx, expert_tokens, nullptr, workspace,
+                                     workspace_bytes, stream);
+    if (rc != MOE355_OK || R == 0) return rc;
+    hipLaunchKernelGGL(gather_scale_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       expanded_row_idx, x_scale, R, top_k, expanded_scale);
+    return launch_status();
 }
 
 // ------------------------------------------------------------------ the form that allocates nothing

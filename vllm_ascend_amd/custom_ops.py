@@ -172,11 +172,15 @@ def _gmm_swiglu_quant_v2(x, weight, weight_scale, x_scale, group_list, smooth_sc
         raise RuntimeError("grouped_matmul_swiglu_quant_v2: weight holds a different number of int4 values than K*N")
     eff_bias = None
     if weight_assist_matrix is not None:
-        key = (w.data_ptr(), s.data_ptr(), group)
+        # keyed on the caller's tensors and their version counters: an in-place swap of an expert's weights or
+        # scales bumps the counter, so a stale correction is never reused (the decoded scale `s` may be a
+        # temporary whose address means nothing)
+        ws0 = weight_scale[0]
+        key = (w.data_ptr(), w._version, ws0.data_ptr(), ws0._version, group)
         corr = _W4_CORR.get(key)
         if corr is None:
             if len(_W4_CORR) > 16:
-                _W4_CORR.clear()
+                _W4_CORR.clear()  # safe: a correction is consumed inside the call that looks it up
             corr = kernels.w4_offset_correction(w_bytes, s, group, n, k)
             _W4_CORR[key] = corr
         eff_bias = (weight_assist_matrix[0].to(torch.float32).reshape(e, n) - corr).contiguous()

@@ -63,6 +63,9 @@ class MI355XDeviceAdaptor:
             from . import custom_ops, kernels
 
             custom_ops._reject_unsupported(bias, None)
+            if weight_scale.dtype != torch.float32 or weight_scale.dim() != 2:
+                # the reference keeps scales in the model dtype and as [E, N, 1]: same conversion as the operator path
+                weight_scale = weight_scale.to(torch.float32).reshape(weight.shape[0], -1)
             out, out_scale = kernels.gmm1_swiglu_quant(x, weight, weight_scale, x_scale, group_list, 1,
                                                        weight.shape[2], weight.shape[1], swiglu_limit)
             return out, out_scale, None

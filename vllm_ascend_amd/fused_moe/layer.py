@@ -31,6 +31,7 @@ class AscendRoutedExperts(torch.nn.Module):
         self.global_redundant_expert_num = 0
         self.ascend_mc2_mask = None
         self.ascend_pertoken_scale = None
+        self.enable_force_load_balance = False  # profile runs only (routed_experts.py:484-492)
         specs = dict(quant_method.get_weight(moe_config.num_experts, moe_config.intermediate_size_per_partition,
                                              moe_config.hidden_dim, params_dtype))
         specs.update(quant_method.get_dynamic_quant_param(moe_config.num_experts,
@@ -52,7 +53,14 @@ class AscendRoutedExperts(torch.nn.Module):
 
     def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
         hidden_states, router_logits, _, _ = self.moe_comm_method.prepare(hidden_states, router_logits)
-        topk_weights, topk_ids = self.router.select_experts(hidden_states, router_logits)
+        # int8 hidden states = activations the caller quantised (their scales in ascend_pertoken_scale): the
+        # routing weights then take the model dtype of the scheme
+        weights_dtype = None
+        if hidden_states.dtype == torch.int8:
+            weights_dtype = getattr(self.quant_method, "in_dtype", torch.bfloat16)
+        topk_weights, topk_ids = self.router.select_experts(
+            hidden_states, router_logits, enable_force_load_balance=self.enable_force_load_balance,
+            weights_dtype=weights_dtype)
         result = self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
         result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
         return result

@@ -69,12 +69,23 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
 
     if dynamic_eplb or (isinstance(w1, (list, tuple)) and len(w1) > 1):
         # per-expert weight lists (the form dynamic expert load balancing swaps in place)
-        hidden_states, swiglu_out_scale, _ = torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz_tensor_list(
-            x=hidden_states, weight=list(w1), weight_scale=list(w1_scale), x_scale=pertoken_scale,
-            group_list=cumsum_group_list(group_list, group_list_type, 0), bias=None, swiglu_limit=swiglu_limit)
+        from ..kernels import ExpertTensorList, gmm1_swiglu_quant_list
+
+        if isinstance(w1, ExpertTensorList) and isinstance(w1_scale, ExpertTensorList) and group_list_type in (0, 1):
+            # the layer's own lists: their address tables were built at load time and are reused (a Tensor[]
+            # argument of a torch operator arrives as a plain list and would need a table of its own per call)
+            hidden_states, swiglu_out_scale = gmm1_swiglu_quant_list(hidden_states, w1, w1_scale, pertoken_scale,
+                                                                     group_list, group_list_type, swiglu_limit)
+        else:
+            hidden_states, swiglu_out_scale, _ = (
+                torch.ops._C_ascend.grouped_matmul_swiglu_quant_weight_nz_tensor_list(
+                    x=hidden_states, weight=list(w1), weight_scale=list(w1_scale), x_scale=pertoken_scale,
+                    group_list=cumsum_group_list(group_list, group_list_type, 0), bias=None,
+                    swiglu_limit=swiglu_limit))
         before_gmm2_evt = torch.cuda.current_stream().record_event() if hidden_states.is_cuda else None
         out = DeviceOperator.npu_grouped_matmul_gmm2(
-            hidden_states=hidden_states, weight=list(w2), weight_scale=list(w2_scale),
+            hidden_states=hidden_states, weight=w2 if isinstance(w2, ExpertTensorList) else list(w2),
+            weight_scale=w2_scale if isinstance(w2_scale, ExpertTensorList) else list(w2_scale),
             per_token_scale=swiglu_out_scale, group_list=group_list, group_list_type=group_list_type,
             input_dtype=input_dtype)
         return out, before_gmm2_evt

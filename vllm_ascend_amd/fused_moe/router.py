@@ -25,12 +25,21 @@ class AscendFusedTopKRouter:
         self.e_score_correction_bias = e_score_correction_bias
 
     def select_experts(self, hidden_states: torch.Tensor, router_logits: torch.Tensor,
-                       indices_type: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+                       indices_type: torch.dtype | None = None, enable_force_load_balance: bool = False,
+                       weights_dtype: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
         """-> (topk_weights in the hidden-state dtype, topk_ids int32)
-        (``vllm_ascend/ops/fused_moe/routed_experts.py:438-494``)."""
+        (``vllm_ascend/ops/fused_moe/routed_experts.py:438-494``).  ``enable_force_load_balance`` (profile runs
+        only, ``routed_experts.py:484-492``): the ids are replaced by the first k entries of a random
+        permutation of the experts per token, so that no expert collects the whole dummy batch; the weights
+        stay.  ``weights_dtype``: dtype of the returned weights when the hidden states are int8 (pre-quantised)."""
+        if weights_dtype is None:
+            weights_dtype = hidden_states.dtype
         topk_weights, topk_ids = self._compute_routing(hidden_states, router_logits, indices_type,
-                                                       weights_dtype=hidden_states.dtype)
-        return topk_weights.to(hidden_states.dtype), topk_ids
+                                                       weights_dtype=weights_dtype)
+        if enable_force_load_balance:
+            random_matrix = torch.rand(topk_ids.size(0), self.global_num_experts, device=topk_ids.device)
+            topk_ids = torch.argsort(random_matrix, dim=1)[:, : topk_ids.size(1)].to(topk_ids.dtype)
+        return topk_weights.to(weights_dtype), topk_ids
 
     def _compute_routing(self, hidden_states, router_logits, indices_type=None, weights_dtype=None):
         bias = self.e_score_correction_bias

@@ -41,9 +41,11 @@ class TokenDispatcherWithAllGather:
         with_quant = tdi.quant.dispatch_with_quant
         # the first quantisation of the MLP is folded into the gather unless the caller
         # already quantised the activations (then hidden_states is int8 and only moves)
+        # (pertoken_scale given: quant_mode -1 and the scale travels with the rows, token_dispatcher.py:399-435)
         quant_mode = 1 if (with_quant and dynamic_scale is None) else -1
-        if dynamic_scale is not None:
-            raise NotImplementedError("pre-quantised activations (pertoken_scale) come from the EP prepare stage")
+        if dynamic_scale is not None and hidden_states.dtype != torch.int8:
+            raise ValueError("pertoken_scale goes with int8 hidden states (activations quantised by the caller), "
+                             f"got {hidden_states.dtype}")
         restore_shape = hidden_states.shape
         num_tokens = hidden_states.shape[:-1].numel()
         if routing.apply_router_weight_on_input:
@@ -52,7 +54,7 @@ class TokenDispatcherWithAllGather:
             hidden_states = hidden_states * topk_weights.to(hidden_states.dtype)
 
         sorted_hidden_states, expanded_row_idx, expert_tokens, dynamic_scale = DeviceOperator.npu_moe_init_routing(
-            hidden_states, tdi.topk_ids, scale=None, active_num=num_tokens * self.top_k,
+            hidden_states, tdi.topk_ids, scale=dynamic_scale, active_num=num_tokens * self.top_k,
             expert_num=self.num_experts_local, expert_tokens_num_type=1, expert_tokens_num_flag=True,
             active_expert_range=[0, self.num_experts_local], quant_mode=quant_mode)
         return MoETokenDispatchOutput(

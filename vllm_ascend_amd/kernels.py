@@ -134,6 +134,36 @@ def init_routing(x, expert_idx, num_experts, quant_mode, tokens_num_type):
     return xs, row_idx, tokens, scale
 
 
+def init_routing_prequant(xq, x_scale, expert_idx, num_experts, tokens_num_type):
+    """int8 activations [T, H] with their fp32 per-token scales [T]: rows and scales are moved to the
+    expert-sorted order, nothing is quantised again.  -> (expanded_x int8 [R, H], expanded_row_idx, expert_tokens,
+    expanded_scale [R])."""
+    xq = _dev(xq, "x")
+    x_scale = _dev(x_scale, "scale")
+    expert_idx = _dev(expert_idx, "expert_idx")
+    if xq.dtype != torch.int8:
+        raise TypeError(f"x: pre-quantised activations must be int8, got {xq.dtype}")
+    if x_scale.dtype != torch.float32:
+        x_scale = x_scale.to(torch.float32)
+    if expert_idx.dtype != torch.int32:
+        expert_idx = expert_idx.to(torch.int32)
+    T, k = expert_idx.shape
+    H = xq.shape[-1]
+    if xq.numel() != T * H or x_scale.numel() != T:
+        raise ValueError(f"x {tuple(xq.shape)} / scale {tuple(x_scale.shape)} do not match {T} tokens")
+    lib = _lib.load()
+    R, dev = T * k, xq.device
+    xs = torch.empty((R, H), dtype=torch.int8, device=dev)
+    row_idx = torch.empty((R,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((num_experts,), dtype=torch.int64, device=dev)
+    scale = torch.empty((R,), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.moe355_init_routing_workspace(T, k, num_experts), dev)
+    check(lib.moe355_init_routing_prequant(_ptr(xq), _ptr(x_scale), T, H, _ptr(expert_idx), k, num_experts,
+                                           tokens_num_type, _ptr(xs), _ptr(row_idx), _ptr(tokens), _ptr(scale),
+                                           _ptr(ws), ws.numel(), _stream(xq)), "moe355_init_routing_prequant")
+    return xs, row_idx, tokens, scale
+
+
 def format_cast_nz(w: torch.Tensor, layout: int) -> torch.Tensor:
     """int8 [E, N, K] (layout W_ENK) or [E, K, N] (W_EKN) -> same shape, MFMA-tiled storage."""
     w = _dev(w, "weight")
@@ -160,13 +190,44 @@ def _gl(group_list: torch.Tensor) -> torch.Tensor:
     return group_list if group_list.dtype == torch.int64 else group_list.to(torch.int64)
 
 
+def _check_gmm_operands(op, x, rows, k, n, E, group_list, row_scale=None, row_scale_name="x_scale", weight=None,
+                        weight_numel=None, channel_scale=None, channel_scale_numel=None):
+    """Host-side argument checks of the grouped-GEMM launchers: the C ABI takes raw pointers, so a tensor of the
+    wrong dtype or length would be read out of bounds on the device instead of raising."""
+    if x.dtype != torch.int8:
+        raise TypeError(f"{op}: x must be int8, got {x.dtype}")
+    if x.dim() != 2 or x.shape[1] != k:
+        raise ValueError(f"{op}: x must be [rows, K = {k}], got {tuple(x.shape)}")
+    if group_list.dim() != 1 or group_list.numel() != E:
+        raise ValueError(f"{op}: group_list must hold one entry per expert ({E}), got {tuple(group_list.shape)}")
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32:
+            raise TypeError(f"{op}: {row_scale_name} must be float32, got {row_scale.dtype}")
+        if row_scale.numel() != rows:
+            raise ValueError(f"{op}: {row_scale_name} must hold one scale per row ({rows}), got {row_scale.numel()}")
+    if weight is not None:
+        if weight.dtype not in (torch.int8, torch.uint8):
+            raise TypeError(f"{op}: weight must be int8 tiled storage, got {weight.dtype}")
+        if weight.numel() != weight_numel:
+            raise ValueError(f"{op}: weight holds {weight.numel()} bytes, E x N x K needs {weight_numel}")
+    if channel_scale is not None:
+        if channel_scale.dtype != torch.float32:
+            raise TypeError(f"{op}: the weight scale must be float32, got {channel_scale.dtype} "
+                            "(convert once after loading)")
+        if channel_scale.numel() != channel_scale_numel:
+            raise ValueError(f"{op}: the weight scale holds {channel_scale.numel()} values, expected "
+                             f"{channel_scale_numel}")
+
+
 def gmm1_swiglu_quant(x, weight_nz, weight_scale, x_scale, group_list, group_list_type, n, k, swiglu_limit=0.0,
                       out=None, out_scale=None):
-    x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz.shape[0]
     dev = x.device
+    _check_gmm_operands("gmm1_swiglu_quant", x, rows, k, n, E, group_list, x_scale, "x_scale", weight_nz, E * n * k,
+                        weight_scale, E * n)
+    x = _dev(x, "x")
     if out is None:
         out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
     if out_scale is None:
@@ -181,10 +242,12 @@ def gmm1_swiglu_quant(x, weight_nz, weight_scale, x_scale, group_list, group_lis
 
 
 def gmm2_dequant(x, weight_nz, scale, per_token_scale, group_list, group_list_type, n, k, out_dtype=torch.bfloat16):
-    x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz.shape[0]
+    _check_gmm_operands("gmm2_dequant", x, rows, k, n, E, group_list, per_token_scale, "per_token_scale", weight_nz,
+                        E * n * k, scale, E * n)
+    x = _dev(x, "x")
     out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm2_dequant(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_dev(scale, "scale")),
@@ -196,10 +259,11 @@ def gmm2_dequant(x, weight_nz, scale, per_token_scale, group_list, group_list_ty
 
 def gmm_i32(x, weight_nz, group_list, group_list_type, n, k):
     """Raw int32 accumulators of the grouped product (rows outside every group are zero)."""
-    x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz.shape[0]
+    _check_gmm_operands("gmm_i32", x, rows, k, n, E, group_list, weight=weight_nz, weight_numel=E * n * k)
+    x = _dev(x, "x")
     acc = torch.zeros((rows, n), dtype=torch.int32, device=x.device)
     ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm_i32(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_gl(group_list)),
@@ -260,11 +324,16 @@ def format_cast_nz_int4(w: torch.Tensor, source: int, n: int, k: int) -> torch.T
 
 def gmm1_swiglu_quant_w4(x, weight_nz4, weight_scale, group_size, x_scale, group_list, group_list_type, n, k,
                          bias=None, swiglu_limit=0.0):
-    x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz4.shape[0]
     dev = x.device
+    groups = k // group_size if group_size else 1
+    _check_gmm_operands("gmm1_swiglu_quant_w4", x, rows, k, n, E, group_list, x_scale, "x_scale", weight_nz4,
+                        E * n * k // 2, weight_scale, E * groups * n)
+    x = _dev(x, "x")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != E * n or not bias.is_cuda):
+        raise ValueError(f"gmm1_swiglu_quant_w4: bias must be a float32 GPU tensor of E x N = {E * n} values")
     out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
     out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
     ws = _workspace(rows * (n // 2) * 4 + 256, dev)
@@ -279,10 +348,15 @@ def gmm1_swiglu_quant_w4(x, weight_nz4, weight_scale, group_size, x_scale, group
 
 def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_list, group_list_type, n, k, bias=None,
                     out_dtype=torch.bfloat16):
-    x = _dev(x, "x")
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz4.shape[0]
+    groups = k // group_size if group_size else 1
+    _check_gmm_operands("gmm2_dequant_w4", x, rows, k, n, E, group_list, per_token_scale, "per_token_scale",
+                        weight_nz4, E * n * k // 2, scale, E * groups * n)
+    x = _dev(x, "x")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != E * n or not bias.is_cuda):
+        raise ValueError(f"gmm2_dequant_w4: bias must be a float32 GPU tensor of E x N = {E * n} values")
     out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     check(lib.moe355_gmm2_dequant_w4(_ptr(x), _ptr(_dev(weight_nz4, "weight")), _ptr(_dev(scale, "scale")),
                                      group_size, _ptr(bias), _ptr(_dev(per_token_scale, "per_token_scale")),
@@ -292,39 +366,79 @@ def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_lis
 
 
 # ------------------------------------------------------------------ per-expert tensor lists
-_PTR_TABLES: dict = {}
+class ExpertTensorList(list):
+    """E per-expert tensors of one shape and dtype together with the device array of their addresses that the
+    ``*_list`` entry points of the library follow.  The table is built once, when the list is created (after
+    weight loading), and lives as long as the list: a HIP graph that captured a launch keeps reading the same
+    table.  Replacing an expert (``lst[e] = tensor``, what dynamic expert load balancing does when it cannot
+    copy in place) rewrites that one entry of the same table; copying into an expert's tensor in place needs
+    nothing."""
+
+    def __init__(self, tensors, name="weight", dtype=None):
+        super().__init__(tensors)
+        if len(self) == 0:
+            raise ValueError(f"{name}: an empty list of per-expert tensors")
+        self.name = name
+        dtype = dtype or self[0].dtype
+        for t in self:
+            self._check_one(t, dtype)
+        self.table = torch.tensor([t.data_ptr() for t in self], dtype=torch.int64, device=self[0].device)
+
+    def _check_one(self, t, dtype):
+        first = self[0]
+        if t.dtype != dtype or t.shape != first.shape or t.device != first.device or not t.is_contiguous():
+            raise RuntimeError(f"{self.name}: every per-expert tensor must be a contiguous {dtype} tensor of one "
+                               "shape on one device")
+
+    def __setitem__(self, e, tensor):
+        if not isinstance(e, int):
+            raise TypeError("per-expert tensors are replaced one at a time")
+        self._check_one(tensor, self[0].dtype)
+        super().__setitem__(e, tensor)
+        self.table[e] = tensor.data_ptr()  # same table, one entry rewritten
+
+    def _frozen(self, *a, **k):
+        raise TypeError("the number of experts of an ExpertTensorList is fixed")
+
+    append = extend = insert = pop = remove = clear = __delitem__ = __iadd__ = __imul__ = sort = reverse = _frozen
 
 
-def _ptr_table(tensors) -> torch.Tensor:
-    """Device array with the data pointers of ``tensors`` (cached per exact list of pointers)."""
-    key = tuple(t.data_ptr() for t in tensors)
-    tab = _PTR_TABLES.get(key)
-    if tab is None:
-        if len(_PTR_TABLES) > 64:
-            _PTR_TABLES.clear()
-        tab = torch.tensor(key, dtype=torch.int64, device=tensors[0].device)
-        _PTR_TABLES[key] = tab
-    return tab
+def _as_expert_list(tensors, name, dtype) -> ExpertTensorList:
+    """A plain list gets a table of its own for this one call (a synchronous host-to-device copy: not usable
+    under graph capture); layers hold ExpertTensorList objects, whose table is reused."""
+    if isinstance(tensors, ExpertTensorList):
+        if tensors[0].dtype != dtype:
+            raise RuntimeError(f"{name}: per-expert tensors must be {dtype}, got {tensors[0].dtype}")
+        return tensors
+    return ExpertTensorList(list(tensors), name, dtype)
 
 
-def _check_list(tensors, name, dtype):
-    for t in tensors:
-        if not t.is_cuda or not t.is_contiguous() or t.dtype != dtype or t.shape != tensors[0].shape:
-            raise RuntimeError(f"{name}: every per-expert tensor must be a contiguous {dtype} GPU tensor of one shape")
+def _check_list_operands(op, x, weights, scales, row_scale, row_scale_name, group_list):
+    if not weights[0].is_cuda or not scales[0].is_cuda:
+        raise RuntimeError(f"{op}: per-expert tensors must live on the GPU")
+    if len(weights) != len(scales):
+        raise ValueError(f"{op}: {len(weights)} weights but {len(scales)} scales")
+    if weights[0].dim() != 2:
+        raise ValueError(f"{op}: per-expert weights are [K, N] tiled tensors, got {tuple(weights[0].shape)}")
+    k, n = weights[0].shape
+    if scales[0].numel() != n:
+        raise ValueError(f"{op}: per-expert scales must hold N = {n} values, got {scales[0].numel()}")
+    _check_gmm_operands(op, x, x.shape[0], k, n, len(weights), group_list, row_scale, row_scale_name)
+    return k, n
 
 
 def gmm1_swiglu_quant_list(x, weight_list, scale_list, x_scale, group_list, group_list_type, swiglu_limit=0.0):
     """weight_list: E tiled int8 tensors of logical shape [K, N]; scale_list: E fp32 tensors [N]."""
     x = _dev(x, "x")
     lib = _lib.load()
-    _check_list(weight_list, "weight", torch.int8)
-    _check_list(scale_list, "weight_scale", torch.float32)
-    k, n = weight_list[0].shape
+    weight_list = _as_expert_list(weight_list, "weight", torch.int8)
+    scale_list = _as_expert_list(scale_list, "weight_scale", torch.float32)
+    k, n = _check_list_operands("gmm1_swiglu_quant_list", x, weight_list, scale_list, x_scale, "x_scale", group_list)
     rows, E, dev = x.shape[0], len(weight_list), x.device
     out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
     out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
     ws = _workspace(lib.moe355_gmm1_swiglu_quant_workspace(rows, n, k, E), dev)
-    check(lib.moe355_gmm1_swiglu_quant_list(_ptr(x), _ptr(_ptr_table(weight_list)), _ptr(_ptr_table(scale_list)),
+    check(lib.moe355_gmm1_swiglu_quant_list(_ptr(x), _ptr(weight_list.table), _ptr(scale_list.table),
                                             _ptr(_dev(x_scale, "x_scale")), _ptr(_gl(group_list)),
                                             _gl_type(group_list_type), rows, k, n, E, float(swiglu_limit), _ptr(out),
                                             _ptr(out_scale), _ptr(ws), ws.numel(), _stream(x)),
@@ -336,13 +450,14 @@ def gmm2_dequant_list(x, weight_list, scale_list, per_token_scale, group_list, g
                       out_dtype=torch.bfloat16):
     x = _dev(x, "x")
     lib = _lib.load()
-    _check_list(weight_list, "weight", torch.int8)
-    _check_list(scale_list, "scale", torch.float32)
-    k, n = weight_list[0].shape
+    weight_list = _as_expert_list(weight_list, "weight", torch.int8)
+    scale_list = _as_expert_list(scale_list, "scale", torch.float32)
+    k, n = _check_list_operands("gmm2_dequant_list", x, weight_list, scale_list, per_token_scale, "per_token_scale",
+                                group_list)
     rows, E = x.shape[0], len(weight_list)
     out = torch.empty((rows, n), dtype=_half_dtype(out_dtype), device=x.device)
     ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
-    check(lib.moe355_gmm2_dequant_list(_ptr(x), _ptr(_ptr_table(weight_list)), _ptr(_ptr_table(scale_list)),
+    check(lib.moe355_gmm2_dequant_list(_ptr(x), _ptr(weight_list.table), _ptr(scale_list.table),
                                        _ptr(_dev(per_token_scale, "per_token_scale")), _ptr(_gl(group_list)),
                                        _gl_type(group_list_type), rows, k, n, E, _ptr(out), _DT[out.dtype], _ptr(ws),
                                        ws.numel(), _stream(x)), "moe355_gmm2_dequant_list")

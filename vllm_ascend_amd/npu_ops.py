@@ -41,8 +41,11 @@ def npu_moe_init_routing_v2(x, expert_idx, *, scale=None, offset=None, active_nu
                             expert_num=-1, drop_pad_mode=0, expert_tokens_num_type=0, expert_tokens_num_flag=False,
                             quant_mode=-1, active_expert_range=None, row_idx_type=0):
     """-> (expanded_x, expanded_row_idx, expert_tokens, dynamic_scale)."""
-    if scale is not None or offset is not None:
-        raise NotImplementedError("npu_moe_init_routing_v2: smooth `scale`/`offset` inputs are not supported")
+    if offset is not None:
+        raise NotImplementedError("npu_moe_init_routing_v2: `offset` is not supported")
+    if scale is not None and not (quant_mode == -1 and x.dtype == torch.int8):
+        raise NotImplementedError("npu_moe_init_routing_v2: `scale` is only supported as the per-token scale of "
+                                  "int8 activations that are moved without re-quantisation (quant_mode=-1)")
     if drop_pad_mode != 0 or expert_capacity not in (-1, 0) or row_idx_type != 0:
         raise NotImplementedError("npu_moe_init_routing_v2: drop/pad mode is not supported")
     if quant_mode not in (-1, 1):
@@ -56,6 +59,13 @@ def npu_moe_init_routing_v2(x, expert_idx, *, scale=None, offset=None, active_nu
         raise NotImplementedError("npu_moe_init_routing_v2: a partial active_expert_range (expert parallelism) "
                                   "is not supported on one GPU")
     x2 = x.reshape(-1, x.shape[-1])
+    if x.dtype == torch.int8:
+        if scale is None or quant_mode != -1:
+            raise NotImplementedError("npu_moe_init_routing_v2: int8 activations need their per-token `scale` and "
+                                      "quant_mode=-1")
+        return kernels.init_routing_prequant(x2, scale.reshape(-1),
+                                             expert_idx.reshape(x2.shape[0], expert_idx.shape[-1]), expert_num,
+                                             expert_tokens_num_type)
     xs, row_idx, tokens, dyn = kernels.init_routing(x2, expert_idx.reshape(x2.shape[0], expert_idx.shape[-1]), expert_num, quant_mode,
                                                     expert_tokens_num_type)
     return xs, row_idx, tokens, dyn
@@ -80,8 +90,12 @@ def npu_grouped_matmul(x, weight, *, bias=None, scale=None, offset=None, antiqua
         # one tiled [K, N] weight and one [N] scale per expert
         if output_dtype not in (None, torch.bfloat16, torch.float16):
             raise NotImplementedError(f"npu_grouped_matmul: output_dtype {output_dtype} is not supported")
-        scales = [s_ if s_.dtype == torch.float32 else s_.to(torch.float32) for s_ in ss]
-        return [kernels.gmm2_dequant_list(xs[0], list(ws), scales, ps[0], group_list, group_list_type,
+        if isinstance(ws, kernels.ExpertTensorList) and isinstance(ss, kernels.ExpertTensorList):
+            weights, scales = ws, ss  # the layer's lists: address tables built at load time
+        else:
+            weights = list(ws)
+            scales = [s_ if s_.dtype == torch.float32 else s_.to(torch.float32) for s_ in ss]
+        return [kernels.gmm2_dequant_list(xs[0], weights, scales, ps[0], group_list, group_list_type,
                                           output_dtype or torch.bfloat16)]
     if len(xs) != 1 or len(ws) != 1 or len(ss) != 1 or len(ps) != 1 or ss[0] is None or ps[0] is None:
         raise NotImplementedError("npu_grouped_matmul: expects exactly one x, weight, scale and per_token_scale")
@@ -112,7 +126,9 @@ def _single_group_list(rows: int, device) -> torch.Tensor:
     key = (rows, str(device))
     t = _ONE_GROUP.get(key)
     if t is None:
-        t = torch.tensor([rows], dtype=torch.int64, device=device)
+        # a fill kernel on the current stream, not a host-to-device copy: no synchronisation, and legal while a
+        # HIP graph is being captured (the tensor is created on first use of a row count)
+        t = torch.full((1,), rows, dtype=torch.int64, device=device)
         _ONE_GROUP[key] = t
     return t
 

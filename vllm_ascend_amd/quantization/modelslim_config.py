@@ -37,45 +37,48 @@ packed_modules_model_mapping: dict[str, dict[str, list[str]]] = {
     "glm4_moe": {"qkv_proj": ["q_proj", "k_proj", "v_proj"], **_GATE_UP_EXPERTS},
 }
 
-_MOE_WEIGHT_LOADER_NAME_MAP = {
-    "w13_scale_bias": "w13_scale",
-    "w2_scale_bias": "w2_scale",
-}
+# ModelSlim stores the MoE scale-bias tensors under their own names; the stacked layer keeps them with the scales
+_SCALE_BIAS_SUFFIX = "_scale_bias"
 
 
 def _make_modelslim_moe_weight_loader(weight_loader: Callable[..., bool | None]) -> Callable[..., bool | None]:
-    """Map ModelSlim MoE scale-bias names to the scale path of the wrapped loader."""
+    """Wrap a fused-MoE ``weight_loader`` so that a tensor named ``<...>.w13_scale_bias`` / ``<...>.w2_scale_bias``
+    is loaded as ``<...>.w13_scale`` / ``<...>.w2_scale``; every other name passes through unchanged
+    (behaviour of ``vllm_ascend/quantization/modelslim_config.py:55-91``)."""
 
     @wraps(weight_loader)
-    def modelslim_moe_weight_loader(param, loaded_weight, weight_name: str, shard_id: str, expert_id: int,
-                                    return_success: bool = False) -> bool | None:
-        prefix, separator, param_name = weight_name.rpartition(".")
-        mapped_name = _MOE_WEIGHT_LOADER_NAME_MAP.get(param_name, param_name)
-        return weight_loader(param=param, loaded_weight=loaded_weight,
-                             weight_name=f"{prefix}{separator}{mapped_name}", shard_id=shard_id,
+    def load(param, loaded_weight, weight_name: str, shard_id: str, expert_id: int, return_success: bool = False):
+        leaf = weight_name.rsplit(".", 1)[-1]
+        if leaf in ("w13" + _SCALE_BIAS_SUFFIX, "w2" + _SCALE_BIAS_SUFFIX):
+            weight_name = weight_name[: -len("_bias")]
+        return weight_loader(param=param, loaded_weight=loaded_weight, weight_name=weight_name, shard_id=shard_id,
                              expert_id=expert_id, return_success=return_success)
 
-    return modelslim_moe_weight_loader
+    return load
+
+
+def _shard_keys(prefix: str, packed_modules_mapping: Mapping[str, list[str]]) -> list[str]:
+    """Description keys (``<module>.weight``) that make up the layer at ``prefix``: one per checkpoint module when
+    the layer's last name component is a fused module, the layer's own key otherwise."""
+    fused_name = prefix.rsplit(".", 1)[-1]
+    parts = packed_modules_mapping.get(fused_name)
+    if parts is None:
+        return [prefix + ".weight"]
+    return [prefix.replace(fused_name, part) + ".weight" for part in parts]
 
 
 def get_linear_quant_type(quant_description: dict[str, Any], prefix: str,
                           packed_modules_mapping: Mapping[str, list[str]]) -> str | None:
     """Quant type of a (possibly packed) layer; every shard of a packed layer must agree.  A shard that the
-    description does not list raises ``KeyError``, as the reference does."""
-    proj_name = prefix.split(".")[-1]
-    if proj_name in packed_modules_mapping:
-        quant_type = None
-        for shard_proj_name in packed_modules_mapping[proj_name]:
-            shard_quant_type = quant_description[prefix.replace(proj_name, shard_proj_name) + ".weight"]
-            if quant_type is None:
-                quant_type = shard_quant_type
-            elif shard_quant_type != quant_type:
-                raise ValueError(
-                    f"Not all shards of {prefix} are quantized with same quant type. "
-                    f"Shard {proj_name} uses {shard_quant_type}, but another shard "
-                    f"uses {quant_type}. Please check quantization config.")
-        return quant_type
-    return quant_description[prefix + ".weight"]
+    description does not list raises ``KeyError``, as the reference does
+    (``vllm_ascend/quantization/modelslim_config.py:431-470``)."""
+    keys = _shard_keys(prefix, packed_modules_mapping)
+    kinds = [quant_description[key] for key in keys]
+    for key, kind in zip(keys, kinds):
+        if kind != kinds[0]:
+            raise ValueError(f"Not all shards of {prefix} are quantized with same quant type: {keys[0]} is "
+                             f"{kinds[0]} but {key} is {kind}. Please check quantization config.")
+    return kinds[0] if kinds else None
 
 
 def get_quant_type_for_layer(quant_description: dict[str, Any], prefix: str, layer_type: str,
@@ -137,24 +140,17 @@ class AscendModelSlimConfig:
 
     def is_layer_skipped_ascend(self, prefix: str,
                                 fused_mapping: Mapping[str, list[str]] = MappingProxyType({})) -> bool:
-        """True when the layer's weights are stored as FLOAT (not quantised)."""
-        proj_name = prefix.split(".")[-1]
-        if proj_name in fused_mapping:
-            is_skipped = None
-            for shard_proj_name in fused_mapping[proj_name]:
-                shard_key = prefix.replace(proj_name, shard_proj_name) + ".weight"
-                is_shard_skipped = self.quant_description[shard_key] == "FLOAT"
-                if is_skipped is None:
-                    is_skipped = is_shard_skipped
-                elif is_shard_skipped != is_skipped:
-                    raise ValueError(
-                        f"Detected some but not all shards of {prefix} are quantized. All shards of fused "
-                        "layers to have the same precision.")
-        else:
-            is_skipped = any(key.startswith(prefix) and key.endswith(".weight") and value == "FLOAT"
-                             for key, value in self.quant_description.items())
-        assert is_skipped is not None
-        return is_skipped
+        """True when the layer's weights are stored as FLOAT (not quantised).  A fused layer must be FLOAT in all
+        of its shards or in none (``vllm_ascend/quantization/modelslim_config.py:776-808``); a plain prefix counts
+        as skipped when any ``.weight`` entry below it is FLOAT."""
+        if prefix.rsplit(".", 1)[-1] in fused_mapping:
+            floats = [self.quant_description[key] == "FLOAT" for key in _shard_keys(prefix, fused_mapping)]
+            if any(floats) != all(floats):
+                raise ValueError(f"Detected some but not all shards of {prefix} are quantized. All shards of fused "
+                                 "layers to have the same precision.")
+            return all(floats)
+        return any(kind == "FLOAT" for key, kind in self.quant_description.items()
+                   if key.startswith(prefix) and key.endswith(".weight"))
 
     def get_moe_scheme(self, prefix: str, model_type: str = "qwen3_moe", **scheme_kwargs):
         """Scheme for the fused-MoE layer at ``prefix`` (e.g. ``model.layers.3.mlp.experts``): the MoE branch of

@@ -63,10 +63,18 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         layer.w13_weight_scale_fp32 = layer.w13_weight_scale.data.to(torch.float32)
         layer.w2_weight_scale_fp32 = layer.w2_weight_scale.data.to(torch.float32)
         if self.use_expert_weight_list:
-            layer.w13_weight_list = [w.clone() for w in layer.w13_weight.data.unbind(dim=0)]
-            layer.w2_weight_list = [w.clone() for w in layer.w2_weight.data.unbind(dim=0)]
-            layer.w13_weight_scale_fp32_list = [s.clone() for s in layer.w13_weight_scale_fp32.unbind(dim=0)]
-            layer.w2_weight_scale_list = [s.clone() for s in layer.w2_weight_scale_fp32.unbind(dim=0)]
+            # each list carries the device table of its tensors' addresses, built here once; swapping an expert
+            # (lst[e] = tensor) rewrites one entry of that table
+            from ..kernels import ExpertTensorList
+
+            layer.w13_weight_list = ExpertTensorList([w.clone() for w in layer.w13_weight.data.unbind(dim=0)],
+                                                     "w13_weight")
+            layer.w2_weight_list = ExpertTensorList([w.clone() for w in layer.w2_weight.data.unbind(dim=0)],
+                                                    "w2_weight")
+            layer.w13_weight_scale_fp32_list = ExpertTensorList(
+                [s.clone() for s in layer.w13_weight_scale_fp32.unbind(dim=0)], "w13_weight_scale")
+            layer.w2_weight_scale_list = ExpertTensorList(
+                [s.clone() for s in layer.w2_weight_scale_fp32.unbind(dim=0)], "w2_weight_scale")
             del layer.w13_weight, layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale
             del layer.w13_weight_scale_fp32, layer.w2_weight_scale_fp32
 
