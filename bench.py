@@ -234,23 +234,27 @@ def run_workload(name, args, lib, torch, np):
             step()
         torch.cuda.synchronize()
         hooked = {"i": 0, "fired": 0}
-        hook_name = "gmm1_swiglu_quant_w4" if cfg.w4_group >= 0 else "gmm1_swiglu_quant"
-        orig = getattr(K, hook_name)
-        rows_seen = {}
+        # the launchers of the routed gate_up GEMM (small batches read their rows through a row -> token map)
+        hook_names = ["gmm1_swiglu_quant_w4"] if cfg.w4_group >= 0 else ["gmm1_swiglu_quant",
+                                                                          "gmm1_swiglu_quant_gather"]
+        origs = {h: getattr(K, h) for h in hook_names}
 
-        def timed_gmm1(x_, *a, **kw):
-            if x_.shape[0] != R:  # the shared expert's dense GEMMs go through the same launcher
+        def make_timed(orig, routed):
+            def timed_gmm1(x_, *a, **kw):
+                if not routed(x_):  # the shared expert's dense GEMMs go through the same launcher
+                    return orig(x_, *a, **kw)
+                s, e = evs[hooked["i"]]
+                hooked["fired"] += 1
+                # create the underlying hipEvent handles, then let the library record them around the GEMM kernel
+                s.record()
+                e.record()
+                lib.moe355_profile_next_gemm(ctypes.c_void_p(s.cuda_event), ctypes.c_void_p(e.cuda_event))
                 return orig(x_, *a, **kw)
-            s, e = evs[hooked["i"]]
-            hooked["fired"] += 1
-            rows_seen["rows"] = x_.shape[0]
-            # create the underlying hipEvent handles, then let the library record them around the GEMM kernel
-            s.record()
-            e.record()
-            lib.moe355_profile_next_gemm(ctypes.c_void_p(s.cuda_event), ctypes.c_void_p(e.cuda_event))
-            return orig(x_, *a, **kw)
+            return timed_gmm1
 
-        setattr(K, hook_name, timed_gmm1)
+        for h in hook_names:
+            setattr(K, h, make_timed(origs[h], (lambda x_: True) if h.endswith("gather")
+                                     else (lambda x_: x_.shape[0] == R)))
         try:
             torch.cuda.synchronize()
             te0 = time.perf_counter()
@@ -260,7 +264,8 @@ def run_workload(name, args, lib, torch, np):
             torch.cuda.synchronize()
             out["eager_ms_per_step"] = round((time.perf_counter() - te0) * 1e3 / n, 5)
         finally:
-            setattr(K, hook_name, orig)
+            for h in hook_names:
+                setattr(K, h, origs[h])
         if hooked["fired"] == n:
             durs = sorted(s.elapsed_time(e) for s, e in evs)  # ms
             avg_ms = sum(durs) / len(durs)

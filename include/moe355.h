@@ -154,6 +154,33 @@ int moe355_init_routing_static(const void *x, int x_dtype, int64_t num_tokens, i
                                int64_t *expert_tokens, float *dynamic_scale, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Small batches (decode): the gating op and the init-routing op in ONE launch.
+ * No single counterpart in the reference: it stands in for the pair
+ *   torch.ops._C_ascend.moe_gating_top_k (vllm_ascend/ops/fused_moe/router/fused_topk_router.py:84-159) +
+ *   torch_npu.npu_moe_init_routing_v2(quant_mode=1) (vllm_ascend/ops/fused_moe/token_dispatcher.py:424-435)
+ * with the arithmetic of moe355_gating_top_k and moe355_init_routing, for batches of at most 1024 (token, slot)
+ * pairs over at most 256 experts (moe355_route_quant_small_supported() != 0), where two launches of a few
+ * microseconds each are a visible part of the layer.  Some workgroups gate four tokens each and the last of
+ * them to finish sorts the pairs (nobody waits); the others quantise one token row each.
+ * The int8 rows are written ONCE, in token order: row r of the expert-sorted
+ * activation is xq[row_token[r]] with scale x_scale[row_token[r]], which is how moe355_gmm1_swiglu_quant_gather
+ * reads it; nothing is copied k times.
+ *   logits [T, E] (logits_dtype), bias [E] (logits_dtype) or NULL, x [T, H] bf16 / fp16 ->
+ *   topk_weights [T, k] in x's dtype (the gate's weights rounded to the logits dtype, then to x's dtype),
+ *   topk_ids [T, k] int32, xq [T, H] int8, x_scale [T] fp32, expanded_row_idx [T*k] int32,
+ *   row_token [T*k] int32, expert_tokens [E] int64 (counts, or their running sum for tokens_num_type 0).
+ * sync_counter: ONE int32 in device memory that is 0 when the call starts to execute; the call leaves it at 0.
+ * (Allocate it once, zeroed, and keep it; calls that may overlap in time need counters of their own.)
+ */
+int moe355_route_quant_small_supported(int64_t num_tokens, int top_k, int num_experts);
+int moe355_route_quant_small(const void *x, int x_dtype, const void *logits, int logits_dtype, const void *bias,
+                             int64_t num_tokens, int64_t hidden, int num_experts, int k, int k_group,
+                             int group_count, int group_select_mode, int renorm, int norm_type,
+                             float routed_scaling_factor, float eps, int tokens_num_type, void *topk_weights,
+                             int32_t *topk_ids, int8_t *xq, float *x_scale, int32_t *expanded_row_idx,
+                             int32_t *row_token, int64_t *expert_tokens, int32_t *sync_counter, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Weight format cast: dense int8 weights -> the MFMA-tiled storage the grouped
  * GEMMs stream ("NZ" of this build).  Stands in for
  * torch_npu.npu_format_cast(w, ACL_FORMAT_FRACTAL_NZ) in
@@ -197,6 +224,16 @@ int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const flo
                              const float *x_scale, const int64_t *group_list, int group_list_type, int64_t rows,
                              int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
                              float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The same op on activations that were quantised in token order and not gathered (moe355_route_quant_small):
+ * x [T, K] int8, x_scale [T]; row r of the expert-sorted order is x[row_token[r]] with scale
+ * x_scale[row_token[r]] (row_token [rows] int32).  out / out_scale are in the expert-sorted order, as above.
+ * Always runs the weight-streaming kernel (the form is meant for small batches). */
+int moe355_gmm1_swiglu_quant_gather(const int8_t *x, const float *x_scale, const int32_t *row_token,
+                                    const int8_t *weight_nz, const float *weight_scale, const int64_t *group_list,
+                                    int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts,
+                                    float swiglu_limit, int8_t *out, float *out_scale, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 
 /* Per-expert tensors: weight_nz_list / weight_scale_list are DEVICE arrays of num_experts pointers,
  * entry e pointing at expert e's tiled [N, K] weights / its [N] fp32 scales (experts that can be

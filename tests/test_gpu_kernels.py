@@ -151,6 +151,84 @@ def test_init_routing_of_prequantised_activations(K, orc, T, k, E, H):
     assert np.array_equal(sx.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
+SMALL_ROUTE_CASES = [
+    # T, k, E, H, norm_type, renorm, bias, G, k_group, rsf, logits dtype, hidden dtype
+    (64, 8, 128, 2048, 0, 1, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
+    (64, 8, 256, 7168, 1, 1, True, 8, 4, 2.5, torch.float32, torch.bfloat16),
+    (1, 1, 8, 64, 0, 0, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
+    (128, 8, 64, 512, 0, 1, False, 1, 1, 1.0, torch.bfloat16, torch.bfloat16),   # 1024 pairs: the limit
+    (33, 6, 96, 9216, 1, 0, True, 4, 2, 1.5, torch.float16, torch.float16),      # rows longer than one pass
+    (17, 2, 3, 72, 0, 1, False, 1, 1, 1.0, torch.float32, torch.float16),
+    (100, 4, 256, 128, 0, 1, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", SMALL_ROUTE_CASES)
+def test_route_quant_small_equals_gating_plus_init_routing(K, orc, case):
+    """The one-launch form for small batches against the checker's gating and dispatch: ids, weights (rounded to
+    the logits dtype, then to the hidden dtype), permutation, histogram; and, through the row -> token map, the
+    int8 rows and scales of the expert-sorted activation."""
+    T, k, E, H, norm_type, renorm, use_bias, G, k_group, rsf, ldt, xdt = case
+    print(f"route_quant_small {case}", flush=True)
+    assert K.route_quant_small_supported(T, k, E)
+    g = torch.Generator().manual_seed(T * 31 + E)
+    x = torch.randn(T, H, generator=g).to(xdt)
+    logits = (torch.rand(T, E, generator=g) * 4 - 2).to(ldt)
+    bias = (torch.rand(E, generator=g) * 0.4 - 0.2).to(ldt) if use_bias else None
+    counter = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for _ in range(3):  # the arrival counter is left at zero: calls in a row share it
+        tw, ids, xq, xs, dst, row_token, cnt = K.route_quant_small(
+            x.to(DEV), logits.to(DEV), k, k_group, G, 1, renorm, norm_type, rsf, 1e-20,
+            bias.to(DEV) if use_bias else None, sync_counter=counter)
+    torch.cuda.synchronize()
+    lname = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[ldt]
+    with orc.half_kind("f16" if xdt == torch.float16 else "bf16"):
+        y, ids_want, _ = orc.gating_top_k(bits(logits), k, bias=bits(bias) if use_bias else None, k_group=k_group,
+                                          group_count=G, group_select_mode=1, renorm=renorm, norm_type=norm_type,
+                                          routed_scaling_factor=rsf, eps=1e-20, x_dtype=lname)
+        # the reference's caller casts the gate's weights (logits dtype) to the hidden dtype
+        yf = y if lname == "f32" else (orc.bf16_to_f32(y) if lname == "bf16" else orc.f16_to_f32(y))
+        tw_want = orc.f32_to_half(yf)
+        xs_want, dst_want, cnt_want, sx_want = orc.init_routing(bits(x), ids_want, E, quant=True)
+    assert np.array_equal(ids.cpu().numpy(), ids_want)
+    assert np.array_equal(bits(tw), tw_want)
+    assert np.array_equal(dst.cpu().numpy(), dst_want)
+    assert np.array_equal(cnt.cpu().numpy(), cnt_want)
+    rt = row_token.cpu().numpy()
+    assert np.array_equal(rt[dst_want], np.arange(T * k) // k)            # row -> token is the inverse map
+    assert np.array_equal(xq.cpu().numpy()[rt], xs_want)                   # the expert-sorted rows, read through it
+    assert np.array_equal(xs.cpu().numpy()[rt].view(np.uint32), sx_want.view(np.uint32))
+    assert int(counter.item()) == 0
+    assert not K.route_quant_small_supported(129, 8, 128) and not K.route_quant_small_supported(8, 8, 257)
+
+
+@pytest.mark.parametrize("R,E,Kd,N,T", [(512, 128, 2048, 1536, 64), (40, 4, 64, 128, 40), (300, 16, 768, 256, 75),
+                                        (512, 256, 1024, 4096, 64), (100, 8, 64, 4160, 25)])
+def test_gmm1_swiglu_quant_gather(K, orc, R, E, Kd, N, T):
+    """Rows read through the row -> token map give what the gathered copy gives."""
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(R + E + 9)
+    xq = torch.randint(-128, 128, (T, Kd), generator=g, dtype=torch.int8)
+    sx = torch.rand(T, generator=g) * 0.05 + 0.001
+    row_token = torch.randint(0, T, (R,), generator=g, dtype=torch.int32)
+    w = torch.randint(-127, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    cnt = _rand_groups(g, E, R)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    q, qs = K.gmm1_swiglu_quant_gather(xq.to(DEV), sx.to(DEV), row_token.to(DEV), wnz, sw.to(DEV), cnt.to(DEV), 1, N,
+                                       Kd)
+    idx = row_token.long()
+    q2, qs2 = K.gmm1_swiglu_quant(xq[idx].contiguous().to(DEV), wnz, sw.to(DEV), sx[idx].contiguous().to(DEV),
+                                  cnt.to(DEV), 1, N, Kd)
+    torch.cuda.synchronize()
+    assert torch.equal(q, q2) and torch.equal(qs, qs2)
+    cum = torch.cumsum(cnt, 0)
+    acc = orc.gmm_i32(xq[idx].numpy(), w.numpy(), cum.numpy())
+    qo, so = orc.swiglu_quant(orc.dequant_acc(acc, sx[idx].numpy(), sw.numpy(), cum.numpy()))
+    assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(qs.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
 def test_init_routing_known_answer(K):
     """Permutation known-answer vector of the reference (tests/ut/lora/test_lora.py:151-165)."""
     ids = torch.tensor([[1, 0], [0, 1], [1, 1]], dtype=torch.int32)

@@ -11,14 +11,20 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+# fused: small batches take the four-launch form (gating + dispatch in one kernel) unless it is switched off;
+# c3_small (2560 pairs) is beyond it either way
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("name", ["c1_tiny", "c2_small", "c3_small", "c4_small", "c2_qwen3_decode"])
-def test_layer_bit_exact(name):
+def test_layer_bit_exact(name, fused):
     from oracle import oracle as orc
 
     cfg = CONFIGS[name]
-    print(f"layer {name}", flush=True)
+    print(f"layer {name} fused={fused}", flush=True)
     d = make_layer(cfg, seed=0)
     layer = build_layer(cfg, d, DEV)
+    layer.use_fused_small_batch = fused
+    takes_fused = layer.quant_method.supports_small_batch(layer, d["x"].to(DEV), d["logits"].to(DEV), layer.router)
+    assert takes_fused == (cfg.T * cfg.k <= 1024)
     x, logits = d["x"].to(DEV), d["logits"].to(DEV)
     res = layer.forward_impl(x, logits)
     torch.cuda.synchronize()

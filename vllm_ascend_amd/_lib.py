@@ -36,6 +36,14 @@ PROTOTYPES = {
                                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe355_init_routing_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int, c_int, c_int,
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "moe355_route_quant_small_supported": (c_int, [c_int64, c_int, c_int]),
+    "moe355_route_quant_small": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int, c_int,
+                                         c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p]),
+    "moe355_gmm1_swiglu_quant_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p,
+                                                c_void_p, c_size_t, c_void_p]),
     "moe355_format_cast_nz": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "moe355_format_cast_nz_int4": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "moe355_w4_offset_correction": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_void_p]),

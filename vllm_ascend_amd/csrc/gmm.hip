@@ -123,9 +123,10 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     for (int64_t r0 = row0; r0 < row1; r0 += 32) {
         const int64_t row = r0 + tok;
         const bool valid = row < row1;
-        const int8_t* xr = a.x + row * a.K + kh * 16;
+        const int64_t src = a.row_src ? (int64_t)a.row_src[valid ? row : row0] : row;  // where the row's values lie
+        const int8_t* xr = a.x + src * a.K + kh * 16;
         float rs = 0.0f;
-        if constexpr (EPI != EPI_I32) rs = a.row_scale[valid ? row : row0];
+        if constexpr (EPI != EPI_I32) rs = a.row_scale[a.row_src ? src : (valid ? row : row0)];
         v16i c0 = {0}, c1 = {0};
         if (r0 != row0) load_weights(kb_begin);
         for (int kb = kb_begin; kb < kb_end; kb += UN) {
@@ -432,7 +433,7 @@ static int gmm1_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* con
                      const float* weight_scale, const float* const* scale_list, const float* x_scale,
                      const int64_t* group_list, int group_list_type, int64_t rows, int64_t k, int64_t n,
                      int num_experts, float swiglu_limit, int8_t* out, float* out_scale, void* workspace,
-                     size_t workspace_bytes, void* stream)
+                     size_t workspace_bytes, void* stream, const int32_t* row_src = nullptr)
 {
     const void* wany = weight_list ? (const void*)weight_list : (const void*)weight_nz;
     int rc = check_gmm(x, wany, group_list, group_list_type, rows, k, n, num_experts);
@@ -461,7 +462,9 @@ static int gmm1_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* con
     a.s_list = scale_list;
     a.limit = swiglu_limit;
     a.y = y;
-    void* tile_ws = (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
+    a.row_src = row_src;
+    // rows read through row_src: the weight-streaming kernel (the form exists for small batches)
+    void* tile_ws = row_src ? nullptr : (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
     rc = launch_gemm_auto<EPI_SWIGLU>(a, tile_ws, st);
     if (rc != MOE355_OK) return rc;
     launch_swiglu_requant(y, group_list, group_list_type, num_experts, rows, I, out, out_scale, st);
@@ -476,6 +479,17 @@ extern "C" int moe355_gmm1_swiglu_quant(const int8_t* x, const int8_t* weight_nz
 {
     return gmm1_impl(x, weight_nz, nullptr, weight_scale, nullptr, x_scale, group_list, group_list_type, rows, k, n,
                      num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_gather(const int8_t* x, const float* x_scale, const int32_t* row_token,
+                                               const int8_t* weight_nz, const float* weight_scale,
+                                               const int64_t* group_list, int group_list_type, int64_t rows,
+                                               int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t* out,
+                                               float* out_scale, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (rows > 0 && !row_token) return MOE355_E_ARG;
+    return gmm1_impl(x, weight_nz, nullptr, weight_scale, nullptr, x_scale, group_list, group_list_type, rows, k, n,
+                     num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream, row_token);
 }
 
 extern "C" int moe355_gmm1_swiglu_quant_list(const int8_t* x, const int8_t* const* weight_nz_list,

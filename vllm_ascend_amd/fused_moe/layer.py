@@ -32,6 +32,8 @@ class AscendRoutedExperts(torch.nn.Module):
         self.ascend_mc2_mask = None
         self.ascend_pertoken_scale = None
         self.enable_force_load_balance = False  # profile runs only (routed_experts.py:484-492)
+        # small batches (decode): gating and dispatch in one launch when the scheme has the fused form
+        self.use_fused_small_batch = True
         specs = dict(quant_method.get_weight(moe_config.num_experts, moe_config.intermediate_size_per_partition,
                                              moe_config.hidden_dim, params_dtype))
         specs.update(quant_method.get_dynamic_quant_param(moe_config.num_experts,
@@ -53,6 +55,12 @@ class AscendRoutedExperts(torch.nn.Module):
 
     def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
         hidden_states, router_logits, _, _ = self.moe_comm_method.prepare(hidden_states, router_logits)
+        fused = getattr(self.quant_method, "supports_small_batch", None)
+        if self.use_fused_small_batch and fused is not None and fused(self, hidden_states, router_logits, self.router):
+            result = self.quant_method.apply_small_batch(self, hidden_states, router_logits, self.router,
+                                                         self.shared_experts, None)
+            result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
+            return result
         # int8 hidden states = activations the caller quantised (their scales in ascend_pertoken_scale): the
         # routing weights then take the model dtype of the scheme
         weights_dtype = None

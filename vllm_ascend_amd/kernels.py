@@ -164,6 +164,72 @@ def init_routing_prequant(xq, x_scale, expert_idx, num_experts, tokens_num_type)
     return xs, row_idx, tokens, scale
 
 
+def route_quant_small_supported(num_tokens: int, top_k: int, num_experts: int) -> bool:
+    return bool(_lib.load().moe355_route_quant_small_supported(num_tokens, top_k, num_experts))
+
+
+def route_quant_small(x, logits, k, k_group, group_count, group_select_mode, renorm, norm_type,
+                      routed_scaling_factor, eps, bias, sync_counter=None):
+    """Gating and dispatch of a small batch in one launch.  -> (topk_weights [T, k] in x's dtype, topk_ids,
+    xq int8 [T, H] in TOKEN order, x_scale [T], expanded_row_idx [T*k], row_token [T*k], expert_tokens [E] counts).
+    sync_counter: a one-element int32 GPU tensor that is zero between calls
+    (a layer keeps one); without it a zeroed one is made for this call (one more small launch)."""
+    x = _dev(x, "x")
+    logits = _dev(logits, "router_logits")
+    if bias is not None:
+        bias = _dev(bias, "bias")
+        if bias.dtype != logits.dtype:
+            raise RuntimeError("The dtype of x and bias should be same")
+    lib = _lib.load()
+    T, E = logits.shape
+    H = x.shape[-1]
+    if x.numel() != T * H:
+        raise ValueError(f"hidden states {tuple(x.shape)} do not match {T} rows of router logits")
+    dev = x.device
+    tw = torch.empty((T, k), dtype=x.dtype, device=dev)
+    ids = torch.empty((T, k), dtype=torch.int32, device=dev)
+    xq = torch.empty((T, H), dtype=torch.int8, device=dev)
+    xs = torch.empty((T,), dtype=torch.float32, device=dev)
+    dst = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    row_token = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((E,), dtype=torch.int64, device=dev)
+    if sync_counter is None:
+        sync_counter = torch.zeros((1,), dtype=torch.int32, device=dev)
+    elif sync_counter.dtype != torch.int32 or sync_counter.numel() != 1 or sync_counter.device != dev:
+        raise ValueError("sync_counter must be a one-element int32 tensor on the device of x")
+    check(lib.moe355_route_quant_small(_ptr(x), _dt(x, "x"), _ptr(logits), _dt(logits, "router_logits"), _ptr(bias),
+                                       T, H, E, k, k_group, group_count, group_select_mode, int(renorm), norm_type,
+                                       float(routed_scaling_factor), float(eps), 1, _ptr(tw), _ptr(ids), _ptr(xq),
+                                       _ptr(xs), _ptr(dst), _ptr(row_token), _ptr(tokens), _ptr(sync_counter),
+                                       _stream(x)), "moe355_route_quant_small")
+    return tw, ids, xq, xs, dst, row_token, tokens
+
+
+def gmm1_swiglu_quant_gather(xq, x_scale, row_token, weight_nz, weight_scale, group_list, group_list_type, n, k,
+                             swiglu_limit=0.0):
+    """gate_up GEMM + SwiGLU + re-quantisation on rows that are read through ``row_token`` from activations kept
+    in token order (route_quant_small).  -> (int8 [R, n/2], fp32 [R]) in the expert-sorted order."""
+    lib = _lib.load()
+    rows = row_token.numel()
+    E = weight_nz.shape[0]
+    if row_token.dtype != torch.int32:
+        raise TypeError(f"row_token must be int32, got {row_token.dtype}")
+    _check_gmm_operands("gmm1_swiglu_quant_gather", xq, xq.shape[0], k, n, E, group_list, x_scale, "x_scale",
+                        weight_nz, E * n * k, weight_scale, E * n)
+    xq = _dev(xq, "x")
+    dev = xq.device
+    out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
+    out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.moe355_gmm1_swiglu_quant_workspace(rows, n, k, E), dev)
+    check(lib.moe355_gmm1_swiglu_quant_gather(_ptr(xq), _ptr(_dev(x_scale, "x_scale")),
+                                              _ptr(_dev(row_token, "row_token")), _ptr(_dev(weight_nz, "weight")),
+                                              _ptr(_dev(weight_scale, "scale")), _ptr(_gl(group_list)),
+                                              _gl_type(group_list_type), rows, k, n, E, float(swiglu_limit),
+                                              _ptr(out), _ptr(out_scale), _ptr(ws), ws.numel(), _stream(xq)),
+          "moe355_gmm1_swiglu_quant_gather")
+    return out, out_scale
+
+
 def format_cast_nz(w: torch.Tensor, layout: int) -> torch.Tensor:
     """int8 [E, N, K] (layout W_ENK) or [E, K, N] (W_EKN) -> same shape, MFMA-tiled storage."""
     w = _dev(w, "weight")

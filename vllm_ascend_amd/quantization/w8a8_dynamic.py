@@ -112,6 +112,73 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 w2_scale=layer.w2_weight_scale_list if self.use_expert_weight_list else [layer.w2_weight_scale_fp32],
             ))
 
+    # ------------------------------------------------------------------ small batches (decode)
+    def supports_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
+        """Whether ``apply_small_batch`` can take this call: plain W8A8 weights (no per-expert lists), 16-bit
+        hidden states as a [T, H] matrix, none of the optional inputs of ``apply``, SiLU, and a batch of at most
+        1024 (token, slot) pairs over at most 256 experts."""
+        from .. import kernels
+
+        if self.use_expert_weight_list or not x.is_cuda or x.dim() != 2 or router_logits.dim() != 2:
+            return False
+        if x.dtype not in (torch.bfloat16, torch.float16) or x.dtype != self.in_dtype:
+            return False
+        if router_logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            return False
+        if (getattr(layer, "apply_router_weight_on_input", False) or getattr(layer, "ascend_pertoken_scale", None)
+                is not None or getattr(layer, "ascend_expert_map", None) is not None
+                or getattr(layer, "ascend_mc2_mask", None) is not None
+                or getattr(layer, "global_redundant_expert_num", 0) or getattr(layer, "enable_force_load_balance", False)):
+            return False
+        act = getattr(layer, "activation", "silu")
+        if (getattr(act, "value", act) or "silu") != "silu":
+            return False
+        return kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
+
+    def apply_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router,
+                          shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
+        """router + ``apply`` for a small batch in four launches instead of six: gating and dispatch are one
+        kernel (the token rows are quantised once, in token order, and the gate_up GEMM reads them through the
+        row -> token map), then the gate_up GEMM with SwiGLU and re-quantisation, the down GEMM and the combine.
+        Same results, bit for bit, as ``router.select_experts`` followed by ``apply``
+        (``vllm_ascend/ops/fused_moe/routed_experts.py:496-609``, ``w8a8_dynamic.py:224-301``)."""
+        from .. import kernels
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        bias = router.e_score_correction_bias
+        if bias is not None and bias.dtype != router_logits.dtype:
+            bias = router.e_score_correction_bias = bias.to(router_logits.dtype)
+        stream = torch.cuda.current_stream()
+        before_dispatch_evt = stream.record_event()
+        # the routing kernel's arrival counter: one zeroed int32 per layer (and device), which every call leaves at
+        # zero; created on the first call (run the layer once before capturing it into a graph)
+        counter = getattr(layer, "_small_batch_counter", None)
+        if counter is None or counter.device != x.device:
+            counter = layer._small_batch_counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
+        topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = kernels.route_quant_small(
+            x, router_logits, router.top_k, router.topk_group if router.topk_group is not None else 1,
+            router.num_expert_group if router.num_expert_group is not None else 1, 1, int(router.renormalize),
+            0 if router.scoring_func == "softmax" else 1, router.routed_scaling_factor, 1e-20, bias,
+            sync_counter=counter)
+        shared_out = None
+        if shared_experts is not None:
+            shared_out = shared_experts(x if shared_experts_input is None else shared_experts_input)
+        w13, w2 = layer.w13_weight, layer.w2_weight
+        cfg = getattr(layer, "moe_config", None)
+        swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
+        q1, q1_scale = kernels.gmm1_swiglu_quant_gather(xq, x_scale, row_token, w13, layer.w13_weight_scale_fp32,
+                                                        expert_tokens, 1, w13.shape[2], w13.shape[1], swiglu_limit)
+        before_gmm2_evt = stream.record_event()
+        out = kernels.gmm2_dequant(q1, w2, layer.w2_weight_scale_fp32, q1_scale, expert_tokens, 1, w2.shape[2],
+                                   w2.shape[1], out_dtype=x.dtype)
+        before_combine_evt = stream.record_event()
+        if shared_experts is not None and shared_out is not None:
+            shared_experts.wait()
+        routed_out = kernels.token_unpermute(out, expanded_row_idx, topk_weights, shared_out)
+        return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
+                                  before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
+                                  group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
+
     @staticmethod
     def get_eplb_weight_views(layer) -> list:
         if hasattr(layer, "w13_weight_list"):
