@@ -257,7 +257,10 @@ GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100
              # many experts (a lane of the tile map / a thread of the scans owns more than one expert from 257
              # on): weight streaming, 128-row tiles and the weight-streaming tiles, each with 256 and with more
              (2000, 256, 128, 128), (1500, 320, 64, 64), (16000, 256, 128, 256), (20000, 320, 192, 128),
-             (32000, 256, 1024, 128), (40000, 320, 1024, 64)]
+             (32000, 256, 1024, 128), (40000, 320, 1024, 64),
+             # one expert with at most 64 rows and a long K (the shared expert of a decode batch): the int32 product
+             # cuts K into slabs and adds the partial sums into the zeroed result
+             (64, 1, 7168, 256), (33, 1, 2048, 1024), (1, 1, 4096, 128)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)

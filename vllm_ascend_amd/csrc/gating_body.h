@@ -70,6 +70,27 @@ __device__ __forceinline__ unsigned long long make_key(float score, int index)
 
 __device__ __forceinline__ int key_index(unsigned long long key) { return (int)(0xffffffffu - (unsigned)key); }
 
+// Score of one expert group from its gs selection scores: the best one (mode 0) or the sum of the best two, best
+// first ("larger value, then lower index").  One pass that keeps the two leaders.
+__device__ __forceinline__ float group_score(const float* s, int gs, int mode)
+{
+    int i1 = 0, i2 = -1;
+    float v1 = s[0], v2 = 0.0f;
+    for (int j = 1; j < gs; ++j) {
+        const float v = s[j];
+        if (ranks_before(v, j, v1, i1)) {
+            v2 = v1;
+            i2 = i1;
+            v1 = v;
+            i1 = j;
+        } else if (i2 < 0 || ranks_before(v, j, v2, i2)) {
+            v2 = v;
+            i2 = j;
+        }
+    }
+    return (mode != 0 && gs >= 2) ? v1 + v2 : v1;
+}
+
 // One token row by one wavefront.  Every wavefront of the workgroup calls this the same number of times (it
 // contains workgroup barriers); a call with live == false computes a valid row and stores nothing.
 // sc_lds: E floats, w_lds: 64 floats, both private to the wavefront.  y may be null (only y_alt wanted);
@@ -134,17 +155,7 @@ __device__ __forceinline__ void gate_row(const void* __restrict__ x, const void*
         unsigned long long gkey = 0ull;
         if (lane < G) {
             const float* s = sc_lds + lane * gs;
-            int i1 = 0;
-            for (int j = 1; j < gs; ++j)
-                if (ranks_before(s[j], j, s[i1], i1)) i1 = j;
-            float score = s[i1];
-            if (mode != 0 && gs >= 2) {
-                int i2 = (i1 == 0) ? 1 : 0;
-                for (int j = 0; j < gs; ++j)
-                    if (j != i1 && ranks_before(s[j], j, s[i2], i2)) i2 = j;
-                score = s[i1] + s[i2];
-            }
-            gkey = make_key(score, lane);
+            gkey = make_key(group_score(s, gs, mode), lane);
         }
         unsigned long long keep = 0ull;
         for (int c = 0; c < k_group; ++c) {
@@ -270,18 +281,7 @@ __device__ __forceinline__ void gate_rows(const void* __restrict__ x, const void
         for (int r = 0; r < NR; ++r) {
             gkey[r] = 0ull;
             if (lane < G) {
-                const float* s = grp_lds + r * E + lane * gs;
-                int i1 = 0;
-                for (int j = 1; j < gs; ++j)
-                    if (ranks_before(s[j], j, s[i1], i1)) i1 = j;
-                float score = s[i1];
-                if (mode != 0 && gs >= 2) {
-                    int i2 = (i1 == 0) ? 1 : 0;
-                    for (int j = 0; j < gs; ++j)
-                        if (j != i1 && ranks_before(s[j], j, s[i2], i2)) i2 = j;
-                    score = s[i1] + s[i2];
-                }
-                gkey[r] = make_key(score, lane);
+                gkey[r] = make_key(group_score(grp_lds + r * E + lane * gs, gs, mode), lane);
             }
         }
         unsigned long long keep[NR];

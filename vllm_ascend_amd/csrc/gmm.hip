@@ -64,9 +64,14 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     const int nb0 = (EPI == EPI_SWIGLU) ? p : 2 * p;
     const int nb1 = (EPI == EPI_SWIGLU) ? p + upe : 2 * p + 1;
 
+    // K is cut into gridDim.y slabs (1 except for the dense small-batch product, whose workgroups add their int32
+    // partial sums into a zeroed result with atomics: integer addition, exact and order free), and a slab into
+    // KSPLIT pieces, one per wavefront
     const int ks = (KSPLIT == 1) ? 0 : wave;
-    const int kb_begin = (KB * ks) / KSPLIT;
-    const int kb_end = (KB * (ks + 1)) / KSPLIT;
+    const int slab_begin = (int)(((int64_t)KB * blockIdx.y) / gridDim.y);
+    const int slab_end = (int)(((int64_t)KB * (blockIdx.y + 1)) / gridDim.y);
+    const int kb_begin = slab_begin + ((slab_end - slab_begin) * ks) / KSPLIT;
+    const int kb_end = slab_begin + ((slab_end - slab_begin) * (ks + 1)) / KSPLIT;
 
     const int8_t* we = expert_weights(a, e);
     const int8_t* w0 = we + ((int64_t)nb0 * KB) * 1024 + lane * 16;
@@ -167,7 +172,17 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
                 u[j] = red[(16 + 4 * wave + j) * 64 + lane];
             }
             const int ch = quad_channel(wave, lane);
-            epilogue_run<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u, rs, cs0[0], cs1[0]);
+            if (EPI == EPI_I32 && gridDim.y > 1) {
+                if (valid) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        atomicAdd(a.acc + row * a.N + nb0 * 32 + ch + j, g[j]);
+                        atomicAdd(a.acc + row * a.N + nb1 * 32 + ch + j, u[j]);
+                    }
+                }
+            } else {
+                epilogue_run<EPI>(a, row, valid, nb0 * 32 + ch, nb1 * 32 + ch, g, u, rs, cs0[0], cs1[0]);
+            }
             __syncthreads();
         } else {
 #pragma unroll
@@ -290,6 +305,12 @@ void take_profile_events(hipEvent_t& start, hipEvent_t& stop)
     t_ev_stop = nullptr;
 }
 
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, int64_t n4)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) ((v4i*)p)[i] = (v4i){0, 0, 0, 0};
+}
+
 template <typename KernelT>
 static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs& a)
 {
@@ -332,7 +353,8 @@ static size_t tiled_ws_max(int64_t rows, int E)
 template <int EPI>
 static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
 {
-    const int bm = tile_ws ? tiled_bm(a) : 0;
+    int bm = tile_ws ? tiled_bm(a) : 0;
+    if (EPI == EPI_I32 && a.E == 1 && a.R <= 64 && (a.K >> 5) >= 64 && a.N / 64 < 256) bm = 0;  // dense, few rows
     if (bm) {
         launch_tiled_any(EPI, bm, a, tile_ws, st, t_ev_start, t_ev_stop);
         t_ev_start = nullptr;
@@ -340,6 +362,22 @@ static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
         return launch_status();
     }
     const int64_t units = (int64_t)a.E * (a.N / 64);
+    if constexpr (EPI == EPI_I32) {
+        // One expert with at most 64 rows (the shared expert of a decode batch: a dense product over a few tokens):
+        // too few workgroups for a chip that needs thousands of loads in flight to stream at full rate.  K is cut
+        // into slabs, one workgroup per (pair of tiles, slab), partial sums added into the zeroed result.
+        const int KB = a.K >> 5;
+        if (a.E == 1 && a.R <= 64 && units < 256 && KB >= 64) {
+            int slabs = (int)(512 / units);
+            if (slabs > KB / 8) slabs = KB / 8;
+            if (slabs > 1) {
+                const int64_t n4 = a.R * (int64_t)a.N / 4;  // N % 64 == 0
+                hipLaunchKernelGGL(zero_i32_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, a.acc, n4);
+                launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units, (unsigned)slabs), st, a);
+                return launch_status();
+            }
+        }
+    }
     // Occupancy 3 keeps the SwiGLU epilogue out of scratch memory (131 registers).  With enough units to
     // fill the chip four times over, the down GEMM lets every wavefront stream a whole unit by itself (no
     // K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K.
