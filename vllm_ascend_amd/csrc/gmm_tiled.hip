@@ -168,9 +168,13 @@ __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16
                     *(v4i*)(a.acc + orow * a.N + nb1 * 32 + c16 * 4) =
                         *(const v4i*)(patch + 32 * ROWB + r * ROWB + c16 * 16);
                 } else if constexpr (EPI == EPI_DEQUANT) {
-                    *(v4i*)(a.out + orow * a.N + nb0 * 32 + c16 * 8) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                    // Non-temporal stores for the two large outputs: written back through the L2 in the ordinary
+                    // way they slowed the weight streams of every other workgroup (K loops 8 % longer).
+                    __builtin_nontemporal_store(*(const v4i*)(patch + r * ROWB + c16 * 16),
+                                                (v4i*)(a.out + orow * a.N + nb0 * 32 + c16 * 8));
                 } else {
-                    *(v4i*)(a.y + orow * (a.N >> 1) + nb0 * 32 + c16 * 4) = *(const v4i*)(patch + r * ROWB + c16 * 16);
+                    __builtin_nontemporal_store(*(const v4i*)(patch + r * ROWB + c16 * 16),
+                                                (v4i*)(a.y + orow * (a.N >> 1) + nb0 * 32 + c16 * 4));
                 }
             }
         }
@@ -398,6 +402,8 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : 2)) void gmm_tiled_kernel(GmmA
 // is written by hand, before the barrier that publishes the stage.
 constexpr int kWideLdsBytes = 163840;
 
+constexpr int ring_gcd(int a, int b) { return b == 0 ? a : ring_gcd(b, a % b); }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
@@ -416,13 +422,20 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     static_assert(NBLK == 4 || (WIDE && NBLK > 4 && NBLK <= 8), "tall tiles have two halves of four blocks");
     constexpr int GROUPS = WIDE ? 8 : 4;            // channel groups (two storage tiles each) per workgroup
     constexpr int A_BYTES = GROUPS * 4096;          // weights of a stage
-    constexpr int STAGE = A_BYTES + (WIDE ? NBLK * 2048 : 16384);
-    constexpr int S = kWideLdsBytes / STAGE;        // 4 wide (3 with more than four token blocks), 5 tall
+    constexpr int X_BYTES = WIDE ? NBLK * 2048 : 16384;  // tokens of a stage
+    // Two rings.  The weights come from HBM: their ring takes the LDS that is left once the tokens (L2 hits,
+    // a third of the latency) have a ring of at least three stages.  wide: 4 + 4 (4 + 3 with five token
+    // blocks); tall: 6 + 4.
+    constexpr int SX = WIDE ? (NBLK > 4 ? 3 : 4) : 4;
+    constexpr int SW = (kWideLdsBytes - SX * X_BYTES) / A_BYTES;
+    constexpr int XBASE = SW * A_BYTES;
+    constexpr int CYCLE = SW / ring_gcd(SW, SX) * SX;  // steps after which both rings are back at stage 0
     constexpr int NA = WIDE ? 4 : 2;                // weight loads per wavefront and stage
     constexpr int ROWB = TiledLds<EPI, 4, 3>::ROWB;
     constexpr int PATCHES = TiledLds<EPI, 4, 3>::PATCHES;
-    static_assert(8 * PATCHES * 32 * ROWB <= S * STAGE, "epilogue patches fit the stages");
-    static_assert(S * STAGE <= kWideLdsBytes && S >= 3, "stages fit LDS");
+    static_assert(8 * PATCHES * 32 * ROWB <= SW * A_BYTES + SX * X_BYTES, "epilogue patches fit the stages");
+    static_assert(SW * A_BYTES + SX * X_BYTES <= kWideLdsBytes && SX >= 3 && SW >= SX, "stages fit LDS");
+    static_assert(CYCLE % SW == 0 && CYCLE % SX == 0, "the unrolled steps return to stage 0 of both rings");
 
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
@@ -481,7 +494,7 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     const int8_t* xsrc1 = a.x + xr1 * a.K + xchunk * 16;
     // operand reads of this lane: token l % 32 of a block, K half l / 32, K step s -> chunk 2 s + l / 32
     const int r16 = lane & 15;
-    const int frag_off = A_BYTES + (h * 8 + ((lane >> 4) & 1)) * 1024 + r16 * 64;
+    const int frag_off = XBASE + (h * 8 + ((lane >> 4) & 1)) * 1024 + r16 * 64;
     const int frag_s0 = frag_off + (((lane >> 5) + (r16 >> 2)) & 3) * 16;
     const int frag_s1 = frag_off + ((2 + (lane >> 5) + (r16 >> 2)) & 3) * 16;
     const int a_off = g * 4096 + lane * 16;
@@ -490,32 +503,35 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     const int last_it = n_iter - 1;
     // loads past the last K block are redirected to it (never used), so that the number of loads in flight,
     // which the hand-written waits rely on, is the same in every step
-    auto load_stage = [&](int it, int st) {
+    auto load_weights = [&](int it, int st) {
         const int itc = it < last_it ? it : last_it;
-        int8_t* base = lds + st * STAGE;
-        // weights are read once: non-temporal (cache policy bit 1), so they do not push the tokens out of L2
+        int8_t* base = lds + st * A_BYTES;
+        // plain cache policy: marked non-temporal, the same loads made the kernel 5 % slower
         if constexpr (WIDE) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const int8_t* wp = wsrc[t] + (int64_t)itc * 2048;
                 __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp), MOE355_LPTR(base + wave * 4096 + t * 2048), 16, 0,
-                                                 2);
+                                                 0);
                 __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp + 1024),
-                                                 MOE355_LPTR(base + wave * 4096 + t * 2048 + 1024), 16, 0, 2);
+                                                 MOE355_LPTR(base + wave * 4096 + t * 2048 + 1024), 16, 0, 0);
             }
         } else {
             const int8_t* wp = wsrc[0] + (int64_t)itc * 2048;
-            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp), MOE355_LPTR(base + wave * 2048), 16, 0, 2);
-            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp + 1024), MOE355_LPTR(base + wave * 2048 + 1024), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp), MOE355_LPTR(base + wave * 2048), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(MOE355_GPTR(wp + 1024), MOE355_LPTR(base + wave * 2048 + 1024), 16, 0, 0);
         }
+    };
+    auto load_tokens = [&](int it, int st) {
+        const int itc = it < last_it ? it : last_it;
+        int8_t* base = lds + XBASE + st * X_BYTES;
         if (n_xloads >= 1)
             __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc0 + (int64_t)itc * kBK),
-                                             MOE355_LPTR(base + A_BYTES + wave * (XROWS * 64)), 16, 0, 0);
+                                             MOE355_LPTR(base + wave * (XROWS * 64)), 16, 0, 0);
         if constexpr (X2) {
             if (n_xloads >= 2)
                 __builtin_amdgcn_global_load_lds(MOE355_GPTR(xsrc1 + (int64_t)itc * kBK),
-                                                 MOE355_LPTR(base + A_BYTES + (WIDE ? (wave + 8) * 1024
-                                                                                    : wave * 2048 + 1024)),
+                                                 MOE355_LPTR(base + (WIDE ? (wave + 8) * 1024 : wave * 2048 + 1024)),
                                                  16, 0, 0);
         }
     };
@@ -526,41 +542,51 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
 #pragma unroll
         for (int b = 0; b < NBLK; ++b) acc[t][b] = (v16i){0};
 
+    // Every step requests the tokens SX - 1 steps ahead and then the weights SW - 1 steps ahead; the steps before
+    // the first one do the same for what lies at or after K block 0, so that the order of the requests, which the
+    // hand-written waits count on, is the same from the start.
 #pragma unroll
-    for (int r = 0; r + 1 < S; ++r) load_stage(r, r);
+    for (int j = 1 - SW; j < 0; ++j) {
+        if (j + SX - 1 >= 0) load_tokens(j + SX - 1, j + SX - 1);
+        load_weights(j + SW - 1, j + SW - 1);
+    }
 
-    // One K block on LDS stage u.  A stage is complete for this wavefront when at most (loads per step) x
-    // (stages - 2) younger loads are in flight; the barrier then covers the other wavefronts and also says that
-    // everybody is done reading the stage that the next loads overwrite.
-    auto step = [&](int u, int it) {
-        if (n_xloads == 2) wait_vmcnt<(NA + 2) * (S - 2)>();
-        else if (n_xloads == 1) wait_vmcnt<(NA + 1) * (S - 2)>();
-        else wait_vmcnt<NA * (S - 2)>();
+    // One K block on stage uw of the weights and ux of the tokens.  Requests retire in order.  The younger of the
+    // two requests that this step needs is its tokens (its weights, in the same step, if the rings are equally
+    // deep): what was requested after it may still be in flight.  The barrier then covers the other wavefronts and
+    // also says that everybody is done reading the stages that the next requests overwrite.
+    constexpr int NAFTER = (SW > SX) ? NA : 0;  // the weights requested right behind those tokens
+    auto step = [&](int uw, int ux, int it) {
+        if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
+        else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
+        else wait_vmcnt<NAFTER + NA * (SX - 2)>();
         __builtin_amdgcn_s_barrier();
-        load_stage(it + S - 1, (u + S - 1) % S);
+        load_tokens(it + SX - 1, (ux + SX - 1) % SX);
+        load_weights(it + SW - 1, (uw + SW - 1) % SW);
         if (active) {
-            const int8_t* base = lds + u * STAGE;
+            const int8_t* wbase = lds + uw * A_BYTES;
+            const int8_t* xbase = lds + ux * X_BYTES;
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const v4i a0 = *(const v4i*)(base + a_off + s * 1024);
-                const v4i a1 = *(const v4i*)(base + a_off + 2048 + s * 1024);
+                const v4i a0 = *(const v4i*)(wbase + a_off + s * 1024);
+                const v4i a1 = *(const v4i*)(wbase + a_off + 2048 + s * 1024);
 #pragma unroll
                 for (int b = 0; b < NBLK; ++b) {
-                    const v4i f = *(const v4i*)(base + (s ? frag_s1 : frag_s0) + b * 2048);
+                    const v4i f = *(const v4i*)(xbase + (s ? frag_s1 : frag_s0) + b * 2048);
                     acc[0][b] = mfma_i8(a0, f, acc[0][b]);
                     acc[1][b] = mfma_i8(a1, f, acc[1][b]);
                 }
             }
         }
     };
-    const int n_full = (n_iter / S) * S;
-    for (int i0 = 0; i0 < n_full; i0 += S) {
+    const int n_full = (n_iter / CYCLE) * CYCLE;
+    for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
 #pragma unroll
-        for (int u = 0; u < S; ++u) step(u, i0 + u);
+        for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
     }
 #pragma unroll
-    for (int u = 0; u + 1 < S; ++u)
-        if (n_full + u < n_iter) step(u, n_full + u);
+    for (int u = 0; u + 1 < CYCLE; ++u)
+        if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
 
     wait_vmcnt<0>();  // the redirected loads past the end still write LDS
     __builtin_amdgcn_s_barrier();
@@ -592,6 +618,9 @@ __global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm,
     } else if (row_end - row0 <= 160) {
         if (nt * 2 >= n_col_blocks) return;
         stream_tile_body<EPI, true, 5>(a, e, row0, row_end, nt, wide_lds);
+    } else if (row_end - row0 <= 192) {
+        if (nt * 2 >= n_col_blocks) return;
+        stream_tile_body<EPI, true, 6>(a, e, row0, row_end, nt, wide_lds);
     } else {
         stream_tile_body<EPI, false>(a, e, row0, row_end, nt, wide_lds);
     }
