@@ -45,10 +45,11 @@ WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE / WRITE_SIZE scaled by a copy
 # kernel of known size), taken from the committed summaries: NOT measured in this run.
 TRAFFIC_FROM_PROFILES = {
-    "c2_qwen3_decode": (399_300_000, "profiles/moe_layer_qwen3_decode_hbm_traffic.md"),
-    "c3_qwen3_prefill": (988_000_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
-    "c4_dsv3_prefill": (8_137_900_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
-    "c5_w4a8_zipf": (1_878_600_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
+    "c2_qwen3_decode": (401_500_000, "profiles/moe_layer_qwen3_decode_hbm_traffic.md"),
+    "c3_qwen3_prefill": (940_500_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
+    "c4_dsv3_prefill": (8_039_400_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
+    "c5_w4a8_zipf": (1_735_100_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
+    "c6_dsv3_decode": (6_628_300_000, "profiles/moe_layer_dsv3_decode_kernel_trace.md"),
 }
 
 
@@ -216,7 +217,7 @@ def run_workload(name, args, lib, torch, np):
         out["us_per_layer_single_steps_after_cache_flush"] = single_steps_us(run, min(n_pct, 50), torch,
                                                                               before=flush.zero_)
         del flush
-    if cfg.shared:
+    if cfg.shared and not args.no_side_stream:
         # the shared expert on the side stream, next to the routed experts
         layer.shared_experts.multistream_overlap = True
         g2 = capture(step, torch) if mode == "graph" else None
@@ -370,6 +371,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-side-stream", action="store_true",
+                    help="skip the extra timing with the shared expert on its side stream (kernel profiles: keeps "
+                         "overlapped launches out of the per-kernel durations)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole MoE layer on ONE GPU (no expert parallelism, no collectives); "
