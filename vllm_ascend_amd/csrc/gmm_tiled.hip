@@ -390,14 +390,16 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : 2)) void gmm_tiled_kernel(GmmA
 // ------------------------------------------------------------------ weight-streaming tiles
 // Tiles for shapes whose grouped GEMM is bound by streaming the weights (a few hundred rows per expert at
 // most).  A workgroup of eight wavefronts works on up to 256 rows of one expert, so that an expert with up to
-// 256 rows fetches its weights from HBM exactly once; every wavefront computes 128 tokens x one channel group
-// (two storage tiles) with the accumulator layout and the epilogue of the 128-row tiles.
-//   tall tile (129..256 rows left): wavefront (h, g) = token half h x channel group g of 4 -> 256 x 256;
-//   wide tile (at most 128 rows left): wavefront g = channel group g of 8 -> 128 x 512, which halves the
-//   token traffic per weight byte (tokens come from L2, and that traffic costs weight bandwidth).
-// Both operands reach LDS by LDS-direct loads (no register staging, so the prefetch depth costs no registers).
-// A stage holds the weights of 64 K values (every storage tile x 2 K steps is a contiguous 1 KiB MFMA operand
-// that is copied as it lies) and the tokens' 64 bytes (row-major, with a rotation of the 16-byte chunks).
+// 256 rows fetches its weights from HBM exactly once; every wavefront computes its token blocks x one channel
+// group (two storage tiles) with the accumulator layout and the epilogue of the 128-row tiles.
+//   wide tile (at most 192 rows left): wavefront g = channel group g of 8, all 4, 5 or 6 token blocks of 32
+//   -> 128 / 160 / 192 x 512;
+//   tall tile (193..256 rows left): wavefront (h, g) = token half h x channel group g of 4 -> 256 x 256, twice
+//   the token traffic per weight byte (tokens come from L2, and that traffic costs weight bandwidth).
+// Both operands reach LDS by LDS-direct loads (no register staging, so the prefetch depth costs no registers),
+// each into a ring of its own.  A weight stage holds the weights of 64 K values (every storage tile x 2 K steps
+// is a contiguous 1 KiB MFMA operand that is copied as it lies), a token stage the tokens' 64 bytes (row-major,
+// with a rotation of the 16-byte chunks).
 // The compiler does not count LDS-direct loads against the LDS reads that consume them: the wait for a stage
 // is written by hand, before the barrier that publishes the stage.
 constexpr int kWideLdsBytes = 163840;
@@ -413,7 +415,7 @@ __device__ __forceinline__ void wait_vmcnt()
 #define MOE355_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define MOE355_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-// NBLK: 32-row token blocks per wavefront (4; a wide tile of 5 takes up to 160 rows, so that an expert a little
+// NBLK: 32-row token blocks per wavefront (4 in a tall tile; 4, 5 or 6 in a wide one, so that an expert a little
 // above 128 rows keeps the wide shape instead of paying the token traffic of a tall tile).
 template <int EPI, bool WIDE, int NBLK = 4>
 __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
