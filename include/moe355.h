@@ -126,6 +126,17 @@ int moe355_init_routing(const void *x, int x_dtype, int64_t num_tokens, int64_t 
                         int32_t *expanded_row_idx, int64_t *expert_tokens, float *dynamic_scale, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* The maps of the permutation alone, nothing moved: expanded_row_idx [T*k] (pair -> sorted row, T*k for a
+ * dropped pair), row_token [T*k] (sorted row -> token; entries past the last kept pair are left untouched) and
+ * expert_tokens, exactly as moe355_init_routing computes them.  For callers that quantise the token rows once
+ * (moe355_dynamic_quant) and let moe355_gmm1_swiglu_quant_gather read them through row_token instead of
+ * writing k copies of every row: no counterpart of its own in the reference, it is the index half of
+ * torch_npu.npu_moe_init_routing_v2 (vllm_ascend/ops/fused_moe/token_dispatcher.py:424-435).  The workspace is
+ * the one of moe355_init_routing_workspace. */
+int moe355_route_map(const int32_t *expert_idx, int64_t num_tokens, int top_k, int num_experts, int tokens_num_type,
+                     int32_t *expanded_row_idx, int32_t *row_token, int64_t *expert_tokens, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
 /* The same permutation for activations that are already quantised: x int8 [T, H] with one fp32 scale per
  * token; rows and scales are only moved (expanded_x[row] = x[t], expanded_scale[row] = x_scale[t]).
  * Stands in for torch_npu.npu_moe_init_routing_v2(x, ids, scale=pertoken_scale, quant_mode=-1), the call the
@@ -225,10 +236,10 @@ int moe355_gmm1_swiglu_quant(const int8_t *x, const int8_t *weight_nz, const flo
                              int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t *out,
                              float *out_scale, void *workspace, size_t workspace_bytes, void *stream);
 
-/* The same op on activations that were quantised in token order and not gathered (moe355_route_quant_small):
- * x [T, K] int8, x_scale [T]; row r of the expert-sorted order is x[row_token[r]] with scale
- * x_scale[row_token[r]] (row_token [rows] int32).  out / out_scale are in the expert-sorted order, as above.
- * Always runs the weight-streaming kernel (the form is meant for small batches). */
+/* The same op on activations that were quantised in token order and not gathered (moe355_route_quant_small, or
+ * moe355_dynamic_quant + moe355_route_map): x [T, K] int8, x_scale [T]; row r of the expert-sorted order is
+ * x[row_token[r]] with scale x_scale[row_token[r]] (row_token [rows] int32).  out / out_scale are in the
+ * expert-sorted order, as above.  Every kernel family reads its token rows through the map. */
 int moe355_gmm1_swiglu_quant_gather(const int8_t *x, const float *x_scale, const int32_t *row_token,
                                     const int8_t *weight_nz, const float *weight_scale, const int64_t *group_list,
                                     int group_list_type, int64_t rows, int64_t k, int64_t n, int num_experts,

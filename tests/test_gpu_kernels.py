@@ -203,7 +203,11 @@ def test_route_quant_small_equals_gating_plus_init_routing(K, orc, case):
 
 
 @pytest.mark.parametrize("R,E,Kd,N,T", [(512, 128, 2048, 1536, 64), (40, 4, 64, 128, 40), (300, 16, 768, 256, 75),
-                                        (512, 256, 1024, 4096, 64), (100, 8, 64, 4160, 25)])
+                                        (512, 256, 1024, 4096, 64), (100, 8, 64, 4160, 25),
+                                        # many rows per expert: the LDS-tiled kernel (128- and 64-row tiles) and the
+                                        # weight-streaming tiles (wide and tall) read through the map as well
+                                        (4096, 8, 512, 256, 700), (1300, 16, 192, 128, 400), (1100, 8, 1024, 256, 300),
+                                        (700, 4, 4096, 128, 200), (1500, 6, 4096, 192, 1500)])
 def test_gmm1_swiglu_quant_gather(K, orc, R, E, Kd, N, T):
     """Rows read through the row -> token map give what the gathered copy gives."""
     from vllm_ascend_amd._lib import W_ENK
@@ -227,6 +231,29 @@ def test_gmm1_swiglu_quant_gather(K, orc, R, E, Kd, N, T):
     acc = orc.gmm_i32(xq[idx].numpy(), w.numpy(), cum.numpy())
     qo, so = orc.swiglu_quant(orc.dequant_acc(acc, sx[idx].numpy(), sw.numpy(), cum.numpy()))
     assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(qs.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+@pytest.mark.parametrize("T,k,E,bad", [(3, 2, 2, False), (64, 8, 128, False), (300, 8, 256, True), (4096, 8, 256, False),
+                                       (1000, 6, 40, True), (2500, 1, 7, False)])
+def test_route_map_equals_init_routing_maps(K, T, k, E, bad):
+    """The maps alone (nothing moved) against the ones of the init-routing op; row -> token inverts pair -> row."""
+    g = torch.Generator().manual_seed(T + 5 * k + E)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if bad:
+        drop = torch.rand(T, k, generator=g) < 0.1
+        drop[0, 0] = True
+        ids[drop] = E + 3
+    x = torch.randn(T, 64, generator=g).to(torch.bfloat16)
+    _, dst_want, cnt_want, _ = K.init_routing(x.to(DEV), ids.to(DEV), E, 1, 1)
+    dst, row_token, cnt = K.route_map(ids.to(DEV), E, 1)
+    _, _, cum = K.route_map(ids.to(DEV), E, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, dst_want) and torch.equal(cnt, cnt_want)
+    assert torch.equal(cum, torch.cumsum(cnt_want, 0))
+    d = dst.cpu().numpy()
+    kept = d < T * k
+    assert int(kept.sum()) == int(cnt.sum())
+    assert np.array_equal(row_token.cpu().numpy()[d[kept]], (np.arange(T * k) // k)[kept])
 
 
 def test_init_routing_known_answer(K):

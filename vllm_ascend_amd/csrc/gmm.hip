@@ -501,8 +501,7 @@ static int gmm1_impl(const int8_t* x, const int8_t* weight_nz, const int8_t* con
     a.limit = swiglu_limit;
     a.y = y;
     a.row_src = row_src;
-    // rows read through row_src: the weight-streaming kernel (the form exists for small batches)
-    void* tile_ws = row_src ? nullptr : (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
+    void* tile_ws = (char*)workspace + (((size_t)rows * I * 4 + 255) & ~(size_t)255);
     rc = launch_gemm_auto<EPI_SWIGLU>(a, tile_ws, st);
     if (rc != MOE355_OK) return rc;
     launch_swiglu_requant(y, group_list, group_list_type, num_experts, rows, I, out, out_scale, st);

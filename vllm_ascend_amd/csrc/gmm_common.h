@@ -24,8 +24,8 @@ struct GmmArgs {
     int64_t R;
     int K, N, E;
     const float* row_scale; // [R]     token scale
-    // weight-streaming kernel only, when set: row r of the expert-sorted activation is row row_src[r] of x, and
-    // its scale is row_scale[row_src[r]] (the rows were quantised once, in token order, and never copied)
+    // when set: row r of the expert-sorted activation is row row_src[r] of x, and its scale is
+    // row_scale[row_src[r]] (the rows were quantised once, in token order, and never copied)
     const int32_t* row_src;
     const float* ch_scale;  // [E, N]  channel scale
     // per-expert tensors (weights that can be swapped expert by expert): device arrays of E pointers;

@@ -108,7 +108,8 @@ __device__ __forceinline__ void tiled_epilogue_body(const GmmArgs& a, int e, v16
         rs_all[b] = 0.0f;
         if constexpr (EPI != EPI_I32) {
             const int64_t row = row0 + b * 32 + tok;
-            rs_all[b] = a.row_scale[row < row_end ? row : row_end - 1];
+            const int64_t rc = row < row_end ? row : row_end - 1;
+            rs_all[b] = a.row_scale[a.row_src ? (int64_t)a.row_src[rc] : rc];
             if (row >= row_end) rs_all[b] = 0.0f;
         }
     }
@@ -262,6 +263,7 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
         const int kc = (tid >> 4) & 3;
         int64_t r = row0 + row;
         if (r > row_end - 1) r = row_end - 1;  // rows past the expert's end duplicate its last row
+        if (a.row_src) r = a.row_src[r];       // the row's values lie in the token's row
         xrow[j] = a.x + r * a.K + kc * 16;
         const int s = kc >> 1, kh = kc & 1;
         lds_off[j] = (((s * BMT + (row >> 5)) * 64) + kh * 32 + (row & 31)) * 16;
@@ -492,6 +494,10 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
     int64_t xr0 = xfirst + (lane >> 2), xr1 = xr0 + XSECOND;
     if (xr0 > row_end - 1) xr0 = row_end - 1;  // rows past the expert's end duplicate its last row
     if (xr1 > row_end - 1) xr1 = row_end - 1;
+    if (a.row_src) {  // the rows' values lie in their tokens' rows
+        xr0 = a.row_src[xr0];
+        xr1 = a.row_src[xr1];
+    }
     const int8_t* xsrc0 = a.x + xr0 * a.K + xchunk * 16;
     const int8_t* xsrc1 = a.x + xr1 * a.K + xchunk * 16;
     // operand reads of this lane: token l % 32 of a block, K half l / 32, K step s -> chunk 2 s + l / 32

@@ -114,7 +114,8 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
                                                            int nbits, const int32_t* __restrict__ chunk_start,
                                                            const int32_t* __restrict__ off,
                                                            const int32_t* __restrict__ pbase, int cpp,
-                                                           int32_t* __restrict__ dst)
+                                                           int32_t* __restrict__ dst, int32_t* __restrict__ row_token,
+                                                           int top_k)
 {
     extern __shared__ int32_t cursor[];  // [E] next free row of each expert for this chunk
     const int lane = threadIdx.x;
@@ -148,6 +149,7 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
             }
             start = __shfl(start, leader, 64);
             dst[f] = start + rank;
+            if (row_token) row_token[start + rank] = (int32_t)(f / top_k);
         } else if (f < R) {
             dst[f] = (int32_t)R;  // dropped pair: one past the last row
         }
@@ -357,6 +359,35 @@ extern "C" size_t moe355_init_routing_workspace(int64_t num_tokens, int top_k, i
     return align256(n * (size_t)num_experts * 4) + align256(((size_t)num_experts + 1) * 4) + align256(pb * 4);
 }
 
+// histogram, scan, stable scatter: destinations of the pairs, optionally the token of every sorted row, counts
+static void launch_maps(const int32_t* expert_idx, int64_t R, int E, int top_k, int tokens_num_type, const RouteWs& ws,
+                        int nch, int parts, int cpp, int nbits, int32_t* expanded_row_idx, int32_t* row_token,
+                        int64_t* expert_tokens, hipStream_t st)
+{
+    hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E, ws.chunk_hist);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), ((size_t)E + 256 + (size_t)parts * E) * 4, st,
+                       ws.chunk_hist, nch, E, parts, cpp, tokens_num_type, ws.off, ws.pbase, expert_tokens);
+    hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
+                       ws.chunk_hist, ws.off, ws.pbase, cpp, expanded_row_idx, row_token, top_k);
+}
+
+// the workspace cut into the three arrays of the routing kernels, and how the scan is partitioned
+static RouteWs route_ws_of(void* workspace, int64_t R, int E, int& nch, int& parts, int& cpp, int& nbits)
+{
+    nch = nchunks_of(R > 0 ? R : 1);
+    RouteWs ws;
+    ws.chunk_hist = (int32_t*)workspace;
+    ws.off = (int32_t*)((char*)workspace + align256((size_t)nch * E * 4));
+    ws.pbase = (int32_t*)((char*)ws.off + align256(((size_t)E + 1) * 4));
+    parts = E < kScanThreads ? kScanThreads / E : 1;
+    if (parts > nch) parts = nch;
+    cpp = (nch + parts - 1) / parts;
+    parts = (nch + cpp - 1) / cpp;  // no empty partition
+    nbits = 0;
+    while ((1 << nbits) < E) ++nbits;
+    return ws;
+}
+
 static int init_routing_impl(const void* x, int x_dtype, int64_t num_tokens, int64_t hidden,
                              const int32_t* expert_idx, int top_k, int num_experts, int quant_mode,
                              int tokens_num_type, void* expanded_x, int32_t* expanded_row_idx,
@@ -380,17 +411,8 @@ static int init_routing_impl(const void* x, int x_dtype, int64_t num_tokens, int
 
     hipStream_t st = (hipStream_t)stream;
     const int E = num_experts;
-    const int nch = nchunks_of(R > 0 ? R : 1);
-    RouteWs ws;
-    ws.chunk_hist = (int32_t*)workspace;
-    ws.off = (int32_t*)((char*)workspace + align256((size_t)nch * E * 4));
-    ws.pbase = (int32_t*)((char*)ws.off + align256(((size_t)E + 1) * 4));
-    int parts = E < kScanThreads ? kScanThreads / E : 1;
-    if (parts > nch) parts = nch;
-    const int cpp = (nch + parts - 1) / parts;
-    parts = (nch + cpp - 1) / cpp;  // no empty partition
-    int nbits = 0;
-    while ((1 << nbits) < E) ++nbits;
+    int nch, parts, cpp, nbits;
+    const RouteWs ws = route_ws_of(workspace, R, E, nch, parts, cpp, nbits);
 
     if (R <= kSmallMaxIters * 256) {
         const dim3 grid((unsigned)num_tokens + 1);
@@ -409,11 +431,8 @@ static int init_routing_impl(const void* x, int x_dtype, int64_t num_tokens, int
                                top_k, expanded_x, dynamic_scale);
         return launch_status();
     }
-    hipLaunchKernelGGL(route_hist_kernel, dim3(nch), dim3(256), (size_t)E * 4, st, expert_idx, R, E, ws.chunk_hist);
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), ((size_t)E + 256 + (size_t)parts * E) * 4, st,
-                       ws.chunk_hist, nch, E, parts, cpp, tokens_num_type, ws.off, ws.pbase, expert_tokens);
-    hipLaunchKernelGGL(route_scatter_kernel, dim3(nch), dim3(64), (size_t)E * 4, st, expert_idx, R, E, nbits,
-                       ws.chunk_hist, ws.off, ws.pbase, cpp, expanded_row_idx);
+    launch_maps(expert_idx, R, E, top_k, tokens_num_type, ws, nch, parts, cpp, nbits, expanded_row_idx, nullptr,
+                expert_tokens, st);
     if (quant_mode == 1 && x_dtype == MOE355_DT_F16)
         hipLaunchKernelGGL((gather_rows_kernel<true, MOE355_DT_F16>), dim3((unsigned)num_tokens), dim3(256), 0, st,
                            (const uint16_t*)x, hidden, top_k, expanded_row_idx, expanded_x, dynamic_scale);
@@ -435,6 +454,27 @@ extern "C" int moe355_init_routing(const void* x, int x_dtype, int64_t num_token
     return init_routing_impl(x, x_dtype, num_tokens, hidden, expert_idx, top_k, num_experts, quant_mode,
                              tokens_num_type, expanded_x, expanded_row_idx, expert_tokens, dynamic_scale, workspace,
                              workspace_bytes, stream);
+}
+
+extern "C" int moe355_route_map(const int32_t* expert_idx, int64_t num_tokens, int top_k, int num_experts,
+                                int tokens_num_type, int32_t* expanded_row_idx, int32_t* row_token,
+                                int64_t* expert_tokens, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (num_tokens < 0 || top_k <= 0 || num_experts <= 0) return MOE355_E_ARG;
+    if (tokens_num_type != 0 && tokens_num_type != 1) return MOE355_E_UNSUPPORTED;
+    if (top_k > 64 || num_experts > 2048) return MOE355_E_SHAPE;
+    const int64_t R = num_tokens * top_k;
+    if (R >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (!expert_tokens) return MOE355_E_ARG;
+    if (!workspace || ((uintptr_t)workspace & 255) ||
+        workspace_bytes < moe355_init_routing_workspace(num_tokens, top_k, num_experts))
+        return MOE355_E_WORKSPACE;
+    if (R > 0 && (!expert_idx || !expanded_row_idx || !row_token)) return MOE355_E_ARG;
+    int nch, parts, cpp, nbits;
+    const RouteWs ws = route_ws_of(workspace, R, num_experts, nch, parts, cpp, nbits);
+    launch_maps(expert_idx, R, num_experts, top_k, tokens_num_type, ws, nch, parts, cpp, nbits, expanded_row_idx,
+                row_token, expert_tokens, (hipStream_t)stream);
+    return launch_status();
 }
 
 extern "C" int moe355_init_routing_prequant(const int8_t* x, const float* x_scale, int64_t num_tokens, int64_t hidden,

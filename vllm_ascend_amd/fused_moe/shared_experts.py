@@ -39,9 +39,11 @@ class AscendSharedExperts(torch.nn.Module):
         self.swiglu_limit = swiglu_limit
         self.multistream_overlap = multistream_overlap
 
-    def _mlp(self, hidden_states: torch.Tensor) -> torch.Tensor:
+    def _mlp(self, hidden_states: torch.Tensor, quantized=None) -> torch.Tensor:
         original_dtype = hidden_states.dtype
-        quantized_x, pertoken_scale = npu_ops.npu_dynamic_quant(hidden_states)
+        # quantized: (int8 rows, scales) of these hidden states when the caller has them already (the routed
+        # experts quantise the same rows with the same per-token rule)
+        quantized_x, pertoken_scale = quantized if quantized is not None else npu_ops.npu_dynamic_quant(hidden_states)
         acc = npu_ops.npu_quant_matmul(quantized_x, self.gate_up_weight, self.gate_up_scale_fp32,
                                        pertoken_scale=None, bias=None, output_dtype=torch.int32)
         quantized_x, swiglu_out_scale = torch.ops._C_ascend.npu_dequant_swiglu_quant(
@@ -51,18 +53,21 @@ class AscendSharedExperts(torch.nn.Module):
         return npu_ops.npu_quant_matmul(quantized_x, self.down_weight, self.down_scale_fp32,
                                         pertoken_scale=swiglu_out_scale, bias=None, output_dtype=original_dtype)
 
-    def forward(self, hidden_states: torch.Tensor, before_routed_experts_evt=None) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, before_routed_experts_evt=None, quantized=None) -> torch.Tensor:
         if not self.multistream_overlap:
-            return self._mlp(hidden_states)
+            return self._mlp(hidden_states, quantized)
         side = shared_experts_calculation_stream()
         main = torch.cuda.current_stream()
         if before_routed_experts_evt is None:
             before_routed_experts_evt = main.record_event()
         with torch.cuda.stream(side):
             side.wait_event(before_routed_experts_evt)
-            out = self._mlp(hidden_states)
+            out = self._mlp(hidden_states, quantized)
             done = side.record_event()
         hidden_states.record_stream(side)
+        if quantized is not None:
+            for t in quantized:
+                t.record_stream(side)
         out.record_stream(main)
         self._done_evt = done
         return out

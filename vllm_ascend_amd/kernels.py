@@ -164,6 +164,25 @@ def init_routing_prequant(xq, x_scale, expert_idx, num_experts, tokens_num_type)
     return xs, row_idx, tokens, scale
 
 
+def route_map(expert_idx, num_experts, tokens_num_type):
+    """The maps of the permutation, nothing moved: (expanded_row_idx [T*k] pair -> sorted row, row_token [T*k]
+    sorted row -> token, expert_tokens [E])."""
+    expert_idx = _dev(expert_idx, "expert_idx")
+    if expert_idx.dtype != torch.int32:
+        expert_idx = expert_idx.to(torch.int32)
+    lib = _lib.load()
+    T, k = expert_idx.shape
+    dev = expert_idx.device
+    row_idx = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    row_token = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    tokens = torch.empty((num_experts,), dtype=torch.int64, device=dev)
+    nbytes = lib.moe355_init_routing_workspace(T, k, num_experts)
+    ws = _workspace(nbytes, dev)
+    check(lib.moe355_route_map(_ptr(expert_idx), T, k, num_experts, tokens_num_type, _ptr(row_idx), _ptr(row_token),
+                               _ptr(tokens), _ptr(ws), nbytes, _stream(expert_idx)), "moe355_route_map")
+    return row_idx, row_token, tokens
+
+
 def route_quant_small_supported(num_tokens: int, top_k: int, num_experts: int) -> bool:
     return bool(_lib.load().moe355_route_quant_small_supported(num_tokens, top_k, num_experts))
 

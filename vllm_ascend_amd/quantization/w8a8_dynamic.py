@@ -86,6 +86,9 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         moe_comm_method = _EXTRA_CTX.moe_comm_method
         if moe_comm_method is None:
             raise RuntimeError("no MoE communication method is set up (call setup_moe_comm_method first)")
+        if (getattr(layer, "use_fused_small_batch", True) and shared_experts_input is None
+                and self._plain_call(layer, x) and topk_ids.dim() == 2 and topk_ids.shape[0] == x.shape[0]):
+            return self._apply_row_map(layer, x, topk_weights, topk_ids, shared_experts)
         shared_out = None
         if shared_experts is not None:
             # the shared expert sees the same hidden states unless the caller hands over others
@@ -112,26 +115,75 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 w2_scale=layer.w2_weight_scale_list if self.use_expert_weight_list else [layer.w2_weight_scale_fp32],
             ))
 
-    # ------------------------------------------------------------------ small batches (decode)
-    def supports_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
-        """Whether ``apply_small_batch`` can take this call: plain W8A8 weights (no per-expert lists), 16-bit
-        hidden states as a [T, H] matrix, none of the optional inputs of ``apply``, SiLU, and a batch of at most
-        1024 (token, slot) pairs over at most 256 experts."""
-        from .. import kernels
-
-        if self.use_expert_weight_list or not x.is_cuda or x.dim() != 2 or router_logits.dim() != 2:
+    # ------------------------------------------------------------------ token rows quantised once, read through a map
+    def _plain_call(self, layer, x: torch.Tensor) -> bool:
+        """Plain W8A8 weights (no per-expert lists), 16-bit hidden states as a [T, H] matrix, none of the optional
+        inputs of ``apply``, SiLU: the calls whose token rows need not be copied k times."""
+        if self.use_expert_weight_list or not x.is_cuda or x.dim() != 2 or x.shape[0] == 0:
             return False
         if x.dtype not in (torch.bfloat16, torch.float16) or x.dtype != self.in_dtype:
-            return False
-        if router_logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
             return False
         if (getattr(layer, "apply_router_weight_on_input", False) or getattr(layer, "ascend_pertoken_scale", None)
                 is not None or getattr(layer, "ascend_expert_map", None) is not None
                 or getattr(layer, "ascend_mc2_mask", None) is not None
-                or getattr(layer, "global_redundant_expert_num", 0) or getattr(layer, "enable_force_load_balance", False)):
+                or getattr(layer, "global_redundant_expert_num", 0)):
             return False
         act = getattr(layer, "activation", "silu")
-        if (getattr(act, "value", act) or "silu") != "silu":
+        return (getattr(act, "value", act) or "silu") == "silu"
+
+    def _apply_row_map(self, layer, x: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+                       shared_experts: Any | None = None):
+        """``apply`` without the permuted copy of the activations: every token row is quantised once
+        (the k copies that ``npu_moe_init_routing_v2(quant_mode=1)`` writes hold the same bytes and the same
+        scale), the routing step only builds the two index maps, and the gate_up GEMM reads its rows through the
+        row -> token map.  The shared expert takes the same quantised rows.  Same results, bit for bit, as the
+        op-by-op path (``vllm_ascend/ops/fused_moe/moe_comm_method.py:117-162``)."""
+        from .. import kernels
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        stream = torch.cuda.current_stream()
+        before_dispatch_evt = stream.record_event()
+        xq, x_scale = kernels.dynamic_quant(x)
+        shared_out = None
+        if shared_experts is not None:
+            shared_out = shared_experts(x, quantized=(xq, x_scale))
+        expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, layer.w13_weight.shape[0], 1)
+        return self._experts_on_row_map(layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens,
+                                        topk_weights, shared_experts, shared_out, before_dispatch_evt)
+
+    def _experts_on_row_map(self, layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens, topk_weights,
+                            shared_experts, shared_out, before_dispatch_evt):
+        from .. import kernels
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        stream = torch.cuda.current_stream()
+        w13, w2 = layer.w13_weight, layer.w2_weight
+        cfg = getattr(layer, "moe_config", None)
+        swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
+        q1, q1_scale = kernels.gmm1_swiglu_quant_gather(xq, x_scale, row_token, w13, layer.w13_weight_scale_fp32,
+                                                        expert_tokens, 1, w13.shape[2], w13.shape[1], swiglu_limit)
+        before_gmm2_evt = stream.record_event()
+        out = kernels.gmm2_dequant(q1, w2, layer.w2_weight_scale_fp32, q1_scale, expert_tokens, 1, w2.shape[2],
+                                   w2.shape[1], out_dtype=x.dtype)
+        before_combine_evt = stream.record_event()
+        if shared_experts is not None and shared_out is not None:
+            shared_experts.wait()
+        routed_out = kernels.token_unpermute(out, expanded_row_idx, topk_weights, shared_out)
+        return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
+                                  before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
+                                  group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
+
+    # ------------------------------------------------------------------ small batches (decode)
+    def supports_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
+        """Whether ``apply_small_batch`` can take this call: a plain call (see ``_plain_call``), no forced load
+        balance, and a batch of at most 1024 (token, slot) pairs over at most 256 experts."""
+        from .. import kernels
+
+        if not self._plain_call(layer, x) or router_logits.dim() != 2:
+            return False
+        if router_logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            return False
+        if getattr(layer, "enable_force_load_balance", False):
             return False
         return kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
 
@@ -162,22 +214,12 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
             sync_counter=counter)
         shared_out = None
         if shared_experts is not None:
-            shared_out = shared_experts(x if shared_experts_input is None else shared_experts_input)
-        w13, w2 = layer.w13_weight, layer.w2_weight
-        cfg = getattr(layer, "moe_config", None)
-        swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
-        q1, q1_scale = kernels.gmm1_swiglu_quant_gather(xq, x_scale, row_token, w13, layer.w13_weight_scale_fp32,
-                                                        expert_tokens, 1, w13.shape[2], w13.shape[1], swiglu_limit)
-        before_gmm2_evt = stream.record_event()
-        out = kernels.gmm2_dequant(q1, w2, layer.w2_weight_scale_fp32, q1_scale, expert_tokens, 1, w2.shape[2],
-                                   w2.shape[1], out_dtype=x.dtype)
-        before_combine_evt = stream.record_event()
-        if shared_experts is not None and shared_out is not None:
-            shared_experts.wait()
-        routed_out = kernels.token_unpermute(out, expanded_row_idx, topk_weights, shared_out)
-        return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
-                                  before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
-                                  group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
+            if shared_experts_input is None:
+                shared_out = shared_experts(x, quantized=(xq, x_scale))
+            else:
+                shared_out = shared_experts(shared_experts_input)
+        return self._experts_on_row_map(layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens,
+                                        topk_weights, shared_experts, shared_out, before_dispatch_evt)
 
     @staticmethod
     def get_eplb_weight_views(layer) -> list:
