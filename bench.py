@@ -67,11 +67,9 @@ def algorithmic_bytes_gmm1(cfg, counts) -> int:
     active = int((counts > 0).sum())
     R = int(counts.sum())
     w = int(active * weight_bytes(cfg, 2 * cfg.I, cfg.H))
-    if cfg.w4_group < 0:
-        # int8 weights: the token rows are quantised once and read through the row -> token map
-        act_in = cfg.T * cfg.H + cfg.T * 4 + R * 4
-    else:
-        act_in = R * cfg.H + R * 4
+    # the sorted int8 rows and their scales, as the op is defined (the plain W8A8 path reads fewer bytes than that:
+    # it keeps one quantised row per token and a row -> token map)
+    act_in = R * cfg.H + R * 4
     act_out = R * cfg.I + R * 4
     return w + act_in + act_out
 
@@ -91,11 +89,11 @@ def layer_bytes(cfg, counts) -> int:
     w = int(active * (weight_bytes(cfg, 2 * cfg.I, cfg.H) + weight_bytes(cfg, cfg.H, cfg.I)))
     if cfg.shared:
         w += 2 * cfg.I * cfg.H + cfg.H * cfg.I + (2 * cfg.I + cfg.H) * 4
-    # tokens in, quantised (once for int8 weights, one copy per pair otherwise) and read back, SwiGLU values
-    # re-quantised and read back, expert outputs written and combined
-    rows_q = T if cfg.w4_group < 0 else R
-    act = (T * cfg.H * 2 + T * cfg.E * 4 + 2 * rows_q * cfg.H + 2 * rows_q * 4 + 2 * R * 4 + 2 * R * cfg.I
-           + 2 * R * 4 + 2 * R * cfg.H * 2 + T * cfg.H * 2)
+    # tokens and logits in, sorted int8 rows and scales written and read, int8 SwiGLU rows and scales written and
+    # read, expert outputs written and read, result out: the accounting of the operator sequence, whatever part
+    # of it a fused path avoids
+    act = (T * cfg.H * 2 + T * cfg.E * 4 + 2 * R * cfg.H + 2 * R * 4 + 2 * R * cfg.I + 2 * R * 4
+           + 2 * R * cfg.H * 2 + T * cfg.H * 2)
     return w + act
 
 
