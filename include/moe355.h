@@ -309,7 +309,11 @@ int moe355_gmm2_dequant_w4(const int8_t *x, const uint8_t *weight_nz4, const flo
 /* Raw int32 accumulators of the same grouped product (no epilogue):
  * acc [R, N] int32.  The integer stage of both ops above, exposed so a caller
  * can check it exactly (the reference keeps the same intermediate in a global
- * workspace: grouped_matmul_swiglu_quant.h:119,234-265). */
+ * workspace: grouped_matmul_swiglu_quant.h:119,234-265).  The workspace is optional
+ * (NULL / 0 is accepted and only costs speed): moe355_gmm_i32_workspace() bytes let the
+ * call use the tiled kernels and, for one expert with at most 64 rows, partial sums per
+ * slab of K instead of atomics. */
+size_t moe355_gmm_i32_workspace(int64_t rows, int64_t n, int64_t k, int num_experts);
 int moe355_gmm_i32(const int8_t *x, const int8_t *weight_nz, const int64_t *group_list, int group_list_type,
                    int64_t rows, int64_t k, int64_t n, int num_experts, int32_t *acc, void *workspace,
                    size_t workspace_bytes, void *stream);

@@ -313,6 +313,34 @@ def test_gmm_i32(K, orc, R, E, Kd, N, layout):
     assert np.array_equal(acc2.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("R,Kd,N,rows", [(64, 7168, 256, 64), (33, 2048, 1024, 20), (1, 4096, 128, 1), (48, 2048, 128, 0)])
+def test_gmm_i32_dense_few_rows_with_and_without_scratch(K, orc, R, Kd, N, rows):
+    """One expert, at most 64 rows, long K: K is cut into slabs.  With the scratch of moe355_gmm_i32_workspace() the
+    slabs' partial sums are stored and added up, without any scratch they are added with atomics; both are the
+    checker's sums, and the rows behind the expert's last one are zero."""
+    from vllm_ascend_amd import _lib
+    from vllm_ascend_amd._lib import W_ENK
+
+    g = torch.Generator().manual_seed(R + Kd + N)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (1, N, Kd), generator=g, dtype=torch.int8)
+    cnt = torch.tensor([rows], dtype=torch.int64)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cnt.numpy())
+    ref[rows:] = 0
+    acc = K.gmm_i32(x.to(DEV), wnz, cnt.to(DEV), 1, N, Kd)
+    lib = _lib.load()
+    xd, cd = x.to(DEV), cnt.to(DEV)
+    acc2 = torch.full((R, N), 7, dtype=torch.int32, device=DEV)
+    rc = lib.moe355_gmm_i32(xd.data_ptr(), wnz.data_ptr(), cd.data_ptr(), 1, R, Kd, N, 1, acc2.data_ptr(), None, 0,
+                            torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    got2 = acc2.cpu().numpy()
+    assert np.array_equal(got2[:rows], ref[:rows])
+
+
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
 def test_gmm1_swiglu_quant(K, orc, R, E, Kd, N):
     print(f"gmm1 R={R} E={E} K={Kd} N={N}", flush=True)

@@ -65,6 +65,7 @@ PROTOTYPES = {
     "moe355_gmm2_dequant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "moe355_gmm2_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64,
                                     c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "moe355_gmm_i32_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "moe355_gmm_i32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p,
                                c_void_p, c_size_t, c_void_p]),
     "moe355_dequant_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p,

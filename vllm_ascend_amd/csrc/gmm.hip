@@ -173,7 +173,12 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
             }
             const int ch = quad_channel(wave, lane);
             if (EPI == EPI_I32 && gridDim.y > 1) {
-                if (valid) {
+                if (valid && a.acc_part) {
+                    // the slab's partial sums to its own plane of the scratch; slab_sum_kernel adds the planes
+                    int32_t* plane = a.acc_part + ((int64_t)blockIdx.y * a.R + row) * a.N;
+                    *(v4i*)(plane + nb0 * 32 + ch) = (v4i){g[0], g[1], g[2], g[3]};
+                    *(v4i*)(plane + nb1 * 32 + ch) = (v4i){u[0], u[1], u[2], u[3]};
+                } else if (valid) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         atomicAdd(a.acc + row * a.N + nb0 * 32 + ch + j, g[j]);
@@ -311,6 +316,26 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, 
     if (i < n4) ((v4i*)p)[i] = (v4i){0, 0, 0, 0};
 }
 
+// acc = sum of the slabs' planes, for the rows of the one expert (gl[0] of them: count and running sum are the
+// same number for one expert); the other rows become zero.  Integer sums: exact in any order.
+__global__ __launch_bounds__(256) void slab_sum_kernel(const int32_t* __restrict__ part, int slabs, int64_t R, int N,
+                                                       const int64_t* __restrict__ gl, int32_t* __restrict__ acc)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte piece of acc
+    const int64_t n4 = R * (int64_t)N / 4;
+    if (i >= n4) return;
+    int64_t rows = gl[0];
+    if (rows > R) rows = R;
+    v4i s = {0, 0, 0, 0};
+    if (i * 4 / N < rows) {
+        for (int p = 0; p < slabs; ++p) {
+            const v4i v = ((const v4i*)(part + (int64_t)p * R * N))[i];
+            s = (v4i){s[0] + v[0], s[1] + v[1], s[2] + v[2], s[3] + v[3]};
+        }
+    }
+    ((v4i*)acc)[i] = s;
+}
+
 template <typename KernelT>
 static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs& a)
 {
@@ -350,9 +375,23 @@ static size_t tiled_ws_max(int64_t rows, int E)
     return tiled_workspace_bytes(rows, E, 64);  // the smallest tile needs the longest tile list
 }
 
-template <int EPI>
-static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
+// K slabs of the dense few-row product (one expert, at most 64 rows, a long K, too few pairs of tiles to fill
+// the chip); 1 = not that case
+static int dense_slabs(int64_t R, int K, int N, int E)
 {
+    const int64_t units = (int64_t)E * (N / 64);
+    const int KB = K >> 5;
+    if (E != 1 || R > 64 || units >= 256 || units < 1 || KB < 64) return 1;
+    int slabs = (int)(512 / units);
+    if (slabs > KB / 8) slabs = KB / 8;
+    return slabs < 1 ? 1 : slabs;
+}
+
+template <int EPI>
+static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, void* part_ws = nullptr,
+                            size_t part_bytes = 0)
+{
+    GmmArgs a = a_in;
     int bm = tile_ws ? tiled_bm(a) : 0;
     if (EPI == EPI_I32 && a.E == 1 && a.R <= 64 && (a.K >> 5) >= 64 && a.N / 64 < 256) bm = 0;  // dense, few rows
     if (bm) {
@@ -366,14 +405,20 @@ static int launch_gemm_auto(const GmmArgs& a, void* tile_ws, hipStream_t st)
         // One expert with at most 64 rows (the shared expert of a decode batch: a dense product over a few tokens):
         // too few workgroups for a chip that needs thousands of loads in flight to stream at full rate.  K is cut
         // into slabs, one workgroup per (pair of tiles, slab), partial sums added into the zeroed result.
-        const int KB = a.K >> 5;
-        if (a.E == 1 && a.R <= 64 && units < 256 && KB >= 64) {
-            int slabs = (int)(512 / units);
-            if (slabs > KB / 8) slabs = KB / 8;
+        {
+            const int slabs = dense_slabs(a.R, a.K, a.N, a.E);
             if (slabs > 1) {
                 const int64_t n4 = a.R * (int64_t)a.N / 4;  // N % 64 == 0
-                hipLaunchKernelGGL(zero_i32_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, a.acc, n4);
+                const dim3 cover((unsigned)((n4 + 255) / 256));
+                // with scratch for one plane per slab the partial sums are stored and added up afterwards;
+                // without, they are added into the zeroed result with atomics (32 of 47 us at 8 slabs)
+                const bool planes = part_ws && part_bytes >= (size_t)slabs * a.R * a.N * 4;
+                if (planes) a.acc_part = (int32_t*)part_ws;
+                else hipLaunchKernelGGL(zero_i32_kernel, cover, dim3(256), 0, st, a.acc, n4);
                 launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units, (unsigned)slabs), st, a);
+                if (planes)
+                    hipLaunchKernelGGL(slab_sum_kernel, cover, dim3(256), 0, st, a.acc_part, slabs, a.R, a.N, a.gl,
+                                       a.acc);
                 return launch_status();
             }
         }
@@ -443,10 +488,12 @@ extern "C" int moe355_gmm_i32(const int8_t* x, const int8_t* weight_nz, const in
     if (rc != MOE355_OK) return rc;
     if (rows == 0) return MOE355_OK;
     if (!acc || ((uintptr_t)acc & 15)) return MOE355_E_ARG;
-    // the tile map is optional here: without (enough) scratch the streaming kernel is used
-    void* tile_ws = (workspace && !((uintptr_t)workspace & 255) && workspace_bytes >= tiled_ws_max(rows, num_experts))
-                        ? workspace
-                        : nullptr;
+    // the scratch is optional here: without enough of it for the tile map the streaming kernel is used, and
+    // what lies behind the tile map serves the partial sums of a product that cuts K into slabs
+    const size_t map_bytes = (tiled_ws_max(rows, num_experts) + 255) & ~(size_t)255;
+    void* tile_ws = (workspace && !((uintptr_t)workspace & 255) && workspace_bytes >= map_bytes) ? workspace : nullptr;
+    void* part_ws = (tile_ws && workspace_bytes > map_bytes) ? (char*)workspace + map_bytes : nullptr;
+    const size_t part_bytes = part_ws ? workspace_bytes - map_bytes : 0;
     GmmArgs a = {};
     a.x = x;
     a.w = weight_nz;
@@ -457,7 +504,16 @@ extern "C" int moe355_gmm_i32(const int8_t* x, const int8_t* weight_nz, const in
     a.N = (int)n;
     a.E = num_experts;
     a.acc = acc;
-    return launch_gemm_auto<EPI_I32>(a, tile_ws, (hipStream_t)stream);
+    return launch_gemm_auto<EPI_I32>(a, tile_ws, (hipStream_t)stream, part_ws, part_bytes);
+}
+
+extern "C" size_t moe355_gmm_i32_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)
+{
+    if (rows <= 0 || n <= 0 || num_experts <= 0) return 256;
+    size_t bytes = (tiled_ws_max(rows, num_experts) + 255) & ~(size_t)255;
+    const int slabs = dense_slabs(rows, (int)k, (int)n, num_experts);
+    if (slabs > 1) bytes += (size_t)slabs * rows * n * 4;  // one plane of partial sums per slab
+    return bytes;
 }
 
 extern "C" size_t moe355_gmm1_swiglu_quant_workspace(int64_t rows, int64_t n, int64_t k, int num_experts)

@@ -35,6 +35,7 @@ struct GmmArgs {
     float limit;            // swiglu clamp
     // outputs
     int32_t* acc;           // EPI_I32   [R, N]
+    int32_t* acc_part;      // EPI_I32 with K cut into slabs: [slabs][R, N] partial sums (or null: atomics into acc)
     float* y;               // EPI_SWIGLU [R, N/2] fp32 SwiGLU values
     uint16_t* out;          // EPI_DEQUANT [R, N] bf16, or fp16 when out_f16 is set
     int out_f16;

@@ -350,7 +350,7 @@ def gmm_i32(x, weight_nz, group_list, group_list_type, n, k):
     _check_gmm_operands("gmm_i32", x, rows, k, n, E, group_list, weight=weight_nz, weight_numel=E * n * k)
     x = _dev(x, "x")
     acc = torch.zeros((rows, n), dtype=torch.int32, device=x.device)
-    ws = _workspace(lib.moe355_gmm2_dequant_workspace(rows, n, k, E), x.device)
+    ws = _workspace(lib.moe355_gmm_i32_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm_i32(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_gl(group_list)),
                              _gl_type(group_list_type), rows, k, n, E, _ptr(acc), _ptr(ws), ws.numel(), _stream(x)),
           "moe355_gmm_i32")
