@@ -28,7 +28,8 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
     }
     __syncthreads();
     const int64_t nv = H >> 3;
-    for (int64_t i = threadIdx.x; i < nv; i += 256) {
+    // few tokens: a row is cut into gridDim.y pieces, one workgroup each
+    for (int64_t i = (int64_t)blockIdx.y * 256 + threadIdx.x; i < nv; i += 256 * (int64_t)gridDim.y) {
         float acc[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
@@ -88,8 +89,17 @@ extern "C" int moe355_token_unpermute(const void* permuted, int dtype, const int
     if (num_tokens == 0) return MOE355_OK;
     if (!permuted || !sorted_indices || !out) return MOE355_E_ARG;
     if (((uintptr_t)permuted & 15) || ((uintptr_t)out & 15) || ((uintptr_t)residual & 15)) return MOE355_E_SHAPE;
+    // one workgroup per token when the tokens alone fill the chip; otherwise the rows are cut into pieces of 256
+    // 16-byte vectors until there are about 1024 workgroups
+    unsigned pieces = 1;
+    if (num_tokens < 512) {
+        const int64_t per_row = (hidden / 8 + 255) / 256;
+        const int64_t want = (1024 + num_tokens - 1) / num_tokens;
+        pieces = (unsigned)(per_row < want ? per_row : want);
+        if (pieces < 1) pieces = 1;
+    }
 #define MOE355_UNPERMUTE(K, D)                                                                                    \
-    hipLaunchKernelGGL((token_unpermute_kernel<K, D>), dim3((unsigned)num_tokens), dim3(256), 0, (hipStream_t)stream, \
+    hipLaunchKernelGGL((token_unpermute_kernel<K, D>), dim3((unsigned)num_tokens, pieces), dim3(256), 0, (hipStream_t)stream, \
                        (const uint16_t*)permuted, sorted_indices, (const uint16_t*)probs, top_k, hidden,             \
                        permuted_rows, (const uint16_t*)residual, (uint16_t*)out)
     if (dtype == MOE355_DT_F16) {

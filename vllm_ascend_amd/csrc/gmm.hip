@@ -393,7 +393,9 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
 {
     GmmArgs a = a_in;
     int bm = tile_ws ? tiled_bm(a) : 0;
-    if (EPI == EPI_I32 && a.E == 1 && a.R <= 64 && (a.K >> 5) >= 64 && a.N / 64 < 256) bm = 0;  // dense, few rows
+    // dense, few rows (the shared expert of a decode batch): a 64-row tile map gives one workgroup per 256
+    // channels, the streaming kernel one per 64 (and K slabs on top for the int32 form)
+    if (a.E == 1 && a.R <= 64) bm = 0;
     if (bm) {
         launch_tiled_any(EPI, bm, a, tile_ws, st, t_ev_start, t_ev_stop);
         t_ev_start = nullptr;
@@ -454,7 +456,7 @@ extern "C" const char* moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_
     a.K = (int)k;
     a.N = (int)n;
     a.E = num_experts;
-    const int bm = tiled_bm(a);
+    const int bm = (a.E == 1 && a.R <= 64) ? 0 : tiled_bm(a);  // as launch_gemm_auto decides
     if (bm == 256) return "gmm_wide_kernel";
     if (bm != 0) return "gmm_tiled_kernel";
     return "gmm_stream_kernel";
