@@ -48,7 +48,9 @@ __global__ __launch_bounds__(256) void format_cast_nz_kernel(const int8_t* __res
 }
 
 // ------------------------------------------------------------------ streaming GEMM
-template <int EPI, int KSPLIT, int UN, int OCC>
+// SLABS: K is cut into gridDim.y slabs (the dense few-row int32 product only; reading gridDim costs every
+// wavefront a scalar load in front of its first weight request, 4 us per launch of the decode down GEMM)
+template <int EPI, int KSPLIT, int UN, int OCC, bool SLABS = false>
 __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
 {
     static_assert(KSPLIT == 1 || KSPLIT == 4, "workgroup barriers need all four wavefronts on one unit");
@@ -68,8 +70,11 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     // partial sums into a zeroed result with atomics: integer addition, exact and order free), and a slab into
     // KSPLIT pieces, one per wavefront
     const int ks = (KSPLIT == 1) ? 0 : wave;
-    const int slab_begin = (int)(((int64_t)KB * blockIdx.y) / gridDim.y);
-    const int slab_end = (int)(((int64_t)KB * (blockIdx.y + 1)) / gridDim.y);
+    int slab_begin = 0, slab_end = KB;
+    if constexpr (SLABS) {
+        slab_begin = (int)(((int64_t)KB * blockIdx.y) / gridDim.y);
+        slab_end = (int)(((int64_t)KB * (blockIdx.y + 1)) / gridDim.y);
+    }
     const int kb_begin = slab_begin + ((slab_end - slab_begin) * ks) / KSPLIT;
     const int kb_end = slab_begin + ((slab_end - slab_begin) * (ks + 1)) / KSPLIT;
 
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
                 u[j] = red[(16 + 4 * wave + j) * 64 + lane];
             }
             const int ch = quad_channel(wave, lane);
-            if (EPI == EPI_I32 && gridDim.y > 1) {
+            if constexpr (EPI == EPI_I32 && SLABS) {
                 if (valid && a.acc_part) {
                     // the slab's partial sums to its own plane of the scratch; slab_sum_kernel adds the planes
                     int32_t* plane = a.acc_part + ((int64_t)blockIdx.y * a.R + row) * a.N;
@@ -417,7 +422,7 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
                 const bool planes = part_ws && part_bytes >= (size_t)slabs * a.R * a.N * 4;
                 if (planes) a.acc_part = (int32_t*)part_ws;
                 else hipLaunchKernelGGL(zero_i32_kernel, cover, dim3(256), 0, st, a.acc, n4);
-                launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units, (unsigned)slabs), st, a);
+                launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, true>, dim3((unsigned)units, (unsigned)slabs), st, a);
                 if (planes)
                     hipLaunchKernelGGL(slab_sum_kernel, cover, dim3(256), 0, st, a.acc_part, slabs, a.R, a.N, a.gl,
                                        a.acc);
