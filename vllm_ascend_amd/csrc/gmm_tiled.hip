@@ -17,11 +17,64 @@
 namespace moe355 {
 
 // One workgroup.  Thread t owns experts [t*seg, (t+1)*seg).  Tiles are numbered expert by expert.
+// by_length (the 256-row weight-streaming tiles): the tiles are listed longest first -- 161..192 rows, 129..160,
+// up to 128, then the tall ones (more than 192 rows, which become two shorter column items) -- so that the
+// workgroups that start last are the short ones and the compute units finish closer together.
 __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict__ gl, int gl_type, int E, int BM,
-                                                       int max_tiles, TileMap tm)
+                                                       int max_tiles, TileMap tm, int by_length = 0)
 {
     __shared__ int32_t part_rows[16];
     __shared__ int32_t part_tiles[16];
+    if (by_length) {
+        // class of a tile with m rows left in its expert; per-thread counts per class, two classes per scan
+        auto cls = [](int64_t m) -> int { return m > 192 ? 3 : (m > 160 ? 0 : (m > 128 ? 1 : 2)); };
+        const int tid = threadIdx.x;
+        const int seg = (E + 255) / 256;
+        const int e0 = tid * seg;
+        auto rows_of = [&](int e) -> int64_t {
+            int64_t m = (gl_type == MOE355_GL_COUNT) ? gl[e] : gl[e] - (e > 0 ? gl[e - 1] : 0);
+            return m < 0 ? 0 : m;
+        };
+        int32_t rows = 0, n01 = 0, n23 = 0;  // counts packed 16 + 16 bits (at most max_tiles < 32768 tiles)
+        for (int j = 0; j < seg; ++j) {
+            const int e = e0 + j;
+            if (e < E) {
+                const int64_t m = rows_of(e);
+                rows += (int32_t)m;
+                for (int64_t r0 = 0; r0 < m; r0 += BM) {
+                    const int c = cls(m - r0);
+                    if (c < 2) n01 += 1 << (16 * c);
+                    else n23 += 1 << (16 * (c - 2));
+                }
+            }
+        }
+        int32_t all_rows, all01, all23;
+        const int32_t rows_before = block_scan_exclusive_i32(rows, part_rows, all_rows);
+        const int32_t b01 = block_scan_exclusive_i32(n01, part_tiles, all01);
+        const int32_t b23 = block_scan_exclusive_i32(n23, part_tiles, all23);
+        const int32_t total[4] = {all01 & 0xffff, all01 >> 16, all23 & 0xffff, all23 >> 16};
+        const int32_t all_tiles = total[0] + total[1] + total[2] + total[3];
+        if (tid == 0) tm.count[0] = all_tiles < max_tiles ? all_tiles : max_tiles;
+        int32_t next[4] = {b01 & 0xffff, total[0] + (b01 >> 16), total[0] + total[1] + (b23 & 0xffff),
+                           total[0] + total[1] + total[2] + (b23 >> 16)};
+        int64_t row = rows_before;
+        for (int j = 0; j < seg; ++j) {
+            const int e = e0 + j;
+            if (e < E) {
+                const int64_t m = rows_of(e);
+                for (int64_t r0 = 0; r0 < m; r0 += BM) {
+                    const int32_t t = next[cls(m - r0)]++;
+                    if (t < max_tiles) {
+                        tm.expert[t] = e;
+                        tm.row_begin[t] = (int32_t)(row + r0);
+                        tm.row_end[t] = (int32_t)(row + m);
+                    }
+                }
+                row += m;
+            }
+        }
+        return;
+    }
     const int tid = threadIdx.x;
     const int seg = (E + 255) / 256;
     const int e0 = tid * seg;
@@ -603,34 +656,38 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
 }
 
 template <int EPI>
-__global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
+__global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks,
+                                                          int columns)
 {
     extern __shared__ __attribute__((aligned(16))) int8_t wide_lds[];
-    // same XCD-aware walk over (256-row tile, column block of 256 channels) as the 128-row kernel
-    const int total = tm.count[0] * n_col_blocks;
-    const int per_xcd = (total + 7) / 8;
+    // Workgroup i runs on XCD i % 8.  The tiles (listed longest first) go round the XCDs, tile t to XCD t % 8, and
+    // the `columns` workgroups of a tile (a column: 512 channels, two column blocks) follow each other on that XCD,
+    // so they run at the same time and share the tile's tokens in its L2.  Nothing here depends on the number of
+    // tiles: the tile's entries are requested together with the count they are checked against.
     const int slot = (int)(blockIdx.x / 8);
-    const int item = (int)(blockIdx.x % 8) * per_xcd + slot;
-    if (slot >= per_xcd || item >= total) return;
-    const int mt = item / n_col_blocks;
-    const int nt = item % n_col_blocks;
+    const int mt = (slot / columns) * 8 + (int)(blockIdx.x % 8);
+    const int col = slot % columns;
+    if (mt >= max_tiles) return;
+    const int count = tm.count[0];
     const int e = tm.expert[mt];
     const int64_t row0 = tm.row_begin[mt];
     int64_t row_end = tm.row_end[mt];
+    if (mt >= count) return;
     if (row_end > a.R) row_end = a.R;
     if (row0 >= row_end) return;
     if (row_end - row0 <= 128) {
-        // a wide tile spans two column blocks: the first half of this tile's workgroups does the work
-        if (nt * 2 >= n_col_blocks) return;
-        stream_tile_body<EPI, true>(a, e, row0, row_end, nt, wide_lds);
+        stream_tile_body<EPI, true>(a, e, row0, row_end, col, wide_lds);
     } else if (row_end - row0 <= 160) {
-        if (nt * 2 >= n_col_blocks) return;
-        stream_tile_body<EPI, true, 5>(a, e, row0, row_end, nt, wide_lds);
+        stream_tile_body<EPI, true, 5>(a, e, row0, row_end, col, wide_lds);
     } else if (row_end - row0 <= 192) {
-        if (nt * 2 >= n_col_blocks) return;
-        stream_tile_body<EPI, true, 6>(a, e, row0, row_end, nt, wide_lds);
+        stream_tile_body<EPI, true, 6>(a, e, row0, row_end, col, wide_lds);
     } else {
-        stream_tile_body<EPI, false>(a, e, row0, row_end, nt, wide_lds);
+        // a tall tile is one column block wide: the column's two blocks one after the other
+        stream_tile_body<EPI, false>(a, e, row0, row_end, 2 * col, wide_lds);
+        if (2 * col + 1 < n_col_blocks) {
+            __syncthreads();  // the first block's epilogue is out of LDS
+            stream_tile_body<EPI, false>(a, e, row0, row_end, 2 * col + 1, wide_lds);
+        }
     }
 }
 
@@ -681,18 +738,18 @@ static void launch_wide(const GmmArgs& a, void* workspace, hipStream_t st, hipEv
     tm.expert = (int32_t*)((char*)workspace + 256);
     tm.row_begin = (int32_t*)((char*)workspace + 256 + arr);
     tm.row_end = (int32_t*)((char*)workspace + 256 + 2 * arr);
-    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm);
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm, 1);
     const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
     const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
     const int n_col_blocks = (channels + per_block - 1) / per_block;
-    const int total = max_tiles * n_col_blocks;
-    const int grid = ((total + 7) / 8) * 8;
+    const int columns = (n_col_blocks + 1) / 2;
+    const int grid = 8 * ((max_tiles + 7) / 8) * columns;  // one workgroup per (tile, column), no idle ones
     if (ev0 && ev1)
         hipExtLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, ev0, ev1, 0, a, tm,
-                              max_tiles, n_col_blocks);
+                              max_tiles, n_col_blocks, columns);
     else
         hipLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, a, tm, max_tiles,
-                           n_col_blocks);
+                           n_col_blocks, columns);
 }
 
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
