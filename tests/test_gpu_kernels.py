@@ -24,7 +24,8 @@ def orc():
     return oracle
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 8), (3, 1024), (64, 2048), (17, 7168), (5, 200), (2, 30)])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (3, 1024), (64, 2048), (17, 7168), (5, 200), (2, 30), (9, 4096), (4, 3080),
+                                       (3, 8192), (2, 8200), (2, 12288)])
 def test_dynamic_quant(K, orc, rows, cols):
     print(f"dynamic_quant rows={rows} cols={cols}", flush=True)
     g = torch.Generator().manual_seed(rows * 1000 + cols)

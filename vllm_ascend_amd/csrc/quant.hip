@@ -22,7 +22,8 @@ __device__ __forceinline__ float block_max_256(float v, float* lds4)
 }
 
 // x [rows, cols] bf16 or fp16 (DT) -> q int8, scale fp32.  VEC: cols % 8 == 0 and 16-byte aligned rows.
-template <bool VEC, int DT>
+// NV > 0 (VEC only): rows of at most NV x 2048 values stay in registers between the two passes.
+template <bool VEC, int DT, int NV = 0>
 __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __restrict__ x, int64_t cols,
                                                                  int8_t* __restrict__ q, float* __restrict__ scale)
 {
@@ -31,6 +32,39 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __re
     const uint16_t* xr = x + row * cols;
     int8_t* qr = q + row * cols;
     float a = 0.0f;
+    if constexpr (VEC && NV > 0) {
+        const int64_t nv = cols >> 3;
+        const v8u16* xv = (const v8u16*)xr;
+        v8u16 held[NV];
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            const int64_t i = threadIdx.x + 256 * n;
+            held[n] = i < nv ? xv[i] : (v8u16){0, 0, 0, 0, 0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float f = __builtin_fabsf(half_to_f32<DT>(held[n][j]));
+                a = f > a ? f : a;
+            }
+        a = block_max_256(a, lds4);
+        const float s = a / 127.0f;
+        if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
+        uint2* qv = (uint2*)qr;
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            const int64_t i = threadIdx.x + 256 * n;
+            uint32_t w[2] = {0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(held[n][j]) / s);
+                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+            }
+            if (i < nv) qv[i] = make_uint2(w[0], w[1]);
+        }
+        return;
+    }
     if constexpr (VEC) {
         const int64_t nv = cols >> 3;
         const v8u16* xv = (const v8u16*)xr;
@@ -148,13 +182,23 @@ extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, in
 #define MOE355_DQ(V_, D_)                                                                                      \
     hipLaunchKernelGGL((dynamic_quant_kernel<V_, D_>), dim3((unsigned)rows), dim3(256), 0, st, (const uint16_t*)x, \
                        cols, q, scale)
+#define MOE355_DQH(D_, N_)                                                                                        \
+    hipLaunchKernelGGL((dynamic_quant_kernel<true, D_, N_>), dim3((unsigned)rows), dim3(256), 0, st,                \
+                       (const uint16_t*)x, cols, q, scale)
     if (x_dtype == MOE355_DT_BF16) {
-        if (vec) MOE355_DQ(true, MOE355_DT_BF16);
+        if (vec && cols <= 2048) MOE355_DQH(MOE355_DT_BF16, 1);
+        else if (vec && cols <= 4096) MOE355_DQH(MOE355_DT_BF16, 2);
+        else if (vec && cols <= 8192) MOE355_DQH(MOE355_DT_BF16, 4);
+        else if (vec) MOE355_DQ(true, MOE355_DT_BF16);
         else MOE355_DQ(false, MOE355_DT_BF16);
     } else {
-        if (vec) MOE355_DQ(true, MOE355_DT_F16);
+        if (vec && cols <= 2048) MOE355_DQH(MOE355_DT_F16, 1);
+        else if (vec && cols <= 4096) MOE355_DQH(MOE355_DT_F16, 2);
+        else if (vec && cols <= 8192) MOE355_DQH(MOE355_DT_F16, 4);
+        else if (vec) MOE355_DQ(true, MOE355_DT_F16);
         else MOE355_DQ(false, MOE355_DT_F16);
     }
+#undef MOE355_DQH
 #undef MOE355_DQ
     return launch_status();
 }
