@@ -241,8 +241,8 @@ def run_workload(name, args, lib, torch, np):
         torch.cuda.synchronize()
         hooked = {"i": 0, "fired": 0}
         # the launchers of the routed gate_up GEMM (small batches read their rows through a row -> token map)
-        hook_names = ["gmm1_swiglu_quant_w4"] if cfg.w4_group >= 0 else ["gmm1_swiglu_quant",
-                                                                          "gmm1_swiglu_quant_gather"]
+        hook_names = (["gmm1_swiglu_quant_w4", "gmm1_swiglu_quant_w4_gather"] if cfg.w4_group >= 0
+                      else ["gmm1_swiglu_quant", "gmm1_swiglu_quant_gather"])
         origs = {h: getattr(K, h) for h in hook_names}
 
         def make_timed(orig, routed):

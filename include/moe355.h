@@ -298,6 +298,15 @@ int moe355_gmm2_dequant_list(const int8_t *x, const int8_t *const *weight_nz_lis
                              int64_t rows, int64_t k, int64_t n, int num_experts, void *out, int out_dtype,
                              void *workspace, size_t workspace_bytes, void *stream);
 
+/* The W4A8 gate_up op on activations quantised in token order and read through the row -> token map, as
+ * moe355_gmm1_swiglu_quant_gather does for int8 weights: x [T, K] int8, x_scale [T], row_token [rows]. */
+int moe355_gmm1_swiglu_quant_w4_gather(const int8_t *x, const float *x_scale, const int32_t *row_token,
+                                       const uint8_t *weight_nz4, const float *weight_scale, int64_t group_size,
+                                       const float *bias, const int64_t *group_list, int group_list_type,
+                                       int64_t rows, int64_t k, int64_t n, int num_experts, float swiglu_limit,
+                                       int8_t *out, float *out_scale, void *workspace, size_t workspace_bytes,
+                                       void *stream);
+
 /* W4A8 down projection:
  *   out[row, col] = bf16( (sum_g float(acc_g) * scale[e, g, col] + bias[e, col]) * per_token_scale[row] )
  * (the int4 form of torch_npu.npu_grouped_matmul as called from vllm_ascend/ops/fused_moe/moe_mlp.py:552-569). */

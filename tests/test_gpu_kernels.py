@@ -518,6 +518,18 @@ def test_w4_gemms_at_chunk_boundaries(K, orc, Kd, N, group, gl_type):
     torch.cuda.synchronize()
     assert np.array_equal(q.cpu().numpy(), q_want)
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+    # the same rows read through a row -> token map from tokens kept in token order
+    T = 37
+    tq = torch.randint(-128, 128, (T, Kd), generator=g, dtype=torch.int8)
+    ts = torch.rand(T, generator=g) * 0.05 + 0.001
+    row_token = torch.randint(0, T, (R,), generator=g, dtype=torch.int32)
+    idx = row_token.long()
+    q_map, s_map = K.gmm1_swiglu_quant_w4_gather(tq.to(DEV), ts.to(DEV), row_token.to(DEV), w4, sg.to(DEV), gsz, gl,
+                                                 gl_type, N, Kd)
+    q_cpy, s_cpy = K.gmm1_swiglu_quant_w4(tq[idx].contiguous().to(DEV), w4, sg.to(DEV), gsz,
+                                          ts[idx].contiguous().to(DEV), gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert torch.equal(q_map, q_cpy) and torch.equal(s_map, s_cpy)
     # with the bias of the offset-corrected A8W4 form (added before the token scale)
     fb = f + np.repeat(bias.numpy(), W4_COUNTS, axis=0)
     got_b = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), gsz, sx.to(DEV), gl, gl_type, N, Kd, bias=bias.to(DEV))

@@ -88,13 +88,16 @@ def test_cpu_tensors_are_refused():
         K.dynamic_quant(torch.zeros(2, 8, dtype=torch.bfloat16))
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("name", ["c5_small", "c5_small_perchannel"])
-def test_w4a8_layer_bit_exact(name):
-    """W4A8 variant (int4 weights, per-group or per-channel scales, Zipf-skewed routing)."""
+def test_w4a8_layer_bit_exact(name, fused):
+    """W4A8 variant (int4 weights, per-group or per-channel scales, Zipf-skewed routing); fused: token rows
+    quantised once and read through the row -> token map, or the op-by-op path with its permuted copy."""
     cfg = CONFIGS[name]
-    print(f"w4a8 layer {name}", flush=True)
+    print(f"w4a8 layer {name} fused={fused}", flush=True)
     d = make_layer(cfg, seed=0)
     layer = build_layer(cfg, d, DEV)
+    layer.use_fused_small_batch = fused
     res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
     torch.cuda.synchronize()
     tr = oracle_layer(cfg, d)

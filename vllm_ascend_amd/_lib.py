@@ -52,6 +52,9 @@ PROTOTYPES = {
     "moe355_gmm1_swiglu_quant_w4": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                             c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                             c_size_t, c_void_p]),
+    "moe355_gmm1_swiglu_quant_w4_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                                                   c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_float,
+                                                   c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe355_gmm2_dequant_w4": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                        c_int64, c_int64, c_int64, c_int, c_void_p, c_int, c_void_p]),
     "moe355_gmm1_swiglu_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),

@@ -267,6 +267,7 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     const int skc = (threadIdx.x >> 4) & 3;
     int64_t sr = row0 + srow;
     if (sr > row1 - 1) sr = row1 - 1;  // rows past the chunk's end repeat its last row (never stored)
+    if (a.row_src) sr = a.row_src[sr];  // the row's values lie in its token's row
     const int8_t* xs = a.x + sr * a.K + skc * 16;
     const int lds_off = ((((skc >> 1) * 2 + (srow >> 5)) * 64) + (skc & 1) * 32 + (srow & 31)) * 16;
     const bool two = row0 + 32 < row1;  // the second token block holds rows (wavefront-uniform)
@@ -392,7 +393,10 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
     // would wait for it: the memory counter retires in order)
     float rs_pre[2];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) rs_pre[b] = a.row_scale[valid[b] ? row[b] : row0];
+    for (int b = 0; b < 2; ++b) {
+        const int64_t r = valid[b] ? row[b] : row0;
+        rs_pre[b] = a.row_scale[a.row_src ? (int64_t)a.row_src[r] : r];
+    }
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
         if (b == 1 && !two) break;
@@ -487,11 +491,11 @@ extern "C" int moe355_w4_offset_correction(const uint8_t* weight_nz4, const floa
     return launch_status();
 }
 
-extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weight_nz4, const float* weight_scale,
-                                           int64_t group_size, const float* bias, const float* x_scale,
-                                           const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
-                                           int64_t n, int num_experts, float swiglu_limit, int8_t* out,
-                                           float* out_scale, void* workspace, size_t workspace_bytes, void* stream)
+static int gmm1_w4_impl(const int8_t* x, const uint8_t* weight_nz4, const float* weight_scale, int64_t group_size,
+                        const float* bias, const float* x_scale, const int64_t* group_list, int group_list_type,
+                        int64_t rows, int64_t k, int64_t n, int num_experts, float swiglu_limit, int8_t* out,
+                        float* out_scale, void* workspace, size_t workspace_bytes, void* stream,
+                        const int32_t* row_src)
 {
     int rc = check_w4(x, weight_nz4, weight_scale, group_list, group_list_type, rows, k, n, num_experts, group_size);
     if (rc != MOE355_OK) return rc;
@@ -510,6 +514,7 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     p.g.N = (int)n;
     p.g.E = num_experts;
     p.g.row_scale = x_scale;
+    p.g.row_src = row_src;
     p.g.limit = swiglu_limit;
     p.g.y = (float*)workspace;
     p.w4 = weight_nz4;
@@ -522,6 +527,28 @@ extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weigh
     launch_w4<EPI_SWIGLU>(p, blocks, st, ev0, ev1);
     launch_swiglu_requant(p.g.y, group_list, group_list_type, num_experts, rows, (int)(n / 2), out, out_scale, st);
     return launch_status();
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_w4(const int8_t* x, const uint8_t* weight_nz4, const float* weight_scale,
+                                           int64_t group_size, const float* bias, const float* x_scale,
+                                           const int64_t* group_list, int group_list_type, int64_t rows, int64_t k,
+                                           int64_t n, int num_experts, float swiglu_limit, int8_t* out,
+                                           float* out_scale, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gmm1_w4_impl(x, weight_nz4, weight_scale, group_size, bias, x_scale, group_list, group_list_type, rows, k,
+                        n, num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_w4_gather(const int8_t* x, const float* x_scale, const int32_t* row_token,
+                                                  const uint8_t* weight_nz4, const float* weight_scale,
+                                                  int64_t group_size, const float* bias, const int64_t* group_list,
+                                                  int group_list_type, int64_t rows, int64_t k, int64_t n,
+                                                  int num_experts, float swiglu_limit, int8_t* out, float* out_scale,
+                                                  void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (rows > 0 && !row_token) return MOE355_E_ARG;
+    return gmm1_w4_impl(x, weight_nz4, weight_scale, group_size, bias, x_scale, group_list, group_list_type, rows, k,
+                        n, num_experts, swiglu_limit, out, out_scale, workspace, workspace_bytes, stream, row_token);
 }
 
 extern "C" int moe355_gmm2_dequant_w4(const int8_t* x, const uint8_t* weight_nz4, const float* scale,

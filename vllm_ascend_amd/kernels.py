@@ -431,6 +431,36 @@ def gmm1_swiglu_quant_w4(x, weight_nz4, weight_scale, group_size, x_scale, group
     return out, out_scale
 
 
+def gmm1_swiglu_quant_w4_gather(xq, x_scale, row_token, weight_nz4, weight_scale, group_size, group_list,
+                                group_list_type, n, k, bias=None, swiglu_limit=0.0):
+    """The W4A8 gate_up op on token rows that were quantised once and are read through the row -> token map."""
+    lib = _lib.load()
+    rows = row_token.shape[0]
+    T = xq.shape[0]
+    E = weight_nz4.shape[0]
+    dev = xq.device
+    groups = k // group_size if group_size else 1
+    _check_gmm_operands("gmm1_swiglu_quant_w4_gather", xq, T, k, n, E, group_list, x_scale, "x_scale", weight_nz4,
+                        E * n * k // 2, weight_scale, E * groups * n)
+    xq = _dev(xq, "x")
+    row_token = _dev(row_token, "row_token")
+    if row_token.dtype != torch.int32:
+        raise ValueError("gmm1_swiglu_quant_w4_gather: row_token must be int32")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != E * n or not bias.is_cuda):
+        raise ValueError(f"gmm1_swiglu_quant_w4_gather: bias must be a float32 GPU tensor of E x N = {E * n} values")
+    out = torch.empty((rows, n // 2), dtype=torch.int8, device=dev)
+    out_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    ws = _workspace(rows * (n // 2) * 4 + 256, dev)
+    check(lib.moe355_gmm1_swiglu_quant_w4_gather(_ptr(xq), _ptr(_dev(x_scale, "x_scale")), _ptr(row_token),
+                                                 _ptr(_dev(weight_nz4, "weight")),
+                                                 _ptr(_dev(weight_scale, "weight_scale")), group_size, _ptr(bias),
+                                                 _ptr(_gl(group_list)), _gl_type(group_list_type), rows, k, n, E,
+                                                 float(swiglu_limit), _ptr(out), _ptr(out_scale), _ptr(ws), ws.numel(),
+                                                 _stream(xq)),
+          "moe355_gmm1_swiglu_quant_w4_gather")
+    return out, out_scale
+
+
 def gmm2_dequant_w4(x, weight_nz4, scale, group_size, per_token_scale, group_list, group_list_type, n, k, bias=None,
                     out_dtype=torch.bfloat16):
     lib = _lib.load()

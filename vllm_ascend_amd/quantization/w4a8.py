@@ -74,6 +74,9 @@ class AscendW4A8DynamicFusedMoEMethod(AscendMoEScheme):
         moe_comm_method = _EXTRA_CTX.moe_comm_method
         if moe_comm_method is None:
             raise RuntimeError("no MoE communication method is set up (call setup_moe_comm_method first)")
+        if (getattr(layer, "use_fused_small_batch", True) and shared_experts_input is None
+                and self._plain_call(layer, x) and topk_ids.dim() == 2 and topk_ids.shape[0] == x.shape[0]):
+            return self._apply_row_map(layer, x, topk_weights, topk_ids, shared_experts)
         shared_out = None
         if shared_experts is not None:
             # the shared expert sees the same hidden states unless the caller hands over others
@@ -102,6 +105,55 @@ class AscendW4A8DynamicFusedMoEMethod(AscendMoEScheme):
                 is_per_channel_weight=self.group_size == 0,
                 w4_group_size=self.group_size,
             ))
+
+    # ------------------------------------------------------------------ token rows quantised once, read through a map
+    def _plain_call(self, layer, x: torch.Tensor) -> bool:
+        """16-bit hidden states as a [T, H] matrix, none of the optional inputs of ``apply``, SiLU."""
+        if self.use_expert_weight_list or not x.is_cuda or x.dim() != 2 or x.shape[0] == 0:
+            return False
+        if x.dtype not in (torch.bfloat16, torch.float16):
+            return False
+        if (getattr(layer, "apply_router_weight_on_input", False) or getattr(layer, "ascend_pertoken_scale", None)
+                is not None or getattr(layer, "ascend_expert_map", None) is not None
+                or getattr(layer, "ascend_mc2_mask", None) is not None
+                or getattr(layer, "global_redundant_expert_num", 0)):
+            return False
+        act = getattr(layer, "activation", "silu")
+        return (getattr(act, "value", act) or "silu") == "silu"
+
+    def _apply_row_map(self, layer, x, topk_weights, topk_ids, shared_experts=None):
+        """``apply`` without the permuted copy of the activations, as the W8A8 scheme does it: every token row is
+        quantised once, routing builds the index maps only, the gate_up GEMM reads its rows through the
+        row -> token map.  Same results, bit for bit, as the op-by-op path
+        (``vllm_ascend/ops/fused_moe/moe_comm_method.py:117-162``, ``moe_mlp.py:425-451, 552-569``)."""
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        stream = torch.cuda.current_stream()
+        before_dispatch_evt = stream.record_event()
+        xq, x_scale = kernels.dynamic_quant(x)
+        shared_out = None
+        if shared_experts is not None:
+            shared_out = shared_experts(x, quantized=(xq, x_scale))
+        w1, w2 = layer.w13_weight, layer.w2_weight
+        s1, s2 = layer.w13_weight_scale, layer.w2_weight_scale
+        expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, w1.shape[0], 1)
+        k1, n1 = x.shape[1], s1.shape[-1]
+        g1 = k1 // s1.shape[1]
+        k2, n2 = n1 // 2, s2.shape[-1]
+        g2 = k2 // s2.shape[1]
+        cfg = getattr(layer, "moe_config", None)
+        swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
+        q1, q1_scale = kernels.gmm1_swiglu_quant_w4_gather(xq, x_scale, row_token, w1, s1, g1, expert_tokens, 1, n1, k1,
+                                                           swiglu_limit=swiglu_limit)
+        before_gmm2_evt = stream.record_event()
+        out = kernels.gmm2_dequant_w4(q1, w2, s2, g2, q1_scale, expert_tokens, 1, n2, k2, out_dtype=x.dtype)
+        before_combine_evt = stream.record_event()
+        if shared_experts is not None and shared_out is not None:
+            shared_experts.wait()
+        routed_out = kernels.token_unpermute(out, expanded_row_idx, topk_weights, shared_out)
+        return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
+                                  before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
+                                  group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
 
     @staticmethod
     def get_eplb_weight_views(layer) -> list:
