@@ -651,7 +651,7 @@ ORC_API int orc_dequant_swiglu_quant(const int32_t *x, const float *w_scale, con
 
 /*
  * W4A8 down projection tail:  o[r,n] = bf16( (f[r,n] + bias[e,n]) * s1[r] ), f from orc_gmm_w4_grouped.
- * (the token scale is applied last: SURVEY of the A8W4 kernel,
+ * (the token scale is applied last, as in the reference's A8W4 kernel,
  * csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant_a8w4_msd_post.h).
  */
 ORC_API int orc_w4_rows_to_bf16(const float *f, const float *s1, int64_t rows, int64_t N, uint16_t *o)
