@@ -191,6 +191,20 @@ int moe355_route_quant_small(const void *x, int x_dtype, const void *logits, int
                              int32_t *topk_ids, int8_t *xq, float *x_scale, int32_t *expanded_row_idx,
                              int32_t *row_token, int64_t *expert_tokens, int32_t *sync_counter, void *stream);
 
+/* Gating and token quantisation in one launch, for any number of tokens (at most 256 experts:
+ * moe355_gate_quant_supported() != 0): the two steps read different inputs, so their workgroups run side by side.
+ * Stands in for the pair torch.ops._C_ascend.moe_gating_top_k
+ * (vllm_ascend/ops/fused_moe/router/fused_topk_router.py:84-159) + the per-token quantisation inside
+ * torch_npu.npu_moe_init_routing_v2(quant_mode=1) (vllm_ascend/ops/fused_moe/token_dispatcher.py:424-435), with
+ * the arithmetic of moe355_gating_top_k and moe355_dynamic_quant; moe355_route_map then builds the index maps.
+ * Outputs as in moe355_route_quant_small: topk_weights [T, k] in x's dtype, topk_ids [T, k], xq [T, H] int8,
+ * x_scale [T]. */
+int moe355_gate_quant_supported(int64_t num_tokens, int top_k, int num_experts);
+int moe355_gate_quant(const void *x, int x_dtype, const void *logits, int logits_dtype, const void *bias,
+                      int64_t num_tokens, int64_t hidden, int num_experts, int k, int k_group, int group_count,
+                      int group_select_mode, int renorm, int norm_type, float routed_scaling_factor, float eps,
+                      void *topk_weights, int32_t *topk_ids, int8_t *xq, float *x_scale, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Weight format cast: dense int8 weights -> the MFMA-tiled storage the grouped
  * GEMMs stream ("NZ" of this build).  Stands in for

@@ -203,6 +203,31 @@ def test_route_quant_small_equals_gating_plus_init_routing(K, orc, case):
     assert not K.route_quant_small_supported(129, 8, 128) and not K.route_quant_small_supported(8, 8, 257)
 
 
+@pytest.mark.parametrize("case", SMALL_ROUTE_CASES + [(3000, 8, 128, 512, 0, 1, False, 1, 1, 1.0, torch.float32,
+                                                       torch.bfloat16),
+                                                      (1500, 6, 256, 7168, 1, 1, True, 8, 4, 2.5, torch.bfloat16,
+                                                       torch.bfloat16),
+                                                      (700, 2, 40, 200, 1, 0, True, 4, 2, 1.0, torch.float16,
+                                                       torch.float16)])
+def test_gate_quant_equals_gating_plus_dynamic_quant(K, orc, case):
+    """Gating and token quantisation in one launch (any number of tokens) against the two separate kernels."""
+    T, k, E, H, norm_type, renorm, use_bias, G, k_group, rsf, ldt, xdt = case
+    print(f"gate_quant {case}", flush=True)
+    assert K.gate_quant_supported(T, k, E)
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g).to(xdt).to(DEV)
+    logits = (torch.rand(T, E, generator=g) * 4 - 2).to(ldt).to(DEV)
+    bias = (torch.rand(E, generator=g) * 0.4 - 0.2).to(ldt).to(DEV) if use_bias else None
+    tw, ids, xq, xs = K.gate_quant(x, logits, k, k_group, G, 1, renorm, norm_type, rsf, 1e-20, bias)
+    y, ids_want, _, y_alt = K.gating_top_k(logits, k, k_group, G, 1, renorm, norm_type, False, rsf, 1e-20, bias,
+                                           alt_dtype=xdt)
+    xq_want, xs_want = K.dynamic_quant(x)
+    torch.cuda.synchronize()
+    assert torch.equal(ids, ids_want)
+    assert torch.equal(tw.view(torch.int16), y_alt.view(torch.int16))
+    assert torch.equal(xq, xq_want) and torch.equal(xs.view(torch.int32), xs_want.view(torch.int32))
+
+
 @pytest.mark.parametrize("R,E,Kd,N,T", [(512, 128, 2048, 1536, 64), (40, 4, 64, 128, 40), (300, 16, 768, 256, 75),
                                         (512, 256, 1024, 4096, 64), (100, 8, 64, 4160, 25),
                                         # many rows per expert: the LDS-tiled kernel (128- and 64-row tiles) and the

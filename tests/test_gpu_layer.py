@@ -24,7 +24,7 @@ def test_layer_bit_exact(name, fused):
     layer = build_layer(cfg, d, DEV)
     layer.use_fused_small_batch = fused
     takes_fused = layer.quant_method.supports_small_batch(layer, d["x"].to(DEV), d["logits"].to(DEV), layer.router)
-    assert takes_fused == (cfg.T * cfg.k <= 1024)
+    assert takes_fused  # every plain W8A8 call has a router-fused form (one launch up to 1024 pairs)
     x, logits = d["x"].to(DEV), d["logits"].to(DEV)
     res = layer.forward_impl(x, logits)
     torch.cuda.synchronize()

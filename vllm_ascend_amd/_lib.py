@@ -39,6 +39,10 @@ PROTOTYPES = {
     "moe355_init_routing_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int, c_int, c_int,
                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe355_route_quant_small_supported": (c_int, [c_int64, c_int, c_int]),
+    "moe355_gate_quant_supported": (c_int, [c_int64, c_int, c_int]),
+    "moe355_gate_quant": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int, c_int, c_int,
+                                  c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p]),
     "moe355_route_quant_small": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int, c_int,
                                          c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(kSmallThreads) void route_quant_small_kernel(SmallR
         gate_rows<LDT, PER, 1>(a.logits, a.bias, row, live, E, k, a.k_group, a.G, a.mode, a.renorm, a.norm_type, a.rsf,
                                a.eps, a.topk_weights, a.x_dtype, a.topk_ids, lds + (size_t)wave * E, nullptr, lane);
     }
+    if (!a.arrived) return;  // gating and quantisation only (moe355_gate_quant): the maps come from another launch
     // this workgroup's ids have reached memory before it is counted
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -181,19 +182,25 @@ __global__ __launch_bounds__(kSmallThreads) void route_quant_small_kernel(SmallR
 
 using namespace moe355;
 
+extern "C" int moe355_gate_quant_supported(int64_t num_tokens, int top_k, int num_experts)
+{
+    return num_tokens > 0 && num_tokens < (1 << 30) && top_k > 0 && top_k <= 64 && num_experts > 0 &&
+           num_experts <= kSmallMaxExperts && top_k <= num_experts;
+}
+
 extern "C" int moe355_route_quant_small_supported(int64_t num_tokens, int top_k, int num_experts)
 {
     return num_tokens > 0 && top_k > 0 && top_k <= 64 && num_tokens * top_k <= kSmallMaxPairs && num_experts > 0 &&
            num_experts <= kSmallMaxExperts && top_k <= num_experts;
 }
 
-extern "C" int moe355_route_quant_small(const void* x, int x_dtype, const void* logits, int logits_dtype,
-                                        const void* bias, int64_t num_tokens, int64_t hidden, int num_experts, int k,
-                                        int k_group, int group_count, int group_select_mode, int renorm,
-                                        int norm_type, float routed_scaling_factor, float eps, int tokens_num_type,
-                                        void* topk_weights, int32_t* topk_ids, int8_t* xq, float* x_scale,
-                                        int32_t* expanded_row_idx, int32_t* row_token, int64_t* expert_tokens,
-                                        int32_t* sync_counter, void* stream)
+// sort: the whole of moe355_route_quant_small; otherwise gating and quantisation only (any number of tokens)
+static int gate_quant_impl(bool sort, const void* x, int x_dtype, const void* logits, int logits_dtype,
+                           const void* bias, int64_t num_tokens, int64_t hidden, int num_experts, int k, int k_group,
+                           int group_count, int group_select_mode, int renorm, int norm_type,
+                           float routed_scaling_factor, float eps, int tokens_num_type, void* topk_weights,
+                           int32_t* topk_ids, int8_t* xq, float* x_scale, int32_t* expanded_row_idx,
+                           int32_t* row_token, int64_t* expert_tokens, int32_t* sync_counter, void* stream)
 {
     if (num_tokens < 0 || hidden <= 0 || num_experts <= 0 || k <= 0) return MOE355_E_ARG;
     if (norm_type != 0 && norm_type != 1) return MOE355_E_ARG;
@@ -203,12 +210,12 @@ extern "C" int moe355_route_quant_small(const void* x, int x_dtype, const void* 
     if (x_dtype != MOE355_DT_BF16 && x_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
     if (logits_dtype < MOE355_DT_F32 || logits_dtype > MOE355_DT_F16) return MOE355_E_ARG;
     if (num_tokens == 0) return MOE355_OK;
-    if (!moe355_route_quant_small_supported(num_tokens, k, num_experts)) return MOE355_E_SHAPE;
+    if (sort && !moe355_route_quant_small_supported(num_tokens, k, num_experts)) return MOE355_E_SHAPE;
+    if (!sort && !moe355_gate_quant_supported(num_tokens, k, num_experts)) return MOE355_E_SHAPE;
     if (group_count > 64 || num_experts % group_count != 0) return MOE355_E_SHAPE;
     if (hidden % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)xq & 7)) return MOE355_E_SHAPE;
-    if (!x || !logits || !topk_weights || !topk_ids || !xq || !x_scale || !expanded_row_idx || !row_token ||
-        !expert_tokens || !sync_counter)
-        return MOE355_E_ARG;
+    if (!x || !logits || !topk_weights || !topk_ids || !xq || !x_scale) return MOE355_E_ARG;
+    if (sort && (!expanded_row_idx || !row_token || !expert_tokens || !sync_counter)) return MOE355_E_ARG;
     SmallRouteArgs a = {};
     a.x = x;
     a.logits = logits;
@@ -233,12 +240,13 @@ extern "C" int moe355_route_quant_small(const void* x, int x_dtype, const void* 
     a.dst = expanded_row_idx;
     a.row_token = row_token;
     a.expert_tokens = expert_tokens;
-    a.arrived = sync_counter;
+    a.arrived = sort ? sync_counter : nullptr;
     const int E = num_experts;
     int per = 1;
     while (64 * per < E) per *= 2;
     // LDS: the sorting tables; the gating rows need E floats per wavefront and the quantiser 4 floats (less)
-    const size_t lds_bytes = ((size_t)kSmallMaxPairs + (size_t)kSmallChunks * E + E + 16) * 4;
+    const size_t lds_bytes = sort ? ((size_t)kSmallMaxPairs + (size_t)kSmallChunks * E + E + 16) * 4
+                                  : ((size_t)kSmallWaves * E + 16) * 4;
     const dim3 grid((unsigned)((num_tokens + kSmallWaves - 1) / kSmallWaves + num_tokens));
     hipStream_t st = (hipStream_t)stream;
 #define MOE355_SMALL(L_, P_, X_)                                                                                  \
@@ -259,4 +267,29 @@ extern "C" int moe355_route_quant_small(const void* x, int x_dtype, const void* 
 #undef MOE355_SMALL_PER
 #undef MOE355_SMALL
     return launch_status();
+}
+
+extern "C" int moe355_route_quant_small(const void* x, int x_dtype, const void* logits, int logits_dtype,
+                                        const void* bias, int64_t num_tokens, int64_t hidden, int num_experts, int k,
+                                        int k_group, int group_count, int group_select_mode, int renorm,
+                                        int norm_type, float routed_scaling_factor, float eps, int tokens_num_type,
+                                        void* topk_weights, int32_t* topk_ids, int8_t* xq, float* x_scale,
+                                        int32_t* expanded_row_idx, int32_t* row_token, int64_t* expert_tokens,
+                                        int32_t* sync_counter, void* stream)
+{
+    return gate_quant_impl(true, x, x_dtype, logits, logits_dtype, bias, num_tokens, hidden, num_experts, k, k_group,
+                           group_count, group_select_mode, renorm, norm_type, routed_scaling_factor, eps,
+                           tokens_num_type, topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token,
+                           expert_tokens, sync_counter, stream);
+}
+
+extern "C" int moe355_gate_quant(const void* x, int x_dtype, const void* logits, int logits_dtype, const void* bias,
+                                 int64_t num_tokens, int64_t hidden, int num_experts, int k, int k_group,
+                                 int group_count, int group_select_mode, int renorm, int norm_type,
+                                 float routed_scaling_factor, float eps, void* topk_weights, int32_t* topk_ids,
+                                 int8_t* xq, float* x_scale, void* stream)
+{
+    return gate_quant_impl(false, x, x_dtype, logits, logits_dtype, bias, num_tokens, hidden, num_experts, k, k_group,
+                           group_count, group_select_mode, renorm, norm_type, routed_scaling_factor, eps, 1,
+                           topk_weights, topk_ids, xq, x_scale, nullptr, nullptr, nullptr, nullptr, stream);
 }

@@ -224,6 +224,37 @@ def route_quant_small(x, logits, k, k_group, group_count, group_select_mode, ren
     return tw, ids, xq, xs, dst, row_token, tokens
 
 
+def gate_quant_supported(num_tokens: int, top_k: int, num_experts: int) -> bool:
+    return bool(_lib.load().moe355_gate_quant_supported(num_tokens, top_k, num_experts))
+
+
+def gate_quant(x, logits, k, k_group, group_count, group_select_mode, renorm, norm_type, routed_scaling_factor, eps,
+               bias):
+    """Gating and token quantisation in one launch, any number of tokens.  -> (topk_weights [T, k] in x's dtype,
+    topk_ids [T, k] int32, xq int8 [T, H] in token order, x_scale [T])."""
+    x = _dev(x, "x")
+    logits = _dev(logits, "router_logits")
+    if bias is not None:
+        bias = _dev(bias, "bias")
+        if bias.dtype != logits.dtype:
+            raise RuntimeError("The dtype of x and bias should be same")
+    lib = _lib.load()
+    T, E = logits.shape
+    H = x.shape[-1]
+    if x.numel() != T * H:
+        raise ValueError(f"hidden states {tuple(x.shape)} do not match {T} rows of router logits")
+    dev = x.device
+    tw = torch.empty((T, k), dtype=x.dtype, device=dev)
+    ids = torch.empty((T, k), dtype=torch.int32, device=dev)
+    xq = torch.empty((T, H), dtype=torch.int8, device=dev)
+    xs = torch.empty((T,), dtype=torch.float32, device=dev)
+    check(lib.moe355_gate_quant(_ptr(x), _dt(x, "x"), _ptr(logits), _dt(logits, "router_logits"), _ptr(bias), T, H, E,
+                                k, k_group, group_count, group_select_mode, int(renorm), norm_type,
+                                float(routed_scaling_factor), float(eps), _ptr(tw), _ptr(ids), _ptr(xq), _ptr(xs),
+                                _stream(x)), "moe355_gate_quant")
+    return tw, ids, xq, xs
+
+
 def gmm1_swiglu_quant_gather(xq, x_scale, row_token, weight_nz, weight_scale, group_list, group_list_type, n, k,
                              swiglu_limit=0.0):
     """gate_up GEMM + SwiGLU + re-quantisation on rows that are read through ``row_token`` from activations kept

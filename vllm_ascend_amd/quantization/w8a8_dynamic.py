@@ -175,8 +175,10 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
 
     # ------------------------------------------------------------------ small batches (decode)
     def supports_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
-        """Whether ``apply_small_batch`` can take this call: a plain call (see ``_plain_call``), no forced load
-        balance, and a batch of at most 1024 (token, slot) pairs over at most 256 experts."""
+        """Whether ``apply_small_batch`` can take this call, router included: a plain call (see ``_plain_call``),
+        no forced load balance, at most 256 experts.  (The name is from the time when only batches of at most 1024
+        (token, slot) pairs had such a form; those still get gating, dispatch and quantisation in ONE launch,
+        larger ones gating and quantisation.)"""
         from .. import kernels
 
         if not self._plain_call(layer, x) or router_logits.dim() != 2:
@@ -185,7 +187,8 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
             return False
         if getattr(layer, "enable_force_load_balance", False):
             return False
-        return kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
+        return (kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
+                or kernels.gate_quant_supported(x.shape[0], router.top_k, router_logits.shape[1]))
 
     def apply_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router,
                           shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
@@ -202,16 +205,22 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
             bias = router.e_score_correction_bias = bias.to(router_logits.dtype)
         stream = torch.cuda.current_stream()
         before_dispatch_evt = stream.record_event()
-        # the routing kernel's arrival counter: one zeroed int32 per layer (and device), which every call leaves at
-        # zero; created on the first call (run the layer once before capturing it into a graph)
-        counter = getattr(layer, "_small_batch_counter", None)
-        if counter is None or counter.device != x.device:
-            counter = layer._small_batch_counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
-        topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = kernels.route_quant_small(
-            x, router_logits, router.top_k, router.topk_group if router.topk_group is not None else 1,
-            router.num_expert_group if router.num_expert_group is not None else 1, 1, int(router.renormalize),
-            0 if router.scoring_func == "softmax" else 1, router.routed_scaling_factor, 1e-20, bias,
-            sync_counter=counter)
+        gate_args = (router.top_k, router.topk_group if router.topk_group is not None else 1,
+                     router.num_expert_group if router.num_expert_group is not None else 1, 1,
+                     int(router.renormalize), 0 if router.scoring_func == "softmax" else 1,
+                     router.routed_scaling_factor, 1e-20, bias)
+        if kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1]):
+            # the routing kernel's arrival counter: one zeroed int32 per layer (and device), which every call leaves
+            # at zero; created on the first call (run the layer once before capturing it into a graph)
+            counter = getattr(layer, "_small_batch_counter", None)
+            if counter is None or counter.device != x.device:
+                counter = layer._small_batch_counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
+            topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = \
+                kernels.route_quant_small(x, router_logits, *gate_args, sync_counter=counter)
+        else:
+            # larger batches: gating and quantisation side by side in one launch, then the index maps
+            topk_weights, topk_ids, xq, x_scale = kernels.gate_quant(x, router_logits, *gate_args)
+            expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, router_logits.shape[1], 1)
         shared_out = None
         if shared_experts is not None:
             if shared_experts_input is None:
