@@ -7,7 +7,8 @@ import torch
 from _inputs import LayerCfg, bits, gating_kwargs
 
 
-def build_layer(cfg: LayerCfg, d: dict, device="cuda:0", shared=False, overlap=False, dynamic_eplb=False):
+def build_layer(cfg: LayerCfg, d: dict, device="cuda:0", shared=False, overlap=False, dynamic_eplb=False,
+                collect_expert_load=False, heat_interval=None):
     from vllm_ascend_amd.fused_moe.contracts import FusedMoEConfig
     from vllm_ascend_amd.fused_moe.layer import AscendRoutedExperts
     from vllm_ascend_amd.fused_moe.router import AscendFusedTopKRouter
@@ -35,7 +36,8 @@ def build_layer(cfg: LayerCfg, d: dict, device="cuda:0", shared=False, overlap=F
         return layer
     scheme = get_scheme_class("W8A8_DYNAMIC", "moe")(dynamic_eplb=dynamic_eplb)
     layer = AscendRoutedExperts(moe_config, scheme, router, params_dtype=torch.float32, device=device,
-                                shared_experts=shared_experts)
+                                shared_experts=shared_experts, dynamic_eplb=collect_expert_load,
+                                expert_heat_collection_interval=heat_interval)
     layer.load_weights({
         "w13_weight": d["w13"].to(device), "w2_weight": d["w2"].to(device),
         "w13_weight_scale": d["s13"].to(device), "w2_weight_scale": d["s2"].to(device),

@@ -330,3 +330,34 @@ def test_force_load_balance_replaces_the_ids_only():
     assert len(set(ids2.reshape(-1).tolist())) > 8                    # spread over the experts
     w3, ids3 = r.select_experts(torch.zeros(10, 8, dtype=torch.bfloat16), torch.zeros(10, 32))
     assert ids3 is ids
+
+
+def test_expert_load_from_both_group_list_forms():
+    """Counts (type 1) and running totals (type 0) must add the same loads (routed_experts.py:571-587)."""
+    import types
+
+    import torch
+
+    from vllm_ascend_amd.fused_moe.contracts import FusedExpertsResult
+    from vllm_ascend_amd.fused_moe.layer import AscendRoutedExperts
+
+    counts = torch.tensor([3, 0, 5, 1], dtype=torch.int64)
+    for multi_stage in (False, True):
+        holder = types.SimpleNamespace(
+            multi_stage=multi_stage, num_iter=3, load_counter=torch.zeros((), dtype=torch.int32),
+            moe_load=torch.zeros((3, 4), dtype=torch.int32) if multi_stage else torch.zeros(4, dtype=torch.int64))
+        for glt, tokens in ((1, counts), (0, counts.cumsum(0)), (1, counts), (0, counts.cumsum(0))):
+            res = FusedExpertsResult(routed_out=torch.zeros(1), group_list_type=glt, expert_tokens=tokens)
+            AscendRoutedExperts._record_expert_load(holder, res)
+        if multi_stage:
+            assert holder.moe_load.tolist() == [(2 * counts).tolist(), counts.tolist(), counts.tolist()]
+            assert int(holder.load_counter) == 4
+        else:
+            assert holder.moe_load.tolist() == (4 * counts).tolist()
+    res = FusedExpertsResult(routed_out=torch.zeros(1))
+    try:
+        AscendRoutedExperts._record_expert_load(holder, res)
+    except AssertionError as e:
+        assert "should not be None when dynamic_eplb is enabled" in str(e)
+    else:
+        raise AssertionError("a result without expert_tokens must be refused")

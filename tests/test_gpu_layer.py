@@ -238,6 +238,37 @@ def test_layer_with_per_expert_weight_lists():
     assert not torch.equal(res.routed_out, res2.routed_out)
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_expert_load_collection(fused):
+    """The layer sums the tokens every expert received over its forward passes (what the load balancer
+    reads): one row, or one row per pass of a collection interval; collection can be paused and cleared."""
+    print(f"expert load collection fused={fused}", flush=True)
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=2)
+    plain = build_layer(cfg, d, DEV)
+    want = np.bincount(oracle_layer(cfg, d).topk_ids.reshape(-1), minlength=cfg.E)
+    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+    for interval in (None, 2):
+        # with the interval: also the per-expert weight lists that dynamic load balancing swaps in place
+        layer = build_layer(cfg, d, DEV, dynamic_eplb=interval is not None, collect_expert_load=True,
+                            heat_interval=interval)
+        layer.use_fused_small_batch = fused
+        for _ in range(3):
+            out = layer.forward_impl(x, logits).routed_out
+        layer.eplb_heat_collection_status = False
+        layer.forward_impl(x, logits)
+        torch.cuda.synchronize()
+        assert torch.equal(out, plain.forward_impl(x, logits).routed_out)
+        got = layer.moe_load.cpu().numpy()
+        if interval is None:
+            assert got.dtype == np.int64 and np.array_equal(got, 3 * want)
+        else:
+            assert got.dtype == np.int32 and np.array_equal(got, np.stack([2 * want, want]))
+            assert int(layer.load_counter) == 3
+        layer.clear_moe_load()
+        assert int(layer.moe_load.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("name", ["c2_small", "c4_small", "c5_small"])
 def test_empty_and_single_token_batches(name):
     """T = 0 (a rank with nothing to do in a padded step) returns an empty result without launching anything

@@ -16,7 +16,8 @@ from .router import AscendFusedTopKRouter
 
 class AscendRoutedExperts(torch.nn.Module):
     def __init__(self, moe_config: FusedMoEConfig, quant_method: AscendMoEScheme, router: AscendFusedTopKRouter,
-                 params_dtype: torch.dtype = torch.bfloat16, device="cuda", shared_experts=None, gate=None):
+                 params_dtype: torch.dtype = torch.bfloat16, device="cuda", shared_experts=None, gate=None,
+                 dynamic_eplb: bool = False, expert_heat_collection_interval: int | None = None):
         super().__init__()
         self.shared_experts = shared_experts
         # the router's own gate (an AscendGateLinear) when the layer computes its logits itself
@@ -42,6 +43,26 @@ class AscendRoutedExperts(torch.nn.Module):
         for name, t in specs.items():
             self.register_parameter(name, torch.nn.Parameter(t.to(device), requires_grad=False))
         self.moe_comm_method = setup_moe_comm_method(moe_config)
+        # tokens per local expert, summed over forward passes, for the load balancer
+        # (routed_experts.py:343-373): one int64 row, or, with a collection interval, one int32 row per
+        # pass of the interval, indexed by a device-side pass counter
+        self.dynamic_eplb = dynamic_eplb
+        self.eplb_heat_collection_status = True
+        self.multi_stage = bool(dynamic_eplb and expert_heat_collection_interval)
+        self.num_iter = int(expert_heat_collection_interval) if self.multi_stage else None
+        if not self.multi_stage:
+            self.load_counter = None
+        if not dynamic_eplb:
+            self.moe_load = None
+        else:
+            if self.multi_stage:
+                self.register_buffer("load_counter", torch.zeros((), dtype=torch.int32, device=device),
+                                     persistent=False)
+                self.register_buffer("moe_load", torch.zeros((self.num_iter, moe_config.num_experts),
+                                                             dtype=torch.int32, device=device), persistent=False)
+            else:
+                self.register_buffer("moe_load", torch.zeros(moe_config.num_experts, dtype=torch.int64,
+                                                             device=device), persistent=False)
         # per-expert checkpoint tensors -> slices of the stacked parameters (quantization/checkpoint.py)
         self.weight_loader = moe_weight_loader
 
@@ -53,14 +74,42 @@ class AscendRoutedExperts(torch.nn.Module):
             p.data.copy_(t.reshape(p.data.shape).to(p.data.dtype))
         self.quant_method.process_weights_after_loading(self)
 
+    def clear_moe_load(self) -> None:
+        """Zero the collected expert loads (routed_experts.py:423-428)."""
+        assert self.moe_load is not None
+        self.moe_load.zero_()
+        if self.multi_stage:
+            self.load_counter.zero_()
+
+    def _record_expert_load(self, result: FusedExpertsResult) -> None:
+        """Add this pass's tokens per expert to ``moe_load`` (routed_experts.py:567-587)."""
+        expert_tokens, group_list_type = result.expert_tokens, result.group_list_type
+        assert expert_tokens is not None and group_list_type is not None, (
+            "expert_tokens and group_list_type should not be None when dynamic_eplb is enabled.")
+        if group_list_type == 1:
+            local_load = expert_tokens
+        else:  # running totals -> counts
+            local_load = torch.cat([expert_tokens[:1], expert_tokens[1:] - expert_tokens[:-1]])
+        if self.multi_stage:
+            cur_iter = torch.remainder(self.load_counter, self.num_iter)
+            self.moe_load.index_add_(0, cur_iter.view(1), local_load.to(torch.int32).view(1, -1))
+            self.load_counter.add_(1)
+        else:
+            self.moe_load.add_(local_load)
+
     def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
+        result = self._run_experts(hidden_states, router_logits)
+        if self.dynamic_eplb and self.eplb_heat_collection_status:
+            self._record_expert_load(result)
+        result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
+        return result
+
+    def _run_experts(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> FusedExpertsResult:
         hidden_states, router_logits, _, _ = self.moe_comm_method.prepare(hidden_states, router_logits)
         fused = getattr(self.quant_method, "supports_small_batch", None)
         if self.use_fused_small_batch and fused is not None and fused(self, hidden_states, router_logits, self.router):
-            result = self.quant_method.apply_small_batch(self, hidden_states, router_logits, self.router,
-                                                         self.shared_experts, None)
-            result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
-            return result
+            return self.quant_method.apply_small_batch(self, hidden_states, router_logits, self.router,
+                                                       self.shared_experts, None)
         # int8 hidden states = activations the caller quantised (their scales in ascend_pertoken_scale): the
         # routing weights then take the model dtype of the scheme
         weights_dtype = None
@@ -69,9 +118,7 @@ class AscendRoutedExperts(torch.nn.Module):
         topk_weights, topk_ids = self.router.select_experts(
             hidden_states, router_logits, enable_force_load_balance=self.enable_force_load_balance,
             weights_dtype=weights_dtype)
-        result = self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
-        result.routed_out = self.moe_comm_method.finalize(result.routed_out, reduce_results=False)
-        return result
+        return self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
 
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None) -> torch.Tensor:
         if router_logits is None:

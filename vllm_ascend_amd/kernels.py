@@ -373,14 +373,15 @@ def gmm2_dequant(x, weight_nz, scale, per_token_scale, group_list, group_list_ty
     return out
 
 
-def gmm_i32(x, weight_nz, group_list, group_list_type, n, k):
-    """Raw int32 accumulators of the grouped product (rows outside every group are zero)."""
+def gmm_i32(x, weight_nz, group_list, group_list_type, n, k, groups_cover_all_rows=False):
+    """Raw int32 accumulators of the grouped product (rows outside every group are zero; a caller whose
+    groups cover every row says so and saves the fill)."""
     lib = _lib.load()
     rows = x.shape[0]
     E = weight_nz.shape[0]
     _check_gmm_operands("gmm_i32", x, rows, k, n, E, group_list, weight=weight_nz, weight_numel=E * n * k)
     x = _dev(x, "x")
-    acc = torch.zeros((rows, n), dtype=torch.int32, device=x.device)
+    acc = (torch.empty if groups_cover_all_rows else torch.zeros)((rows, n), dtype=torch.int32, device=x.device)
     ws = _workspace(lib.moe355_gmm_i32_workspace(rows, n, k, E), x.device)
     check(lib.moe355_gmm_i32(_ptr(x), _ptr(_dev(weight_nz, "weight")), _ptr(_gl(group_list)),
                              _gl_type(group_list_type), rows, k, n, E, _ptr(acc), _ptr(ws), ws.numel(), _stream(x)),

@@ -150,7 +150,7 @@ def npu_quant_matmul(x1, x2, scale, *, offset=None, pertoken_scale=None, bias=No
     gl = _single_group_list(a.shape[0], a.device)
     w = x2.unsqueeze(0)
     if output_dtype == torch.int32:
-        out = kernels.gmm_i32(a, w, gl, 0, n, k)
+        out = kernels.gmm_i32(a, w, gl, 0, n, k, groups_cover_all_rows=True)
     elif output_dtype in (None, torch.bfloat16, torch.float16):
         if pertoken_scale is None:
             raise NotImplementedError("npu_quant_matmul: bf16 / fp16 output needs pertoken_scale")
