@@ -384,7 +384,8 @@ int moe355_profile_next_gemm(void *start_event, void *stop_event);
 
 /* Which kernel family the int8 grouped GEMMs above launch for a shape, given a workspace of the size their
  * moe355_*_workspace() asks for: "gmm_stream_kernel" (few rows per expert), "gmm_tiled_kernel" (128-row
- * LDS-tiled) or "gmm_wide_kernel" (weight-streaming tiles of up to 256 rows); "" for arguments no GEMM accepts.
+ * LDS-tiled), "gmm_wide_kernel" (weight-streaming tiles of up to 256 rows) or "gmm_dense_kernel" (one expert
+ * with thousands of rows: 256 x 256 tiles, no tile map); "" for arguments no GEMM accepts.
  * epilogue: 0 raw int32 (moe355_gmm_i32), 1 SwiGLU (moe355_gmm1_swiglu_quant), 2 dequant (moe355_gmm2_dequant).
  * A pure function of its arguments, for benchmarks and profiles (no counterpart in the reference). */
 const char *moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_t k, int64_t n, int num_experts);

@@ -233,7 +233,9 @@ def test_gate_quant_equals_gating_plus_dynamic_quant(K, orc, case):
                                         # many rows per expert: the LDS-tiled kernel (128- and 64-row tiles) and the
                                         # weight-streaming tiles (wide and tall) read through the map as well
                                         (4096, 8, 512, 256, 700), (1300, 16, 192, 128, 400), (1100, 8, 1024, 256, 300),
-                                        (700, 4, 4096, 128, 200), (1500, 6, 4096, 192, 1500)])
+                                        (700, 4, 4096, 128, 200), (1500, 6, 4096, 192, 1500),
+                                        # one expert: the dense kernel
+                                        (3100, 1, 128, 4096, 900)])
 def test_gmm1_swiglu_quant_gather(K, orc, R, E, Kd, N, T):
     """Rows read through the row -> token map give what the gathered copy gives."""
     from vllm_ascend_amd._lib import W_ENK
@@ -313,7 +315,10 @@ GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100
              (32000, 256, 1024, 128), (40000, 320, 1024, 64),
              # one expert with at most 64 rows and a long K (the shared expert of a decode batch): the int32 product
              # cuts K into slabs and adds the partial sums into the zeroed result
-             (64, 1, 7168, 256), (33, 1, 2048, 1024), (1, 1, 4096, 128)]
+             (64, 1, 7168, 256), (33, 1, 2048, 1024), (1, 1, 4096, 128),
+             # one expert with thousands of rows (the shared expert of a prefill batch): the dense kernel's 256 x 256
+             # tiles, with a ragged last row tile and a last column block of 64 channels
+             (3000, 1, 128, 4096), (2049, 1, 192, 6464)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
@@ -365,6 +370,24 @@ def test_gmm_i32_dense_few_rows_with_and_without_scratch(K, orc, R, Kd, N, rows)
     assert np.array_equal(acc.cpu().numpy(), ref)
     got2 = acc2.cpu().numpy()
     assert np.array_equal(got2[:rows], ref[:rows])
+
+
+def test_gmm_i32_dense_group_shorter_than_the_buffer(K, orc):
+    """The dense kernel takes the row count from the group list on the device, not from the buffer's size: rows
+    behind the group's last one stay as the caller's fill left them."""
+    from vllm_ascend_amd._lib import W_ENK
+
+    R, Kd, N, rows = 3200, 64, 4096, 2450
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (1, N, Kd), generator=g, dtype=torch.int8)
+    cnt = torch.tensor([rows], dtype=torch.int64)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cnt.numpy())
+    ref[rows:] = 0
+    for glt in (0, 1):
+        acc = K.gmm_i32(x.to(DEV), wnz, cnt.to(DEV), glt, N, Kd)
+        assert np.array_equal(acc.cpu().numpy(), ref)
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)

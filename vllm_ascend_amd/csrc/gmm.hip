@@ -375,6 +375,19 @@ static int tiled_bm(const GmmArgs& a)
     return 128;
 }
 
+// One expert with enough rows and channels for the 256 x 256 tiles to fill the chip: the dense kernel (measured
+// against the 128-row tiles: 13 to 17 % faster from 192 tiles on, 20 to 25 % slower at 64 to 128 tiles).
+static bool dense_tiles(const GmmArgs& a)
+{
+    if (a.E != 1 || a.K % 64 != 0) return false;
+#ifdef MOE355_DEV_KNOBS
+    static const char* force = getenv("MOE355_GEMM");
+    if (force && force[0] == 'D') return true;
+    if (force && force[0]) return false;
+#endif
+    return ((a.R + 255) / 256) * ((int64_t)(a.N + 255) / 256) >= 192;
+}
+
 static size_t tiled_ws_max(int64_t rows, int E)
 {
     return tiled_workspace_bytes(rows, E, 64);  // the smallest tile needs the longest tile list
@@ -401,6 +414,12 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
     // dense, few rows (the shared expert of a decode batch): a 64-row tile map gives one workgroup per 256
     // channels, the streaming kernel one per 64 (and K slabs on top for the int32 form)
     if (a.E == 1 && a.R <= 64) bm = 0;
+    if (dense_tiles(a)) {
+        launch_dense(EPI, a, st, t_ev_start, t_ev_stop);
+        t_ev_start = nullptr;
+        t_ev_stop = nullptr;
+        return launch_status();
+    }
     if (bm) {
         launch_tiled_any(EPI, bm, a, tile_ws, st, t_ev_start, t_ev_stop);
         t_ev_start = nullptr;
@@ -461,6 +480,7 @@ extern "C" const char* moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_
     a.K = (int)k;
     a.N = (int)n;
     a.E = num_experts;
+    if (dense_tiles(a)) return "gmm_dense_kernel";
     const int bm = (a.E == 1 && a.R <= 64) ? 0 : tiled_bm(a);  // as launch_gemm_auto decides
     if (bm == 256) return "gmm_wide_kernel";
     if (bm != 0) return "gmm_tiled_kernel";

@@ -20,4 +20,7 @@ size_t tiled_workspace_bytes(int64_t rows, int E, int BM);
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
                       hipEvent_t ev1);
 
+// One expert owning every row (a.E == 1): 256 x 256 tiles placed by arithmetic, no tile map, no scratch.
+void launch_dense(int epi, const GmmArgs& a, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1);
+
 }  // namespace moe355

@@ -691,6 +691,28 @@ __global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm,
     }
 }
 
+// One expert that owns every row (a dense product: the shared expert of a prefill batch): 256 x 256 tiles of the
+// tall form, one workgroup per tile and compute unit, found by arithmetic on the expert's row count.  This shape
+// is bound by the matrix units and, before them, by what the XCDs fetch: a tile reads 256 token rows and 256
+// weight channels over the whole of K, and only tiles on the same XCD share those reads in its L2.  The 8 XCDs
+// (workgroup i runs on XCD i % 8) therefore split the tile grid into xm x xn rectangles of pm x pn tiles, as
+// square as the shape allows, instead of every XCD streaming all the weights.
+template <int EPI>
+__global__ __launch_bounds__(512, 1) void gmm_dense_kernel(GmmArgs a, int xn, int pm, int pn, int n_col_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) int8_t wide_lds[];
+    const int xcd = (int)(blockIdx.x % 8);
+    const int slot = (int)(blockIdx.x / 8);
+    const int mt = (xcd / xn) * pm + slot / pn;
+    const int nt = (xcd % xn) * pn + slot % pn;
+    if (nt >= n_col_blocks) return;
+    int64_t rows = a.gl[0];  // one group: its count and its running total are the same number
+    if (rows > a.R) rows = a.R;
+    const int64_t row0 = (int64_t)mt * 256;
+    if (row0 >= rows) return;
+    stream_tile_body<EPI, false>(a, 0, row0, rows, nt, wide_lds);
+}
+
 // ------------------------------------------------------------------ host side
 size_t tiled_workspace_bytes(int64_t rows, int E, int BM)
 {
@@ -750,6 +772,43 @@ static void launch_wide(const GmmArgs& a, void* workspace, hipStream_t st, hipEv
     else
         hipLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, a, tm, max_tiles,
                            n_col_blocks, columns);
+}
+
+template <int EPI>
+static void launch_dense_t(const GmmArgs& a, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
+{
+    constexpr int lds_bytes = kWideLdsBytes;
+    static const hipError_t attr = hipFuncSetAttribute((const void*)gmm_dense_kernel<EPI>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    (void)attr;
+    const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
+    const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
+    const int n_col_blocks = (channels + per_block - 1) / per_block;
+    const int row_tiles = (int)((a.R + 255) / 256);
+    // the split of the 8 XCDs over rows x columns with the smallest rectangle perimeter (= bytes fetched per XCD)
+    int xn = 1, best = 0;
+    for (int c = 1; c <= 8; c *= 2) {
+        const int per_m = (row_tiles + 8 / c - 1) / (8 / c), per_n = (n_col_blocks + c - 1) / c;
+        const int cost = per_m + per_n;
+        if (c == 1 || cost < best) {
+            best = cost;
+            xn = c;
+        }
+    }
+    const int pm = (row_tiles + 8 / xn - 1) / (8 / xn), pn = (n_col_blocks + xn - 1) / xn;
+    const int grid = 8 * pm * pn;
+    if (ev0 && ev1)
+        hipExtLaunchKernelGGL((gmm_dense_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, ev0, ev1, 0, a, xn, pm, pn,
+                              n_col_blocks);
+    else
+        hipLaunchKernelGGL((gmm_dense_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, a, xn, pm, pn, n_col_blocks);
+}
+
+void launch_dense(int epi, const GmmArgs& a, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1)
+{
+    if (epi == EPI_I32) launch_dense_t<EPI_I32>(a, st, ev0, ev1);
+    else if (epi == EPI_SWIGLU) launch_dense_t<EPI_SWIGLU>(a, st, ev0, ev1);
+    else launch_dense_t<EPI_DEQUANT>(a, st, ev0, ev1);
 }
 
 void launch_tiled_any(int epi, int bm, const GmmArgs& a, void* workspace, hipStream_t st, hipEvent_t ev0,
