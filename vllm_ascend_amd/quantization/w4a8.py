@@ -21,7 +21,7 @@ from .. import kernels
 from ..fused_moe.contracts import MoEMlpComputeInput, build_fused_experts_input
 from ..fused_moe.forward_context import _EXTRA_CTX
 from ..quant_type import QuantType
-from .base import AscendMoEScheme, register_scheme
+from .base import AscendMoEScheme, fused_front_supported, register_scheme, route_and_quantize
 
 
 @register_scheme("W4A8_DYNAMIC", "moe")
@@ -126,17 +126,42 @@ class AscendW4A8DynamicFusedMoEMethod(AscendMoEScheme):
         quantised once, routing builds the index maps only, the gate_up GEMM reads its rows through the
         row -> token map.  Same results, bit for bit, as the op-by-op path
         (``vllm_ascend/ops/fused_moe/moe_comm_method.py:117-162``, ``moe_mlp.py:425-451, 552-569``)."""
-        from ..fused_moe.contracts import FusedExpertsResult
-
-        stream = torch.cuda.current_stream()
-        before_dispatch_evt = stream.record_event()
+        before_dispatch_evt = torch.cuda.current_stream().record_event()
         xq, x_scale = kernels.dynamic_quant(x)
         shared_out = None
         if shared_experts is not None:
             shared_out = shared_experts(x, quantized=(xq, x_scale))
+        expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, layer.w13_weight.shape[0], 1)
+        return self._experts_on_row_map(layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens,
+                                        topk_weights, shared_experts, shared_out, before_dispatch_evt)
+
+    def supports_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
+        """Whether ``apply_small_batch`` can take this call, router included (the W8A8 scheme's rule)."""
+        return self._plain_call(layer, x) and fused_front_supported(layer, x, router_logits, router)
+
+    def apply_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router,
+                          shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
+        """router + ``apply`` with gating, token quantisation and (for small batches) the dispatch maps in one
+        launch; same results, bit for bit, as ``router.select_experts`` followed by ``apply``."""
+        before_dispatch_evt = torch.cuda.current_stream().record_event()
+        topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = \
+            route_and_quantize(layer, x, router_logits, router)
+        shared_out = None
+        if shared_experts is not None:
+            if shared_experts_input is None:
+                shared_out = shared_experts(x, quantized=(xq, x_scale))
+            else:
+                shared_out = shared_experts(shared_experts_input)
+        return self._experts_on_row_map(layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens,
+                                        topk_weights, shared_experts, shared_out, before_dispatch_evt)
+
+    def _experts_on_row_map(self, layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens, topk_weights,
+                            shared_experts, shared_out, before_dispatch_evt):
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        stream = torch.cuda.current_stream()
         w1, w2 = layer.w13_weight, layer.w2_weight
         s1, s2 = layer.w13_weight_scale, layer.w2_weight_scale
-        expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, w1.shape[0], 1)
         k1, n1 = x.shape[1], s1.shape[-1]
         g1 = k1 // s1.shape[1]
         k2, n2 = n1 // 2, s2.shape[-1]

@@ -13,7 +13,7 @@ from .. import npu_ops
 from ..fused_moe.contracts import build_fused_experts_input
 from ..fused_moe.forward_context import _EXTRA_CTX
 from ..quant_type import QuantType
-from .base import AscendMoEScheme, register_scheme
+from .base import AscendMoEScheme, fused_front_supported, register_scheme, route_and_quantize
 
 
 @register_scheme("W8A8_DYNAMIC", "moe")
@@ -179,16 +179,7 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         no forced load balance, at most 256 experts.  (The name is from the time when only batches of at most 1024
         (token, slot) pairs had such a form; those still get gating, dispatch and quantisation in ONE launch,
         larger ones gating and quantisation.)"""
-        from .. import kernels
-
-        if not self._plain_call(layer, x) or router_logits.dim() != 2:
-            return False
-        if router_logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
-            return False
-        if getattr(layer, "enable_force_load_balance", False):
-            return False
-        return (kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
-                or kernels.gate_quant_supported(x.shape[0], router.top_k, router_logits.shape[1]))
+        return self._plain_call(layer, x) and fused_front_supported(layer, x, router_logits, router)
 
     def apply_small_batch(self, layer, x: torch.Tensor, router_logits: torch.Tensor, router,
                           shared_experts: Any | None = None, shared_experts_input: torch.Tensor | None = None):
@@ -197,30 +188,9 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         row -> token map), then the gate_up GEMM with SwiGLU and re-quantisation, the down GEMM and the combine.
         Same results, bit for bit, as ``router.select_experts`` followed by ``apply``
         (``vllm_ascend/ops/fused_moe/routed_experts.py:496-609``, ``w8a8_dynamic.py:224-301``)."""
-        from .. import kernels
-        from ..fused_moe.contracts import FusedExpertsResult
-
-        bias = router.e_score_correction_bias
-        if bias is not None and bias.dtype != router_logits.dtype:
-            bias = router.e_score_correction_bias = bias.to(router_logits.dtype)
-        stream = torch.cuda.current_stream()
-        before_dispatch_evt = stream.record_event()
-        gate_args = (router.top_k, router.topk_group if router.topk_group is not None else 1,
-                     router.num_expert_group if router.num_expert_group is not None else 1, 1,
-                     int(router.renormalize), 0 if router.scoring_func == "softmax" else 1,
-                     router.routed_scaling_factor, 1e-20, bias)
-        if kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1]):
-            # the routing kernel's arrival counter: one zeroed int32 per layer (and device), which every call leaves
-            # at zero; created on the first call (run the layer once before capturing it into a graph)
-            counter = getattr(layer, "_small_batch_counter", None)
-            if counter is None or counter.device != x.device:
-                counter = layer._small_batch_counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
-            topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = \
-                kernels.route_quant_small(x, router_logits, *gate_args, sync_counter=counter)
-        else:
-            # larger batches: gating and quantisation side by side in one launch, then the index maps
-            topk_weights, topk_ids, xq, x_scale = kernels.gate_quant(x, router_logits, *gate_args)
-            expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, router_logits.shape[1], 1)
+        before_dispatch_evt = torch.cuda.current_stream().record_event()
+        topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = \
+            route_and_quantize(layer, x, router_logits, router)
         shared_out = None
         if shared_experts is not None:
             if shared_experts_input is None:
