@@ -8,13 +8,20 @@ from _inputs import LayerCfg, bits, gating_kwargs
 
 
 def build_layer(cfg: LayerCfg, d: dict, device="cuda:0", shared=False, overlap=False, dynamic_eplb=False,
-                collect_expert_load=False, heat_interval=None):
+                collect_expert_load=False, heat_interval=None, redundant=()):
+    """redundant: logical expert ids whose weights are appended as extra physical experts (the router still
+    scores cfg.E logical experts)."""
     from vllm_ascend_amd.fused_moe.contracts import FusedMoEConfig
     from vllm_ascend_amd.fused_moe.layer import AscendRoutedExperts
     from vllm_ascend_amd.fused_moe.router import AscendFusedTopKRouter
     from vllm_ascend_amd.quantization import get_scheme_class
 
-    moe_config = FusedMoEConfig(num_experts=cfg.E, experts_per_token=cfg.k, hidden_dim=cfg.H,
+    if redundant:
+        d = dict(d)
+        idx = torch.tensor(list(range(cfg.E)) + list(redundant))
+        for name in ("w13", "w2", "s13", "s2"):
+            d[name] = d[name][idx].contiguous()
+    moe_config = FusedMoEConfig(num_experts=cfg.E + len(redundant), experts_per_token=cfg.k, hidden_dim=cfg.H,
                                 intermediate_size_per_partition=cfg.I)
     router = AscendFusedTopKRouter(
         cfg.k, cfg.E, renormalize=bool(cfg.renorm), use_grouped_topk=cfg.n_group > 1,

@@ -269,6 +269,35 @@ def test_expert_load_collection(fused):
         assert int(layer.moe_load.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("name", ["c2_small", "c5_small"])
+@pytest.mark.parametrize("fused", [True, False])
+def test_redundant_experts_through_log2phy(name, fused):
+    """Two physical copies of logical experts behind the logical -> physical map: the router scores the logical
+    experts, the dispatch runs over the physical ones, the output is the one of the layer without copies, and
+    the tokens of a remapped expert are counted on its copy."""
+    print(f"log2phy {name} fused={fused}", flush=True)
+    cfg = CONFIGS[name]
+    d = make_layer(cfg, seed=4)
+    x, logits = d["x"].to(DEV), d["logits"].to(DEV)
+    plain = build_layer(cfg, d, DEV)
+    want = plain.forward_impl(x, logits)
+    layer = build_layer(cfg, d, DEV, redundant=(3, 1))
+    layer.use_fused_small_batch = fused
+    log2phy = torch.arange(cfg.E, dtype=torch.int32, device=DEV)
+    log2phy[3] = cfg.E  # every token of logical expert 3 goes to its copy; the copy of expert 1 stays idle
+    layer.log2phy = log2phy
+    got = layer.forward_impl(x, logits)
+    torch.cuda.synchronize()
+    assert torch.equal(got.routed_out, want.routed_out)
+    assert np.array_equal(bits(got.routed_out), oracle_layer(cfg, d).out)
+    counts, base = got.expert_tokens.cpu(), want.expert_tokens.cpu()
+    assert counts.shape[0] == cfg.E + 2 and int(counts[3]) == 0 and int(counts[cfg.E + 1]) == 0
+    assert int(counts[cfg.E]) == int(base[3])
+    keep = [e for e in range(cfg.E) if e != 3]
+    assert torch.equal(counts[keep], base[keep])
+    assert layer.get_log2phy_map() is log2phy
+
+
 @pytest.mark.parametrize("name", ["c2_small", "c4_small", "c5_small"])
 def test_empty_and_single_token_batches(name):
     """T = 0 (a rank with nothing to do in a padded step) returns an empty result without launching anything

@@ -66,9 +66,9 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     const int nb0 = (EPI == EPI_SWIGLU) ? p : 2 * p;
     const int nb1 = (EPI == EPI_SWIGLU) ? p + upe : 2 * p + 1;
 
-    // K is cut into gridDim.y slabs (1 except for the dense small-batch product, whose workgroups add their int32
-    // partial sums into a zeroed result with atomics: integer addition, exact and order free), and a slab into
-    // KSPLIT pieces, one per wavefront
+    // K is cut into gridDim.y slabs (SLABS: the dense few-row product, whose workgroups store their int32 partial
+    // sums to a plane per slab, or without scratch add them into a zeroed result with atomics: integer addition,
+    // exact and order free), and a slab into KSPLIT pieces, one per wavefront
     const int ks = (KSPLIT == 1) ? 0 : wave;
     int slab_begin = 0, slab_end = KB;
     if constexpr (SLABS) {

@@ -33,6 +33,9 @@ class AscendRoutedExperts(torch.nn.Module):
         self.ascend_mc2_mask = None
         self.ascend_pertoken_scale = None
         self.enable_force_load_balance = False  # profile runs only (routed_experts.py:484-492)
+        # logical -> physical expert ids when the layer holds redundant copies of experts (dynamic load balancing,
+        # routed_experts.py:250, 452-453): the router scores the logical experts, the weights are the physical ones
+        self.log2phy = None
         # small batches (decode): gating and dispatch in one launch when the scheme has the fused form
         self.use_fused_small_batch = True
         specs = dict(quant_method.get_weight(moe_config.num_experts, moe_config.intermediate_size_per_partition,
@@ -73,6 +76,9 @@ class AscendRoutedExperts(torch.nn.Module):
             p = getattr(self, name)
             p.data.copy_(t.reshape(p.data.shape).to(p.data.dtype))
         self.quant_method.process_weights_after_loading(self)
+
+    def get_log2phy_map(self) -> torch.Tensor | None:
+        return self.log2phy
 
     def clear_moe_load(self) -> None:
         """Zero the collected expert loads (routed_experts.py:423-428)."""
@@ -118,6 +124,8 @@ class AscendRoutedExperts(torch.nn.Module):
         topk_weights, topk_ids = self.router.select_experts(
             hidden_states, router_logits, enable_force_load_balance=self.enable_force_load_balance,
             weights_dtype=weights_dtype)
+        if self.log2phy is not None:
+            topk_ids = self.log2phy[topk_ids.long()].to(topk_ids.dtype)
         return self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
 
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None) -> torch.Tensor:

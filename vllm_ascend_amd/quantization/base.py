@@ -61,6 +61,8 @@ def fused_front_supported(layer, x: torch.Tensor, router_logits: torch.Tensor, r
         return False
     if getattr(layer, "enable_force_load_balance", False):
         return False
+    if getattr(layer, "log2phy", None) is not None:  # the ids are remapped between gating and dispatch
+        return kernels.gate_quant_supported(x.shape[0], router.top_k, router_logits.shape[1])
     return (kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
             or kernels.gate_quant_supported(x.shape[0], router.top_k, router_logits.shape[1]))
 
@@ -82,7 +84,8 @@ def route_and_quantize(layer, x: torch.Tensor, router_logits: torch.Tensor, rout
                  router.num_expert_group if router.num_expert_group is not None else 1, 1,
                  int(router.renormalize), 0 if router.scoring_func == "softmax" else 1,
                  router.routed_scaling_factor, 1e-20, bias)
-    if kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1]):
+    log2phy = getattr(layer, "log2phy", None)
+    if log2phy is None and kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1]):
         # the routing kernel's arrival counter: one zeroed int32 per layer (and device), which every call leaves
         # at zero; created on the first call (run the layer once before capturing it into a graph)
         counter = getattr(layer, "_small_batch_counter", None)
@@ -90,5 +93,11 @@ def route_and_quantize(layer, x: torch.Tensor, router_logits: torch.Tensor, rout
             counter = layer._small_batch_counter = torch.zeros((1,), dtype=torch.int32, device=x.device)
         return kernels.route_quant_small(x, router_logits, *gate_args, sync_counter=counter)
     topk_weights, topk_ids, xq, x_scale = kernels.gate_quant(x, router_logits, *gate_args)
-    expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, router_logits.shape[1], 1)
+    num_experts = router_logits.shape[1]
+    if log2phy is not None:
+        # logical -> physical expert ids (redundant experts of dynamic load balancing,
+        # vllm_ascend/ops/fused_moe/routed_experts.py:452-453): the dispatch runs over the physical experts
+        topk_ids = log2phy[topk_ids.long()].to(torch.int32)
+        num_experts = layer.moe_config.num_experts
+    expanded_row_idx, row_token, expert_tokens = kernels.route_map(topk_ids, num_experts, 1)
     return topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens
