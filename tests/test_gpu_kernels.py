@@ -208,7 +208,15 @@ def test_route_quant_small_equals_gating_plus_init_routing(K, orc, case):
                                                       (1500, 6, 256, 7168, 1, 1, True, 8, 4, 2.5, torch.bfloat16,
                                                        torch.bfloat16),
                                                       (700, 2, 40, 200, 1, 0, True, 4, 2, 1.0, torch.float16,
-                                                       torch.float16)])
+                                                       torch.float16),
+                                                      # long rows (several passes of the workgroup over a row) and
+                                                      # a row shorter than a wavefront, on more than a thousand tokens
+                                                      (1100, 2, 16, 8192, 0, 1, False, 1, 1, 1.0, torch.float32,
+                                                       torch.bfloat16),
+                                                      (1030, 2, 16, 8200, 0, 1, False, 1, 1, 1.0, torch.float32,
+                                                       torch.float16),
+                                                      (2049, 4, 64, 72, 1, 1, False, 1, 1, 1.0, torch.bfloat16,
+                                                       torch.bfloat16)])
 def test_gate_quant_equals_gating_plus_dynamic_quant(K, orc, case):
     """Gating and token quantisation in one launch (any number of tokens) against the two separate kernels."""
     T, k, E, H, norm_type, renorm, use_bias, G, k_group, rsf, ldt, xdt = case
