@@ -37,13 +37,18 @@ def _make(cfg, seed=0):
     return dg, to_cpu(dg)
 
 
-@pytest.mark.parametrize("name", ["c3_qwen3_prefill", "c4_dsv3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode"])
+@pytest.mark.parametrize("name", ["c3_qwen3_prefill", "c4_dsv3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode",
+                                  "c3_qwen3_prefill@32768"])
 def test_full_size_properties_and_sampled_rows(K, orc, name):
     """The benchmark configurations at their full sizes (all 256 experts of the DeepSeek-V3 shapes, 4096 / 512 / 64
-    tokens), stage by stage."""
+    tokens), stage by stage; "name@T": the same shape on a batch of T tokens (four times the benchmark's prefill
+    batch: 262,144 sorted rows)."""
+    import dataclasses
+
     from _parity import layer_parity, staged_run
 
-    cfg = CONFIGS[name]
+    base, _, tokens = name.partition("@")
+    cfg = CONFIGS[base] if not tokens else dataclasses.replace(CONFIGS[base], T=int(tokens))
     print(f"full size {name}: T={cfg.T} E={cfg.E} H={cfg.H} I={cfg.I}", flush=True)
     dg, dc = _make(cfg)
     print("  tensors ready", flush=True)
