@@ -631,6 +631,38 @@ def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
+def test_w4_scales_of_every_magnitude(K, orc):
+    """Subnormal scales, scales near the bottom of the normal range, zero and negative scales next to ordinary
+    ones give the checker's bits (a token scale of 2^90 brings the tiny products into bf16 range)."""
+    Kd, N, gsz = 256, 128, 128
+    g = torch.Generator().manual_seed(11)
+    cnt = torch.tensor([40, 70], dtype=torch.int64)
+    cum = torch.cumsum(cnt, 0)
+    R = int(cnt.sum())
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-8, 8, (2, N, Kd), generator=g, dtype=torch.int8)
+    sx = torch.full((R,), 2.0 ** 90)
+    w4 = K.format_cast_nz_int4(w.to(DEV), 0, N, Kd)
+    base = torch.rand(2, Kd // gsz, N, generator=g) * 0.09 + 0.01
+    variants = {"ordinary": base.clone()}
+    t = base.clone()
+    t[0, :, 5] = 1.0000001e-38                  # subnormal
+    t[1, 0, 70] = 1.2345678 * 2.0 ** -124       # normal, a sixteenth of it is not
+    t[1, 1, 3] = 0.0
+    t[0, 1, 9] = -0.05
+    variants["tiny"] = t
+    t = base.clone() * 2.0 ** -100              # small everywhere
+    t[0, 0, 64] = 2.0 ** -122
+    variants["small"] = t
+    for name, sg in variants.items():
+        f = orc.gmm_w4_grouped(x.numpy(), w.numpy(), sg.numpy(), cum.numpy(), gsz)
+        want = orc.w4_rows_to_bf16(f, sx.numpy())
+        got = K.gmm2_dequant_w4(x.to(DEV), w4, sg.to(DEV), gsz, sx.to(DEV), cum.to(DEV), 0, N, Kd)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(got.cpu()), want), name
+        assert np.count_nonzero(want) > want.size // 2, name
+
+
 def test_w4_group_sum_order_on_the_gpu(K, orc):
     """The order-sensitive case of the CPU suite (terms 2^24, 1, 1 over three scale groups) through the kernel."""
     Kd, g, N = 192, 64, 64
