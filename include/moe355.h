@@ -292,6 +292,15 @@ int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, cons
 int moe355_w4_offset_correction(const uint8_t *weight_nz4, const float *weight_scale, int64_t group_size,
                                 int num_experts, int64_t n, int64_t k, float *corr, void *stream);
 
+/* The gate function of the SwiGLU epilogues by itself: out[i] = g[i] / (1 + exp(-g[i])) in fp32, n values.
+ * form 0: the instruction sequence every kernel of this library runs (a division specialised to a divisor in
+ * [1, 2^128)); form 1: the same function with the general IEEE division, which is the definition
+ * (csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:461-485,
+ * csrc/gmm/grouped_matmul_swiglu_quant/README.md:63-67) and what the CPU checker computes.  No operator of the
+ * reference stands behind it: it exists so that a test can run both forms over all 2^32 inputs and find them
+ * equal bit for bit. */
+int moe355_silu_f32(const float *g, float *out, int64_t n, int form, void *stream);
+
 /* ---------------------------------------------------------------------------
  * down grouped GEMM (int8 x int8 -> int32) + dequant to bf16.
  * Stands in for torch_npu.npu_grouped_matmul(scale=, per_token_scale=,

@@ -31,6 +31,9 @@
  *   orc_dynamic_quant   : closed forms (identity rows, zero rows, .5 ties)
  *                         rounding rule itself: PARITY UNPINNED (torch_npu binary)
  *   orc_gmm_i32         : numpy int64 matmul (exact)
+ *   orc_silu            : float64 g / (1 + exp(-g)) within 3 units in the last place on a dense grid,
+ *                         the closed forms silu(g) = g for g >= 17.4, silu(0) = 0, silu(-0) = -0 and the
+ *                         values orc_swiglu_quant returns for the same gates (one expression, two places)
  *   orc_swiglu_quant    : numpy rendering of the reference golden
  *                         (test_gmm_swiglu_quant_weight_nz_tensor_list.py:14-99), +-1 LSB
  *   orc_gmm2_dequant    : numpy float64 product, bf16 rounding closed forms
@@ -565,6 +568,20 @@ ORC_API int orc_swiglu_quant(const float *f, int64_t rows, int64_t N, float swig
         }
         free(y);
     }
+    return 0;
+}
+
+/*
+ * The gate function of the SwiGLU by itself, element by element: out[i] = g[i] / (1 + exp(-g[i])) with the
+ * IEEE division of C (README formula csrc/gmm/grouped_matmul_swiglu_quant/README.md:63-67, kernel
+ * csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:461-485).  The same expression
+ * as inside orc_swiglu_quant; exported so that the GPU's instruction sequence for it can be compared on
+ * arbitrary bit patterns.
+ */
+ORC_API int orc_silu(const float *g, int64_t n, float *out)
+{
+#pragma omp parallel for
+    for (int64_t i = 0; i < n; ++i) out[i] = g[i] / (1.0f + orc_expf(-g[i]));
     return 0;
 }
 

@@ -293,6 +293,14 @@ def swiglu_quant(f, swiglu_limit=0.0, want_y=False):
     return (q, qs, y) if want_y else (q, qs)
 
 
+def silu(g):
+    """g / (1 + exp(-g)) element by element in binary32 (the gate function of the SwiGLU)."""
+    g = np.ascontiguousarray(g, dtype=np.float32)
+    out = np.empty_like(g)
+    lib().orc_silu(_p(g), _i64(g.size), _p(out))
+    return out
+
+
 def gmm2_dequant(acc, s1, s2, cum):
     acc = np.ascontiguousarray(acc, dtype=np.int32)
     s1 = np.ascontiguousarray(s1, dtype=np.float32)

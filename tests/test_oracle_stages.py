@@ -219,6 +219,30 @@ def test_swiglu_quant_closed_forms():
     assert s3[0] == 0 and not q3.any()
 
 
+def test_silu_against_float64_and_closed_forms():
+    """orc_silu pinned outside itself: the float64 quotient on a dense grid, the exact regions, the SwiGLU stage."""
+    g = np.concatenate([np.linspace(-87.0, 20.0, 200001), np.linspace(-1e-3, 1e-3, 2001)]).astype(np.float32)
+    got = orc.silu(g).astype(np.float64)
+    g64 = g.astype(np.float64)
+    want = g64 / (1.0 + np.exp(-g64))
+    ulp = np.spacing(np.abs(want).astype(np.float32)).astype(np.float64)
+    # exp() is within 2 units (its own pin), 1 + E and the quotient add half a unit each
+    assert np.all(np.abs(got - want) <= 3.0 * ulp)
+    # 1 + exp(-g) rounds to 1 from g = 17.33 on (exp(-g) < 2^-25): the quotient is g itself
+    big = np.array([17.4, 18.0, 100.0, 1e10, 3e38], dtype=np.float32)
+    assert np.array_equal(orc.silu(big), big)
+    z = orc.silu(np.array([0.0, -0.0], dtype=np.float32))
+    assert z[0] == 0.0 and z[1] == 0.0 and not np.signbit(z[0]) and np.signbit(z[1])
+    # far negative: the divisor stays finite (the exponential's argument is clamped at 88.72283)
+    far = orc.silu(np.array([-90.0, -1e30], dtype=np.float32))
+    assert np.all(np.isfinite(far)) and np.all(far < 0)
+    # the SwiGLU stage with up = 1 returns exactly these values
+    gates = np.linspace(-30.0, 30.0, 64).astype(np.float32)
+    f = np.concatenate([gates, np.ones_like(gates)])[None, :]
+    _, _, y = orc.swiglu_quant(f, want_y=True)
+    assert np.array_equal(y[0], orc.silu(gates))
+
+
 def test_token_scale_is_applied_before_the_channel_scale():
     """csrc/gmm/grouped_matmul_swiglu_quant/op_kernel/grouped_matmul_swiglu_quant.h:387-399 then :448-459.
     Chosen so that the two orders differ in the last bit."""

@@ -91,7 +91,34 @@ __device__ __forceinline__ float m_expf(float x)
     return __builtin_ldexpf(y, (int)n);
 }
 
-__device__ __forceinline__ float m_silu(float g) { return g / (1.0f + m_expf(-g)); }
+// silu(g) = g / (1 + exp(-g)) with the IEEE quotient written out: the definition, and what the CPU checker
+// computes.  The kernels run m_silu below; this form is kept for the test that compares the two on every
+// binary32 input.
+__device__ __forceinline__ float m_silu_ieee(float g) { return g / (1.0f + m_expf(-g)); }
+
+// The same function of g, bit for bit on all 2^32 inputs (NaN in, NaN out), in seven instructions behind the
+// exponential instead of the twelve of a general division.  The general sequence scales both operands into the
+// range of the hardware reciprocal, refines the reciprocal, corrects the quotient twice and repairs the special
+// cases; here the divisor d = 1 + E is known to lie in [1, 2^128), which leaves one hazard: v_rcp_f32 flushes
+// results below 2^-126, i.e. for d > 2^126 (g < -87.3).  Negative g therefore divide by d / 4 (a power of two
+// commutes with every rounding involved: c * (1 + E) rounds like 1 + E) and scale the quotient back, which is
+// exact too since 4 g / d stays far from overflow when E > 1; non-negative g divide by d itself (4 g would
+// overflow for g > 2^126, and g / 4 would lose bits of subnormal g).  With a divisor in [1/4, 2^126] the
+// reciprocal is within one unit, q0 within two, and one residual correction gives the correctly rounded
+// quotient for every g -- not by a general theorem (the correction step can miss in a tie-like case for some
+// operand pairs) but because d is a function of g: the pairs that occur are 2^32 and a test runs them all.
+// v_div_fixup_f32 restores the two cases the chain cannot get right, the sign of g = -0 and g = +-inf.
+__device__ __forceinline__ float m_silu(float g)
+{
+    const float E = m_expf(-g);
+    const float c = g < 0.0f ? 0.25f : 1.0f;
+    const float ds = __builtin_fmaf(E, c, c);
+    const float r = __builtin_amdgcn_rcpf(ds);
+    const float q0 = g * r;
+    const float e = __builtin_fmaf(-ds, q0, g);
+    const float q1 = __builtin_fmaf(e, r, q0);
+    return __builtin_amdgcn_div_fixupf(q1 * c, ds, g);
+}
 
 // clamp(rint(v), -128, 127) as int8
 __device__ __forceinline__ int8_t sat_rint_i8(float v)

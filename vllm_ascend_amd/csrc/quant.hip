@@ -165,9 +165,30 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
     }
 }
 
+// out[i] = silu(g[i]) by the kernels' instruction sequence (form 0) or by the IEEE quotient (form 1)
+template <int FORM>
+__global__ __launch_bounds__(256) void silu_f32_kernel(const float* __restrict__ g, float* __restrict__ out,
+                                                       int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = FORM == 0 ? m_silu(g[i]) : m_silu_ieee(g[i]);
+}
+
 }  // namespace moe355
 
 using namespace moe355;
+
+extern "C" int moe355_silu_f32(const float* g, float* out, int64_t n, int form, void* stream)
+{
+    if (n < 0 || (form != 0 && form != 1)) return MOE355_E_ARG;
+    if (n == 0) return MOE355_OK;
+    if (!g || !out) return MOE355_E_ARG;
+    if ((n + 255) / 256 > 0x7fffffffLL) return MOE355_E_SHAPE;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (form == 0) hipLaunchKernelGGL(silu_f32_kernel<0>, grid, dim3(256), 0, (hipStream_t)stream, g, out, n);
+    else hipLaunchKernelGGL(silu_f32_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, g, out, n);
+    return launch_status();
+}
 
 extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q, float* scale,
                                     void* stream)
