@@ -10,7 +10,8 @@ the configuration has one) over one batch of synthetic tokens, through the plugi
 Without --workload every configured workload runs in this one process: the DeepSeek-V3-shaped 4096-token prefill
 (the largest single-GPU configuration and the shape the target is stated on: the top-level `value`, `ms_per_step`,
 `roofline` and `cpu_baseline` are its figures), the Qwen3-30B-A3B-shaped decode and prefill batches, the W4A8
-Zipf-routed batch and the DeepSeek-V3-shaped 64-token decode batch; `workloads` carries the same figures for each.
+Zipf-routed batch, the DeepSeek-V3-shaped 64-token decode batch and the same shape with int8 weights under
+Zipf(1.1)-skewed routing at 512 and 4096 tokens; `workloads` carries the same figures for each.
 Inputs are resident in HBM before the timed region (they are drawn on the GPU by a seeded generator).
 Per workload:
   ms_per_step   K timed steps (one HIP-graph replay per step) after W warm-up steps
@@ -20,7 +21,8 @@ Per workload:
                 histogram and the first int8 quantisation on the whole batch; both int32 accumulators, the int8 SwiGLU
                 output, the expert output and the final output on sampled rows / tokens) and the relative error of
                 the 16-bit output against a reference without activation quantisation
-  cpu_baseline  the CPU checker (a C port with OpenMP) timed on this host on a bounded sample of the same batch
+  cpu_baseline  a torch-native CPU rendering of the layer (torch.matmul on int32 tensors; oracle/torch_native.py) timed
+                on this host on a bounded sample of the same batch, with the C checker (OpenMP) beside it as `c_port`
 """
 from __future__ import annotations
 
@@ -40,7 +42,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
 HEADLINE = "c4_dsv3_prefill"
-WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode"]
+WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode",
+             "c7_w8a8_zipf", "c7_w8a8_zipf_4096"]
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (FETCH_SIZE / WRITE_SIZE scaled by a copy
 # kernel of known size), taken from the committed summaries: NOT measured in this run.
@@ -307,6 +310,7 @@ def run_workload(name, args, lib, torch, np):
 
     # ---------------- parity gates against the CPU checker
     dc = None
+    gpu_expert_rows = None
     if not args.no_parity or not args.no_cpu_baseline:
         t0 = time.perf_counter()
         dc = to_cpu(dg)
@@ -321,6 +325,7 @@ def run_workload(name, args, lib, torch, np):
                               shared=cfg.shared)
         parity["seconds"] = round(time.perf_counter() - t0, 1)
         out["parity"] = parity
+        gpu_expert_rows = r["o"]  # kept for the torch-native CPU leg below
         del r
         log(f"{name}: parity {'FAILED ' + str(parity['failed']) if parity['failed'] else 'ok'} "
             f"in {parity['seconds']} s")
@@ -346,16 +351,45 @@ def run_workload(name, args, lib, torch, np):
         from _inputs import bits
 
         ok = bool(np.array_equal(bits(res.routed_out[:sample_T]), tr.out))
-        out["cpu_baseline"] = {
+        c_port = {
             "value": round(sample_T * passes / elapsed, 2), "unit": "tokens/s", "cores": orc.num_threads(),
-            "kind": "port",
+            "kind": "port", "rendering": "the C checker (oracle/moe_oracle.c) with OpenMP",
             "sample": f"the first {sample_T} of {cfg.T} tokens of the same workload, {passes} pass(es) of the whole "
                       f"layer in {elapsed:.2f} s",
             "gpu_output_bit_exact_vs_cpu_on_sample": ok}
-        log(f"{name}: CPU baseline {out['cpu_baseline']['value']} tokens/s ({passes} passes, {elapsed:.1f} s)")
+        log(f"{name}: CPU baseline (C port) {c_port['value']} tokens/s ({passes} passes, {elapsed:.1f} s)")
+        # the torch-native rendering: plain torch CPU operators, the expert MLPs on all rows of the busiest experts
+        # (the workload's own rows-per-expert regime) and extrapolated linearly in rows
+        from oracle import torch_native
+
+        per_row = algorithmic_ops(dataclasses.replace(cfg, shared=False), 1)
+        tn = torch_native.timed_layer(cfg, dc, max_rows=max(64, int(args.cpu_torch_ops / per_row)), max_experts=16,
+                                      threads=orc.num_threads())
+        rel = None
+        if gpu_expert_rows is not None and tn["row_ranges"]:
+            a = torch.cat([tn["expert_rows"][lo:hi] for lo, hi in tn["row_ranges"]]).double()
+            b = torch.cat([gpu_expert_rows[lo:hi].cpu() for lo, hi in tn["row_ranges"]]).double()
+            rel = float((a - b).norm() / b.norm().clamp_min(1e-30))
+        out["cpu_baseline"] = {
+            "value": round(tn["tokens_per_s"], 2), "unit": "tokens/s", "cores": tn["threads"],
+            "kind": "torch-native", "kind_in_the_terms_of_the_contract": "port",
+            "dtype_path": "torch.matmul on int32 CPU tensors (int8 activations and weights widened; the weights once, "
+                          "outside the timed region), fp32 scales and SwiGLU, "
+                          + ("per-group fp32 accumulation over int4 groups" if cfg.w4_group > 0 else
+                             "per-channel scales"),
+            "sample": f"routing, quantisation, dispatch and combine on all {cfg.T} tokens; expert MLPs on "
+                      f"{tn['rows_sampled']} rows of the {tn['experts_sampled']} busiest experts, scaled to the "
+                      f"{tn['rows']} rows of the batch" + (f"; shared expert on {min(cfg.T, 256)} rows, scaled"
+                                                          if cfg.shared else ""),
+            "seconds_by_part": tn["seconds"],
+            "rel_err_of_its_expert_rows_vs_gpu": rel,
+            "c_port": c_port}
+        log(f"{name}: CPU baseline (torch-native) {out['cpu_baseline']['value']} tokens/s, parts {tn['seconds']}, "
+            f"expert rows vs GPU rel {rel}")
+        del tn
     else:
         out["cpu_baseline"] = None
-    del layer, dg, dc, graph
+    del layer, dg, dc, graph, gpu_expert_rows
     torch.cuda.empty_cache()
     log(f"{name}: {out['us_per_layer']} us per layer, done in {time.perf_counter() - t_start:.1f} s")
     return out
@@ -373,6 +407,8 @@ def main() -> int:
                     help="start the step one operator earlier: the fp32 router gate GEMM (hidden states -> logits, "
                          "random fp32 weight) runs inside every step; the headline metric starts at the logits")
     ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU-baseline time per workload")
+    ap.add_argument("--cpu-torch-ops", type=float, default=1.2e11,
+                    help="integer operations the torch-native CPU leg spends on its sample of expert rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")

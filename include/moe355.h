@@ -156,8 +156,10 @@ int moe355_init_routing_prequant(const int8_t *x, const float *x_scale, int64_t 
  * ends; its address is looked up once per device, on the first call with that device current.  The call itself
  * allocates and frees nothing.  Batches whose scratch (moe355_init_routing_workspace) does not fit the array are
  * rejected with MOE355_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on one
- * GPU (different streams, different threads) race and must be serialised by the caller.  Results are identical
- * to moe355_init_routing's. */
+ * GPU (different streams, different threads) race and must be serialised by the caller.  The address is cached
+ * for the device that is current at the call, which must be the device that owns `stream`; the first call on a
+ * device does that lookup (host-side runtime work) and must therefore be made outside stream capture.  Results
+ * are identical to moe355_init_routing's. */
 #define MOE355_INIT_ROUTING_STATIC_BYTES (2u << 20)
 int moe355_init_routing_static(const void *x, int x_dtype, int64_t num_tokens, int64_t hidden,
                                const int32_t *expert_idx, int top_k, int num_experts, int quant_mode,

@@ -39,6 +39,13 @@ CONFIGS = {
     # the north star's decode target: the DeepSeek-V3 shape with a 64-token batch
     "c6_dsv3_decode": LayerCfg("c6_dsv3_decode", 64, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8, topk_group=4,
                                routed_scaling_factor=2.5, bias=True, shared=True),
+    # W8A8 under skewed routing: the DeepSeek-V3 shape with Zipf(1.1) expert popularity, a small and a prefill batch
+    "c7_w8a8_zipf": LayerCfg("c7_w8a8_zipf", 512, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8, topk_group=4,
+                             routed_scaling_factor=2.5, bias=True, zipf=1.1),
+    "c7_w8a8_zipf_4096": LayerCfg("c7_w8a8_zipf_4096", 4096, 7168, 256, 8, 2048, scoring="sigmoid", n_group=8,
+                                  topk_group=4, routed_scaling_factor=2.5, bias=True, zipf=1.1),
+    "c7_small": LayerCfg("c7_small", 512, 512, 64, 4, 256, scoring="sigmoid", n_group=8, topk_group=4,
+                         routed_scaling_factor=2.5, bias=True, zipf=1.1),
     "c5_small": LayerCfg("c5_small", 80, 512, 32, 4, 256, scoring="sigmoid", n_group=4, topk_group=2,
                          routed_scaling_factor=2.5, bias=True, w4_group=128, zipf=1.1),
     "c5_small_perchannel": LayerCfg("c5_small_perchannel", 40, 256, 16, 2, 128, w4_group=0),

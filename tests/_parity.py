@@ -213,6 +213,15 @@ def layer_parity(orc, cfg: LayerCfg, dc: dict, r: dict, n_tokens: int = 8, seed:
         res["rel_err_vs_quantized_fp64_reference"] = float(np.linalg.norm(got - ref_q) /
                                                            max(np.linalg.norm(ref_q), 1e-30))
         res["max_abs_err_vs_quantized_fp64_reference"] = float(np.abs(got - ref_q).max())
+    if cfg.w4_group < 0:
+        # where that error comes from: the reference's golden math in numpy (no checker code) on the same tokens,
+        # routed experts only, with the first / the second / both activation quantisers in place
+        from _noise import error_split
+
+        sp = error_split(x_tok, w_tok, ids_want[tokens], w13, dc["s13"].numpy(), w2, dc["s2"].numpy())
+        res["rel_err_split_routed_experts_golden_math"] = {
+            "first_quant_only": sp["first_quant_only"], "second_quant_only": sp["second_quant_only"],
+            "both": sp["both"]}
     res["failed"] = failed
     return res
 

@@ -38,7 +38,7 @@ def _make(cfg, seed=0):
 
 
 @pytest.mark.parametrize("name", ["c3_qwen3_prefill", "c4_dsv3_prefill", "c5_w4a8_zipf", "c6_dsv3_decode",
-                                  "c3_qwen3_prefill@32768"])
+                                  "c3_qwen3_prefill@32768", "c7_w8a8_zipf", "c7_w8a8_zipf_4096"])
 def test_full_size_properties_and_sampled_rows(K, orc, name):
     """The benchmark configurations at their full sizes (all 256 experts of the DeepSeek-V3 shapes, 4096 / 512 / 64
     tokens), stage by stage; "name@T": the same shape on a batch of T tokens (four times the benchmark's prefill

@@ -631,6 +631,55 @@ def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
+# Skewed histograms: the host picks a kernel family from the mean rows per expert and the device splits the
+# experts between that family and the 128-row tiles.  Mean below 48 with at least 1024 rows: streaming up to 32
+# rows, tiles above (rows at 31 / 32 / 33 sit on the border).  The other two cases keep one family (the
+# weight-streaming tiles) over experts far above and below its range: 255 / 256 / 257 / 511 / 513 rows.
+SKEWED = {
+    "stream+tiled": ([0, 1, 31, 32, 33, 2, 64, 65, 700, 3, 0, 5, 129, 7, 1, 0] + [4] * 48, 256),
+    "stream+tiled, nothing above the border": ([16] * 40 + [32] * 24, 192),
+    "wide": ([255, 256, 257, 511, 513, 1, 0, 33, 128, 160, 161, 192, 193, 40, 90, 100], 1024),
+    "wide, K 4096": ([300, 20, 256, 257, 47, 150, 0, 90], 4096),
+}
+
+
+@pytest.mark.parametrize("name", list(SKEWED))
+@pytest.mark.parametrize("gl_type", [0, 1])
+def test_grouped_gemms_on_skewed_histograms(K, orc, name, gl_type):
+    from vllm_ascend_amd._lib import W_ENK, load
+
+    counts, Kd = SKEWED[name]
+    N = 256
+    cnt = torch.tensor(counts, dtype=torch.int64)
+    E, R = len(counts), int(cnt.sum())
+    print(f"skewed gemm {name}: E={E} R={R} K={Kd} N={N} gl_type={gl_type}", flush=True)
+    lib = load()
+    for epi in (0, 1, 2):
+        kn = lib.moe355_gmm_kernel_name(epi, R, Kd, N, E).decode()
+        assert name.split(",")[0].split("+")[0] in kn and ("+ gmm_tiled_kernel" in kn) == ("+" in name)
+    g = torch.Generator().manual_seed(len(counts) + Kd)
+    cum = torch.cumsum(cnt, 0)
+    gl = (cum if gl_type == 0 else cnt).to(DEV)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    acc = K.gmm_i32(x.to(DEV), wnz, gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    want = orc.gmm2_dequant(ref, sx.numpy(), sw.numpy(), cum.numpy())
+    got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got.cpu()), want)
+    q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw.numpy(), cum.numpy()))
+    q, s_ = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), gl, gl_type, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
 def test_w4_scales_of_every_magnitude(K, orc):
     """Subnormal scales, scales near the bottom of the normal range, zero and negative scales next to ordinary
     ones give the checker's bits (a token scale of 2^90 brings the tiny products into bf16 range)."""

@@ -14,7 +14,7 @@ DEV = "cuda:0"
 # fused: small batches take the four-launch form (gating + dispatch in one kernel) unless it is switched off;
 # c3_small (2560 pairs) is beyond it either way
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("name", ["c1_tiny", "c2_small", "c3_small", "c4_small", "c2_qwen3_decode"])
+@pytest.mark.parametrize("name", ["c1_tiny", "c2_small", "c3_small", "c4_small", "c7_small", "c2_qwen3_decode"])
 def test_layer_bit_exact(name, fused):
     from oracle import oracle as orc
 
@@ -211,6 +211,26 @@ def test_force_load_balance_routes_every_token_to_k_distinct_experts():
     assert torch.isfinite(res.routed_out.float()).all()
     w, ids = layer.router.select_experts(d["x"].to(DEV), d["logits"].to(DEV), enable_force_load_balance=True)
     assert all(len(set(r)) == cfg.k for r in ids.cpu().tolist())
+
+
+def test_force_load_balance_with_log2phy_keeps_the_random_ids_unmapped():
+    """Both profile-run flags at once: the reference maps through log2phy and then overwrites the ids with random
+    logical ids that are not mapped again (routed_experts.py:452-492), so no token may land on a redundant copy."""
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=0)
+    layer = build_layer(cfg, d, DEV, redundant=(3, 1))
+    log2phy = torch.arange(cfg.E, dtype=torch.int32, device=DEV)
+    log2phy[3] = cfg.E
+    log2phy[1] = cfg.E + 1
+    layer.log2phy = log2phy
+    layer.enable_force_load_balance = True
+    res = layer.forward_impl(d["x"].to(DEV), d["logits"].to(DEV))
+    torch.cuda.synchronize()
+    counts = res.expert_tokens.cpu()
+    assert int(counts.sum()) == cfg.T * cfg.k
+    assert int(counts[cfg.E:].sum()) == 0          # the copies stay idle: ids were not mapped
+    assert int(counts[3]) + int(counts[1]) > 0     # ... and the logical experts 1 and 3 are used as they are
+    assert torch.isfinite(res.routed_out.float()).all()
 
 
 def test_layer_with_per_expert_weight_lists():

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
 
     int64_t row0, row1;
     expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
+    if (!expert_in_launch(a, row1 - row0)) return;  // another kernel of this operator call covers the expert
     if (row1 > a.R) row1 = a.R;
     if (row1 <= row0) return;
 
@@ -342,20 +343,17 @@ __global__ __launch_bounds__(256) void slab_sum_kernel(const int32_t* __restrict
 }
 
 template <typename KernelT>
-static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs& a)
+static void launch_gemm(KernelT kernel, dim3 grid, hipStream_t st, const GmmArgs& a, hipEvent_t ev0, hipEvent_t ev1)
 {
-    if (t_ev_start && t_ev_stop) {
-        hipExtLaunchKernelGGL(kernel, grid, dim3(256), 0, st, t_ev_start, t_ev_stop, 0, a);
-        t_ev_start = nullptr;
-        t_ev_stop = nullptr;
-    } else {
-        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
-    }
+    if (ev0 || ev1) hipExtLaunchKernelGGL(kernel, grid, dim3(256), 0, st, ev0, ev1, 0, a);
+    else hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
 }
 
 // Rows per expert decide the kernel: few rows -> weight streaming over single wavefronts; many -> LDS-tiled
 // MFMA kernel with 128-row tiles; in between, when K is long enough to amortise a tile's fill and epilogue, the
-// weight-streaming tiles (up to 256 rows) that fetch an expert's weights once.
+// weight-streaming tiles (up to 256 rows) that fetch an expert's weights once.  The host only knows the mean; the
+// histogram may be skewed (real routers are), so next to the family chosen from the mean a second family covers
+// the experts that fall outside its range, picked expert by expert on the device (GemmPlan below).
 static int tiled_bm(const GmmArgs& a)
 {
     if (a.K % 64 != 0) return 0;
@@ -368,11 +366,40 @@ static int tiled_bm(const GmmArgs& a)
 #endif
     const int64_t avg = a.R / a.E;
     if (avg < 48) return 0;
-    if (avg <= 256 && a.K >= 4096) return 256;
+    // the list of 256-row tiles is built from 16-bit counters (tile_map_kernel, by_length)
+    const bool wide_ok = a.R / 256 + a.E < 32768;
+    if (avg <= 256 && a.K >= 4096 && wide_ok) return 256;
     // around 128 rows per expert most experts fit one wide tile of 128 or 160 rows and fetch their weights once,
     // which pays from K = 1024 on (measured: 6 % at K = 2048 and 1024, a loss at K = 768 and at 64 rows)
-    if (avg >= 96 && avg <= 192 && a.K >= 1024) return 256;
+    if (avg >= 96 && avg <= 192 && a.K >= 1024 && wide_ok) return 256;
     return 128;
+}
+
+// What one operator call launches: the family chosen from the mean rows per expert, restricted to the experts it
+// is good at, and (split > 0) the 128-row tiles for the experts above that range.
+//   mean < 48 and at least 1024 rows: streaming for experts of at most 32 rows (one pass over their weights),
+//     tiles for the others -- a 500-row expert would otherwise stream its weights 16 times while the units of
+//     the cold experts have long finished.  Below 1024 rows (decode batches) a second launch costs more than the
+//     few extra passes of a hot expert.
+//   The weight-streaming tiles (mean 48..256) keep every expert: sending those above 256 rows to the 128-row
+//     tiles measured the same on a Zipf(1.1) batch of 32,768 rows (2149 against 2180 us for the gate_up product,
+//     1136 against 1119 us for the down product) and would cost the uniform batches an empty launch.
+struct GemmPlan {
+    int bm;     // 0 streaming, 64 / 128 LDS-tiled, 256 weight-streaming tiles
+    int split;  // > 0: experts with more than `split` rows run on the 128-row tiles instead
+};
+
+static GemmPlan gemm_plan(const GmmArgs& a, bool have_tile_ws)
+{
+    GemmPlan p = {have_tile_ws ? tiled_bm(a) : 0, 0};
+    if (a.E == 1 && a.R <= 64) p.bm = 0;  // dense, few rows: the streaming kernel, one workgroup per 64 channels
+    if (!have_tile_ws || a.K % 64 != 0 || a.E == 1) return p;
+#ifdef MOE355_DEV_KNOBS
+    static const char* force = getenv("MOE355_GEMM");
+    if (force && force[0]) return p;
+#endif
+    if (p.bm == 0 && a.R >= 1024) p.split = 32;
+    return p;
 }
 
 // One expert with enough rows and channels for the 256 x 256 tiles to fill the chip: the dense kernel (measured
@@ -390,7 +417,8 @@ static bool dense_tiles(const GmmArgs& a)
 
 static size_t tiled_ws_max(int64_t rows, int E)
 {
-    return tiled_workspace_bytes(rows, E, 64);  // the smallest tile needs the longest tile list
+    // the smallest tile needs the longest tile list; a call that splits the experts over two families builds two
+    return 2 * ((tiled_workspace_bytes(rows, E, 64) + 255) & ~(size_t)255);
 }
 
 // K slabs of the dense few-row product (one expert, at most 64 rows, a long K, too few pairs of tiles to fill
@@ -410,28 +438,27 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
                             size_t part_bytes = 0)
 {
     GmmArgs a = a_in;
-    int bm = tile_ws ? tiled_bm(a) : 0;
-    // dense, few rows (the shared expert of a decode batch): a 64-row tile map gives one workgroup per 256
-    // channels, the streaming kernel one per 64 (and K slabs on top for the int32 form)
-    if (a.E == 1 && a.R <= 64) bm = 0;
+    hipEvent_t ev0 = t_ev_start, ev1 = t_ev_stop;  // measurement hook: around the GEMM kernels of this call
+    t_ev_start = nullptr;
+    t_ev_stop = nullptr;
     if (dense_tiles(a)) {
-        launch_dense(EPI, a, st, t_ev_start, t_ev_stop);
-        t_ev_start = nullptr;
-        t_ev_stop = nullptr;
+        launch_dense(EPI, a, st, ev0, ev1);
         return launch_status();
     }
-    if (bm) {
-        launch_tiled_any(EPI, bm, a, tile_ws, st, t_ev_start, t_ev_stop);
-        t_ev_start = nullptr;
-        t_ev_stop = nullptr;
-        return launch_status();
-    }
-    const int64_t units = (int64_t)a.E * (a.N / 64);
-    if constexpr (EPI == EPI_I32) {
-        // One expert with at most 64 rows (the shared expert of a decode batch: a dense product over a few tokens):
-        // too few workgroups for a chip that needs thousands of loads in flight to stream at full rate.  K is cut
-        // into slabs, one workgroup per (pair of tiles, slab), partial sums added into the zeroed result.
-        {
+    const GemmPlan plan = gemm_plan(a, tile_ws != nullptr);
+    // the second family's tile map lies behind the first one's
+    void* tile_ws2 = tile_ws ? (char*)tile_ws + ((tiled_workspace_bytes(a.R, a.E, 64) + 255) & ~(size_t)255) : nullptr;
+    if (plan.split > 0) a.rows_max = plan.split;
+    hipEvent_t first_stop = plan.split > 0 ? nullptr : ev1;
+    if (plan.bm) {
+        launch_tiled_any(EPI, plan.bm, a, tile_ws, st, ev0, first_stop);
+    } else {
+        const int64_t units = (int64_t)a.E * (a.N / 64);
+        bool done = false;
+        if constexpr (EPI == EPI_I32) {
+            // One expert with at most 64 rows (the shared expert of a decode batch: a dense product over a few
+            // tokens): too few workgroups for a chip that needs thousands of loads in flight to stream at full rate.
+            // K is cut into slabs, one workgroup per (pair of tiles, slab), partial sums added into the zeroed result.
             const int slabs = dense_slabs(a.R, a.K, a.N, a.E);
             if (slabs > 1) {
                 const int64_t n4 = a.R * (int64_t)a.N / 4;  // N % 64 == 0
@@ -441,22 +468,30 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
                 const bool planes = part_ws && part_bytes >= (size_t)slabs * a.R * a.N * 4;
                 if (planes) a.acc_part = (int32_t*)part_ws;
                 else hipLaunchKernelGGL(zero_i32_kernel, cover, dim3(256), 0, st, a.acc, n4);
-                launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, true>, dim3((unsigned)units, (unsigned)slabs), st, a);
+                launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, true>, dim3((unsigned)units, (unsigned)slabs), st, a, ev0,
+                            first_stop);
                 if (planes)
                     hipLaunchKernelGGL(slab_sum_kernel, cover, dim3(256), 0, st, a.acc_part, slabs, a.R, a.N, a.gl,
                                        a.acc);
-                return launch_status();
+                done = true;
             }
         }
+        // Occupancy 3 keeps the SwiGLU epilogue out of scratch memory (131 registers).  With enough units to
+        // fill the chip four times over and a short K, the down GEMM lets every wavefront stream a whole unit by
+        // itself (no K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K (from
+        // K = 2048 on that measured 1.5 % faster on the whole layer, below it the same or slower).
+        if (done) {
+        } else if (EPI != EPI_SWIGLU && units >= 2048 && a.K < 2048) {
+            launch_gemm(gmm_stream_kernel<EPI, 1, 4, 2>, dim3((unsigned)((units + 3) / 4)), st, a, ev0, first_stop);
+        } else {
+            launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units), st, a, ev0, first_stop);
+        }
     }
-    // Occupancy 3 keeps the SwiGLU epilogue out of scratch memory (131 registers).  With enough units to
-    // fill the chip four times over and a short K, the down GEMM lets every wavefront stream a whole unit by
-    // itself (no K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K (from
-    // K = 2048 on that measured 1.5 % faster on the whole layer, below it the same or slower).
-    if (EPI != EPI_SWIGLU && units >= 2048 && a.K < 2048)
-        launch_gemm(gmm_stream_kernel<EPI, 1, 4, 2>, dim3((unsigned)((units + 3) / 4)), st, a);
-    else
-        launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3>, dim3((unsigned)units), st, a);
+    if (plan.split > 0) {
+        a.rows_min = plan.split + 1;
+        a.rows_max = 0;
+        launch_tiled_any(EPI, 128, a, tile_ws2, st, nullptr, ev1);
+    }
     return launch_status();
 }
 
@@ -481,10 +516,10 @@ extern "C" const char* moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_
     a.N = (int)n;
     a.E = num_experts;
     if (dense_tiles(a)) return "gmm_dense_kernel";
-    const int bm = (a.E == 1 && a.R <= 64) ? 0 : tiled_bm(a);  // as launch_gemm_auto decides
-    if (bm == 256) return "gmm_wide_kernel";
-    if (bm != 0) return "gmm_tiled_kernel";
-    return "gmm_stream_kernel";
+    const GemmPlan p = gemm_plan(a, true);  // as launch_gemm_auto decides
+    if (p.bm == 256) return "gmm_wide_kernel";
+    if (p.bm != 0) return "gmm_tiled_kernel";
+    return p.split ? "gmm_stream_kernel + gmm_tiled_kernel above 32 rows" : "gmm_stream_kernel";
 }
 
 extern "C" int moe355_format_cast_nz(const int8_t* w, int layout, int64_t num_experts, int64_t n, int64_t k,

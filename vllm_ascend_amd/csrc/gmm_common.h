@@ -33,6 +33,9 @@ struct GmmArgs {
     const int8_t* const* w_list;
     const float* const* s_list;
     float limit;            // swiglu clamp
+    // A launch may cover only the experts whose row count lies in [rows_min, rows_max] (rows_max 0: no upper
+    // bound): a batch with a skewed histogram is split over kernel families by expert, on the device.
+    int rows_min, rows_max;
     // outputs
     int32_t* acc;           // EPI_I32   [R, N]
     int32_t* acc_part;      // EPI_I32 with K cut into slabs: [slabs][R, N] partial sums (or null: atomics into acc)
@@ -119,6 +122,12 @@ __device__ __forceinline__ void epilogue_run(const GmmArgs& a, int64_t row, bool
 // First channel, inside a 32-channel tile, of the run that quarter q of a 32x32 accumulator tile holds in
 // this lane: 8*q + 4*(lane/32), four consecutive channels.
 __device__ __forceinline__ int quad_channel(int q, int lane) { return 8 * q + 4 * (lane >> 5); }
+
+// Whether a launch restricted to [a.rows_min, a.rows_max] covers an expert of m rows.
+__device__ __forceinline__ bool expert_in_launch(const GmmArgs& a, int64_t m)
+{
+    return m >= a.rows_min && (a.rows_max == 0 || m <= a.rows_max);
+}
 
 // Measurement hook (gmm.hip): hands out, once, the events that moe355_profile_next_gemm armed on this thread
 // (both null when nothing is armed); the caller records them around exactly one kernel launch.

@@ -20,9 +20,13 @@ namespace moe355 {
 // by_length (the 256-row weight-streaming tiles): the tiles are listed longest first -- 161..192 rows, 129..160,
 // up to 128, then the tall ones (more than 192 rows, which become two shorter column items) -- so that the
 // workgroups that start last are the short ones and the compute units finish closer together.
+// rows_min / rows_max: experts whose row count lies outside [rows_min, rows_max] (rows_max 0: no upper bound) get
+// no tiles (another kernel of the same operator call covers them); their rows still count for the offsets.
 __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict__ gl, int gl_type, int E, int BM,
-                                                       int max_tiles, TileMap tm, int by_length = 0)
+                                                       int max_tiles, TileMap tm, int by_length, int rows_min,
+                                                       int rows_max)
 {
+    auto tiled_rows = [&](int64_t m) -> int64_t { return (m >= rows_min && (rows_max == 0 || m <= rows_max)) ? m : 0; };
     __shared__ int32_t part_rows[16];
     __shared__ int32_t part_tiles[16];
     if (by_length) {
@@ -41,7 +45,7 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
             if (e < E) {
                 const int64_t m = rows_of(e);
                 rows += (int32_t)m;
-                for (int64_t r0 = 0; r0 < m; r0 += BM) {
+                for (int64_t r0 = 0; r0 < tiled_rows(m); r0 += BM) {
                     const int c = cls(m - r0);
                     if (c < 2) n01 += 1 << (16 * c);
                     else n23 += 1 << (16 * (c - 2));
@@ -62,7 +66,7 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
             const int e = e0 + j;
             if (e < E) {
                 const int64_t m = rows_of(e);
-                for (int64_t r0 = 0; r0 < m; r0 += BM) {
+                for (int64_t r0 = 0; r0 < tiled_rows(m); r0 += BM) {
                     const int32_t t = next[cls(m - r0)]++;
                     if (t < max_tiles) {
                         tm.expert[t] = e;
@@ -88,7 +92,7 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
         if (e < E) {
             const int64_t m = rows_of(e);
             rows += (int32_t)m;
-            tiles += (int32_t)((m + BM - 1) / BM);
+            tiles += (int32_t)((tiled_rows(m) + BM - 1) / BM);
         }
     }
     // exclusive prefix of rows and tiles over the threads (experts in order)
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(256) void tile_map_kernel(const int64_t* __restrict
         const int e = e0 + j;
         if (e < E) {
             const int64_t m = rows_of(e);
-            for (int64_t r0 = row; r0 < row + m; r0 += BM) {
+            for (int64_t r0 = row; r0 < row + tiled_rows(m); r0 += BM) {
                 if (t < max_tiles) {
                     tm.expert[t] = e;
                     tm.row_begin[t] = (int32_t)r0;
@@ -612,42 +616,116 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
         load_weights(j + SW - 1, j + SW - 1);
     }
 
-    // One K block on stage uw of the weights and ux of the tokens.  Requests retire in order.  The younger of the
-    // two requests that this step needs is its tokens (its weights, in the same step, if the rings are equally
-    // deep): what was requested after it may still be in flight.  The barrier then covers the other wavefronts and
-    // also says that everybody is done reading the stages that the next requests overwrite.
-    constexpr int NAFTER = (SW > SX) ? NA : 0;  // the weights requested right behind those tokens
-    auto step = [&](int uw, int ux, int it) {
-        if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
-        else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
-        else wait_vmcnt<NAFTER + NA * (SX - 2)>();
-        __builtin_amdgcn_s_barrier();
-        load_tokens(it + SX - 1, (ux + SX - 1) % SX);
-        load_weights(it + SW - 1, (uw + SW - 1) % SW);
-        if (active) {
-            const int8_t* wbase = lds + uw * A_BYTES;
-            const int8_t* xbase = lds + ux * X_BYTES;
+    constexpr int NAFTER = (SW > SX) ? NA : 0;  // the weights requested right behind a step's tokens
+    const int n_full = (n_iter / CYCLE) * CYCLE;
+    if constexpr (WIDE) {
+        // One K block on stage uw of the weights and ux of the tokens.  Requests retire in order.  The younger of
+        // the two requests that this step needs is its tokens (its weights, in the same step, if the rings are
+        // equally deep): what was requested after it may still be in flight.  The barrier then covers the other
+        // wavefronts and also says that everybody is done reading the stages that the next requests overwrite.
+        auto step = [&](int uw, int ux, int it) {
+            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
+            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
+            else wait_vmcnt<NAFTER + NA * (SX - 2)>();
+            __builtin_amdgcn_s_barrier();
+            load_tokens(it + SX - 1, (ux + SX - 1) % SX);
+            load_weights(it + SW - 1, (uw + SW - 1) % SW);
+            if (active) {
+                const int8_t* wbase = lds + uw * A_BYTES;
+                const int8_t* xbase = lds + ux * X_BYTES;
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const v4i a0 = *(const v4i*)(wbase + a_off + s * 1024);
-                const v4i a1 = *(const v4i*)(wbase + a_off + 2048 + s * 1024);
+                for (int s = 0; s < 2; ++s) {
+                    const v4i a0 = *(const v4i*)(wbase + a_off + s * 1024);
+                    const v4i a1 = *(const v4i*)(wbase + a_off + 2048 + s * 1024);
 #pragma unroll
-                for (int b = 0; b < NBLK; ++b) {
-                    const v4i f = *(const v4i*)(xbase + (s ? frag_s1 : frag_s0) + b * 2048);
-                    acc[0][b] = mfma_i8(a0, f, acc[0][b]);
-                    acc[1][b] = mfma_i8(a1, f, acc[1][b]);
+                    for (int b = 0; b < NBLK; ++b) {
+                        const v4i f = *(const v4i*)(xbase + (s ? frag_s1 : frag_s0) + b * 2048);
+                        acc[0][b] = mfma_i8(a0, f, acc[0][b]);
+                        acc[1][b] = mfma_i8(a1, f, acc[1][b]);
+                    }
                 }
             }
+        };
+        for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
+#pragma unroll
+            for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
         }
-    };
-    const int n_full = (n_iter / CYCLE) * CYCLE;
-    for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
 #pragma unroll
-        for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
+        for (int u = 0; u + 1 < CYCLE; ++u)
+            if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
+    } else {
+        // Tall tiles are bound by the matrix units, and every wavefront meets the others at the barrier of every K
+        // block: operand reads that start behind that barrier leave all eight wavefronts, both of each SIMD, without
+        // an MFMA to issue until the first LDS answer is back.  So the operands stay one K step (32 values) ahead in
+        // registers, across the barrier: a block waits for the stage AFTER its own (one stage less of prefetch
+        // distance: the operands of a tall tile are L2 hits), runs its first K step on operands read during the block
+        // before, reads the second K step's under those MFMAs and the next block's first under the second's.  Reads
+        // and MFMAs are placed one by one (sched_barrier): an MFMA that waits for the matrix pipe holds up whatever
+        // is queued behind it in the wavefront.
+        v4i fa[2][2], fb[2][NBLK];  // [register set][tile] / [register set][token block]
+        auto read_operands = [&](int set, int uw, int ux, int s, int part) {
+            const int8_t* wbase = lds + uw * A_BYTES;
+            const int8_t* xbase = lds + ux * X_BYTES;
+            if (part == 0) {
+                fa[set][0] = *(const v4i*)(wbase + a_off + s * 1024);
+                fa[set][1] = *(const v4i*)(wbase + a_off + 2048 + s * 1024);
+                fb[set][0] = *(const v4i*)(xbase + (s ? frag_s1 : frag_s0));
+            } else {
+                fb[set][part] = *(const v4i*)(xbase + (s ? frag_s1 : frag_s0) + part * 2048);
+            }
+        };
+        // the stage of K block 0 has landed (for everybody): its first operands
+        auto wait_stage = [&]() {
+            // the younger request of the stage waited for is its tokens; behind them: the weights of that step and
+            // every request of the later steps
+            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
+            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
+            else wait_vmcnt<NAFTER + NA * (SX - 2)>();
+        };
+        auto wait_next_stage = [&]() {
+            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 3)>();
+            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 3)>();
+            else wait_vmcnt<NAFTER + NA * (SX - 3)>();
+        };
+        static_assert(SX >= 4, "a block reads the stage after its own: three stages in flight plus the one overwritten");
+        wait_stage();
+        __builtin_amdgcn_s_barrier();
+        if (active) {
+#pragma unroll
+            for (int part = 0; part < NBLK; ++part) read_operands(0, 0, 0, 0, part);
+        }
+        auto step = [&](int uw, int ux, int it) {
+            wait_next_stage();  // stage it + 1 has landed
+            __builtin_amdgcn_s_barrier();
+            load_tokens(it + SX - 1, (ux + SX - 1) % SX);
+            load_weights(it + SW - 1, (uw + SW - 1) % SW);
+            if (active) {
+                // K step 0 on set 0, reading K step 1 into set 1
+#pragma unroll
+                for (int b = 0; b < NBLK; ++b) {
+                    acc[0][b] = mfma_i8(fa[0][0], fb[0][b], acc[0][b]);
+                    acc[1][b] = mfma_i8(fa[0][1], fb[0][b], acc[1][b]);
+                    read_operands(1, uw, ux, 1, b);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // K step 1 on set 1, reading the next block's K step 0 into set 0
+#pragma unroll
+                for (int b = 0; b < NBLK; ++b) {
+                    acc[0][b] = mfma_i8(fa[1][0], fb[1][b], acc[0][b]);
+                    acc[1][b] = mfma_i8(fa[1][1], fb[1][b], acc[1][b]);
+                    read_operands(0, (uw + 1) % SW, (ux + 1) % SX, 0, b);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
+#pragma unroll
+            for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
+        }
+#pragma unroll
+        for (int u = 0; u + 1 < CYCLE; ++u)
+            if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
     }
-#pragma unroll
-    for (int u = 0; u + 1 < CYCLE; ++u)
-        if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
 
     wait_vmcnt<0>();  // the redirected loads past the end still write LDS
     __builtin_amdgcn_s_barrier();
@@ -731,13 +809,14 @@ static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipE
     tm.expert = (int32_t*)((char*)workspace + 256);
     tm.row_begin = (int32_t*)((char*)workspace + 256 + arr);
     tm.row_end = (int32_t*)((char*)workspace + 256 + 2 * arr);
-    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm);
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm, 0, a.rows_min,
+                       a.rows_max);
     const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
     const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
     const int n_col_blocks = (channels + per_block - 1) / per_block;
     const int total = max_tiles * n_col_blocks;
     const int grid = ((total + 7) / 8) * 8;
-    if (ev0 && ev1)
+    if (ev0 || ev1)
         hipExtLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT, RING>), dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm,
                               max_tiles, n_col_blocks);
     else
@@ -760,13 +839,14 @@ static void launch_wide(const GmmArgs& a, void* workspace, hipStream_t st, hipEv
     tm.expert = (int32_t*)((char*)workspace + 256);
     tm.row_begin = (int32_t*)((char*)workspace + 256 + arr);
     tm.row_end = (int32_t*)((char*)workspace + 256 + 2 * arr);
-    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm, 1);
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(256), 0, st, a.gl, a.gl_type, a.E, BM, max_tiles, tm, 1, a.rows_min,
+                       a.rows_max);
     const int channels = (EPI == EPI_SWIGLU) ? a.N / 2 : a.N;
     const int per_block = (EPI == EPI_SWIGLU) ? kBN / 2 : kBN;
     const int n_col_blocks = (channels + per_block - 1) / per_block;
     const int columns = (n_col_blocks + 1) / 2;
     const int grid = 8 * ((max_tiles + 7) / 8) * columns;  // one workgroup per (tile, column), no idle ones
-    if (ev0 && ev1)
+    if (ev0 || ev1)
         hipExtLaunchKernelGGL((gmm_wide_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, ev0, ev1, 0, a, tm,
                               max_tiles, n_col_blocks, columns);
     else
@@ -797,7 +877,7 @@ static void launch_dense_t(const GmmArgs& a, hipStream_t st, hipEvent_t ev0, hip
     }
     const int pm = (row_tiles + 8 / xn - 1) / (8 / xn), pn = (n_col_blocks + xn - 1) / xn;
     const int grid = 8 * pm * pn;
-    if (ev0 && ev1)
+    if (ev0 || ev1)
         hipExtLaunchKernelGGL((gmm_dense_kernel<EPI>), dim3(grid), dim3(512), lds_bytes, st, ev0, ev1, 0, a, xn, pm, pn,
                               n_col_blocks);
     else

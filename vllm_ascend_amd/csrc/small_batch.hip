@@ -103,13 +103,20 @@ __global__ __launch_bounds__(kSmallThreads) void route_quant_small_kernel(SmallR
                                a.eps, a.topk_weights, a.x_dtype, a.topk_ids, lds + (size_t)wave * E, nullptr, lane);
     }
     if (!a.arrived) return;  // gating and quantisation only (moe355_gate_quant): the maps come from another launch
-    // this workgroup's ids have reached memory before it is counted
+    // This workgroup's ids have reached memory before it is counted: every thread waits for its own stores, the
+    // barrier collects the workgroup, and the counting thread issues a device-scope release fence in front of the
+    // atomic (the ids are written with device-scope stores already; the fence is what the memory model asks for,
+    // so that the hand-off does not rest on how those stores happen to be compiled).
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     int32_t* flag = (int32_t*)lds;
-    if (tid == 0) *flag = atomicAdd(a.arrived, 1) == gate_wgs - 1;
+    if (tid == 0) {
+        __threadfence();
+        *flag = atomicAdd(a.arrived, 1) == gate_wgs - 1;
+    }
     __syncthreads();
     if (!*flag) return;
+    __threadfence();  // acquire side: the reads below come after the count that this workgroup has observed
     __syncthreads();
     // ---------------- the last gating workgroup sorts the R pairs (stable counting sort by expert)
     int32_t* ids_l = (int32_t*)lds;             // [kSmallMaxPairs]

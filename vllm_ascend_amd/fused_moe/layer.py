@@ -124,7 +124,10 @@ class AscendRoutedExperts(torch.nn.Module):
         topk_weights, topk_ids = self.router.select_experts(
             hidden_states, router_logits, enable_force_load_balance=self.enable_force_load_balance,
             weights_dtype=weights_dtype)
-        if self.log2phy is not None:
+        # The reference maps the router's ids through log2phy first and then, in a profile run, replaces them by
+        # random ids in [0, num_logical_experts) that are not mapped again (routed_experts.py:452-492).  The
+        # router here draws those random ids itself, so with forced load balance the map is skipped.
+        if self.log2phy is not None and not self.enable_force_load_balance:
             topk_ids = self.log2phy[topk_ids.long()].to(topk_ids.dtype)
         return self.quant_method.apply(self, hidden_states, topk_weights, topk_ids, self.shared_experts, None)
 

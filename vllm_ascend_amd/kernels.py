@@ -419,6 +419,9 @@ def token_unpermute(permuted, sorted_indices, probs, residual=None):
         T, k = sorted_indices.numel(), 1
     if residual is not None:
         residual = _dev(residual, "residual")
+        if residual.dtype != permuted.dtype or tuple(residual.shape) != (T, H):
+            raise ValueError(f"residual must be {permuted.dtype} of shape {(T, H)}, got {residual.dtype} "
+                             f"{tuple(residual.shape)}")
     out = torch.empty((T, H), dtype=permuted.dtype, device=permuted.device)
     check(lib.moe355_token_unpermute(_ptr(permuted), _dt(permuted, "permuted_tokens"), _ptr(sorted_indices),
                                      _ptr(probs), T, k, H, R, _ptr(residual), _ptr(out), _stream(permuted)),

@@ -111,7 +111,7 @@ class AscendW4A8DynamicFusedMoEMethod(AscendMoEScheme):
         """16-bit hidden states as a [T, H] matrix, none of the optional inputs of ``apply``, SiLU."""
         if self.use_expert_weight_list or not x.is_cuda or x.dim() != 2 or x.shape[0] == 0:
             return False
-        if x.dtype not in (torch.bfloat16, torch.float16):
+        if x.dtype not in (torch.bfloat16, torch.float16) or x.dtype != self.in_dtype:
             return False
         if (getattr(layer, "apply_router_weight_on_input", False) or getattr(layer, "ascend_pertoken_scale", None)
                 is not None or getattr(layer, "ascend_expert_map", None) is not None
