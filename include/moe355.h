@@ -294,6 +294,22 @@ int moe355_gmm1_swiglu_quant_w4(const int8_t *x, const uint8_t *weight_nz4, cons
 int moe355_w4_offset_correction(const uint8_t *weight_nz4, const float *weight_scale, int64_t group_size,
                                 int num_experts, int64_t n, int64_t k, float *corr, void *stream);
 
+/* Activations other than SiLU between the two grouped GEMMs.  Stands in for the unfused branch of
+ * quant_apply_mlp (vllm_ascend/ops/fused_moe/moe_mlp.py:484-549): the gate_up product is dequantised to the hidden
+ * dtype (moe355_gmm2_dequant with the gate_up weights), then this call applies the activation and the dynamic
+ * quantiser (torch_npu.npu_dynamic_quant) in one pass:
+ *   MOE355_ACT_GELU / _GELU_TANH  gelu(gate) * up                                  (moe_mlp.py:516-520)
+ *   MOE355_ACT_SWIGLUSTEP         min(silu(gate), L) * clamp(up, -L, L), L = limit > 0   (moe_mlp.py:512-515)
+ *   MOE355_ACT_SWIGLUOAI          g = min(gate, L), u = clamp(up, -L, L) (L = limit, 0: no clamp):
+ *                                 g * sigmoid(alpha * g) * (u + beta)                (moe_mlp.py:123-137, 521-538)
+ * evaluated in fp32 on the 16-bit inputs, rounded once to the 16-bit dtype, then scale = absmax / 127,
+ * q = rint(v / scale).  h [rows, n] bf16 / fp16 (gate = first n/2 columns); q [rows, n/2] int8; scale [rows].
+ * group_list (optional): rows at or beyond its total are left untouched. */
+enum { MOE355_ACT_GELU = 1, MOE355_ACT_GELU_TANH = 2, MOE355_ACT_SWIGLUSTEP = 3, MOE355_ACT_SWIGLUOAI = 4 };
+int moe355_act_mul_quant(const void *h, int h_dtype, const int64_t *group_list, int group_list_type, int num_experts,
+                         int64_t rows, int64_t n, int activation, float limit, float alpha, float beta, int8_t *q,
+                         float *scale, void *stream);
+
 /* The gate function of the SwiGLU epilogues by itself: out[i] = g[i] / (1 + exp(-g[i])) in fp32, n values.
  * form 0: the instruction sequence every kernel of this library runs (a division specialised to a divisor in
  * [1, 2^128)); form 1: the same function with the general IEEE division, which is the definition
@@ -364,6 +380,16 @@ int moe355_gmm_i32(const int8_t *x, const int8_t *weight_nz, const int64_t *grou
 int moe355_dequant_swiglu_quant(const int32_t *x, const float *weight_scale, const float *activation_scale,
                                 int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t *y,
                                 float *scale, void *stream);
+
+/* The same op with quant_mode = 0 (static; csrc/moe/dequant_swiglu_quant/op_kernel/
+ * dequant_swiglu_quant_static_base.hpp:266-305): after the SwiGLU,
+ *   quant_scale_len == n/2:  q = rint(y / quant_scale[col] + quant_offset[col])
+ *   quant_scale_len == 1:    q = rint(y * (1 / quant_scale[0]) + quant_offset[0])
+ * saturated to int8; quant_offset may be NULL (0).  No scale is written. */
+int moe355_dequant_swiglu_quant_static(const int32_t *x, const float *weight_scale, const float *activation_scale,
+                                       const float *quant_scale, int64_t quant_scale_len, const float *quant_offset,
+                                       int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t *y,
+                                       void *stream);
 
 /* ---------------------------------------------------------------------------
  * Weighted un-permute (finalize routing).

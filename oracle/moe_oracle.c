@@ -45,6 +45,12 @@
  *   orc_dequant_swiglu_quant : numpy rendering of test_dequant_swiglu_quant.py:16-45, both
  *                         values of activate_left (the golden's own branch, and the identity
  *                         "swap the halves of x and of the weight scale")
+ *   orc_dequant_swiglu_quant_static : the dynamic mode's SwiGLU values (orc_swiglu_quant's y) pushed through
+ *                         numpy's y / scale + offset and rint, per-channel and per-tensor, with and without offset
+ *   orc_erff, orc_tanhf : math.erf within 5e-7, math.tanh within 3e-7 absolute on a dense grid, odd symmetry, the limits
+ *   orc_act_mul_quant   : float64 formulas of the four activations within 16-bit rounding, clamp closed forms,
+ *                         the quantiser of orc_dynamic_quant on the rounded values; which intermediate roundings
+ *                         the reference's closed kernels apply: PARITY UNPINNED
  *   shared expert (oracle.py: shared_expert_forward, composed of the functions above in the order of
  *                         vllm_ascend/ops/fused_moe/shared_experts.py:254-301): dense float64 MLP on the
  *                         dequantised weights within the quantisation noise, exact agreement with the
@@ -664,6 +670,128 @@ ORC_API int orc_dequant_swiglu_quant(const int32_t *x, const float *w_scale, con
     int rc = orc_swiglu_quant(f, rows, N, clamp_limit, q, qs, NULL);
     free(f);
     return rc;
+}
+
+/*
+ * The static quantisation mode of the same op (quant_mode 0; the mode string "static" of
+ * csrc/moe/dequant_swiglu_quant/op_host/dequant_swiglu_quant_def.cpp:95).  Restates
+ * csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant_static_base.hpp:266-305: after the SwiGLU,
+ *   one scale per output channel (n_quant == N/2):  v = y / quant_scale[c] + quant_offset[c]
+ *   one scale for the tensor     (n_quant == 1):    v = y * (1 / quant_scale[0]) + quant_offset[0]
+ *   q = rint(v), saturated to int8 [one rounding, fixed by build: the kernel goes fp32 -> int16 -> fp16 -> int8].
+ * quant_offset may be NULL (0).  No scale is returned.
+ */
+ORC_API int orc_dequant_swiglu_quant_static(const int32_t *x, const float *w_scale, const float *a_scale,
+                                            const float *quant_scale, int64_t n_quant, const float *quant_offset,
+                                            int64_t rows, int64_t N, int activate_left, float clamp_limit, int8_t *q)
+{
+    const int64_t I = N / 2;
+    const float inv0 = 1.0f / quant_scale[0];
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t i = 0; i < I; ++i) {
+            const int64_t gi = activate_left ? i : i + I, ui = activate_left ? i + I : i;
+            float g = ((float)x[r * N + gi] * w_scale[gi]) * a_scale[r];
+            float u = ((float)x[r * N + ui] * w_scale[ui]) * a_scale[r];
+            if (clamp_limit > 0.0f) {
+                g = g > clamp_limit ? clamp_limit : g;
+                u = u > clamp_limit ? clamp_limit : u;
+                u = u < -clamp_limit ? -clamp_limit : u;
+            }
+            float y = (g / (1.0f + orc_expf(-g))) * u;
+            float v;
+            if (n_quant == 1) v = y * inv0 + (quant_offset ? quant_offset[0] : 0.0f);
+            else v = y / quant_scale[i] + (quant_offset ? quant_offset[i] : 0.0f);
+            float t = rintf(v);
+            t = t > 127.0f ? 127.0f : t;
+            t = t < -128.0f ? -128.0f : t;
+            q[r * I + i] = (int8_t)t;
+        }
+    return 0;
+}
+
+/*
+ * Activations other than SiLU.  The reference runs them unfused: gate_up product dequantised to the hidden dtype,
+ * the activation on that 16-bit tensor, npu_dynamic_quant, down product
+ * (vllm_ascend/ops/fused_moe/moe_mlp.py:484-549):
+ *   gelu / gelu_tanh  F.gelu(gate, approximate=...) * up                                   (moe_mlp.py:516-520)
+ *   swiglustep        silu(gate).clamp(max=L) * up.clamp(-L, L), L = swiglu_limit or 7     (moe_mlp.py:512-515,
+ *                     vllm_ascend/ops/activation.py:63-86)
+ *   swigluoai         g = gate.clamp(max=L), u = up.clamp(-L, L): g * sigmoid(alpha * g) * (u + beta)
+ *                     (moe_mlp.py:123-137, 521-538)
+ * [fixed by build] the activation is evaluated in fp32 on the 16-bit inputs and rounded ONCE to the hidden dtype
+ * (torch would round after every operator; the reference's Triton / torch_npu kernels for these are closed or
+ * compute in fp32 too -- PARITY UNPINNED), with erf by Abramowitz & Stegun 7.1.26 and tanh(z) = 1 - 2 / (1 +
+ * exp(2 z)) on the shared exp; then the dynamic quantiser of orc_dynamic_quant on the rounded values.
+ * h [rows, N] in the hidden dtype (gate = first half); q [rows, N/2] int8; qs [rows].
+ */
+ORC_API float orc_erff(float x)
+{
+    const float ax = fabsf(x);
+    const float t = 1.0f / (1.0f + 0.3275911f * ax);
+    float p = 1.061405429f;
+    p = fmaf(p, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    const float y = 1.0f - (p * t) * orc_expf(-(ax * ax));
+    return copysignf(y, x);
+}
+
+ORC_API float orc_tanhf(float z) { return 1.0f - 2.0f / (1.0f + orc_expf(2.0f * z)); }
+
+enum { ORC_ACT_GELU = 1, ORC_ACT_GELU_TANH = 2, ORC_ACT_SWIGLUSTEP = 3, ORC_ACT_SWIGLUOAI = 4 };
+
+static inline float act_mul(float g, float u, int act, float limit, float alpha, float beta)
+{
+    if (act == ORC_ACT_GELU) return ((0.5f * g) * (1.0f + orc_erff(g * 0.70710678f))) * u;
+    if (act == ORC_ACT_GELU_TANH) {
+        const float inner = 0.7978845608f * (g + 0.044715f * ((g * g) * g));
+        return ((0.5f * g) * (1.0f + orc_tanhf(inner))) * u;
+    }
+    if (act == ORC_ACT_SWIGLUSTEP) {
+        float s = g / (1.0f + orc_expf(-g));
+        s = s > limit ? limit : s;
+        u = u > limit ? limit : u;
+        u = u < -limit ? -limit : u;
+        return s * u;
+    }
+    if (limit > 0.0f) {
+        g = g > limit ? limit : g;
+        u = u > limit ? limit : u;
+        u = u < -limit ? -limit : u;
+    }
+    return (g * (1.0f / (1.0f + orc_expf(-(alpha * g))))) * (u + beta);
+}
+
+ORC_API int orc_act_mul_quant(const uint16_t *h, int64_t rows, int64_t N, int act, float limit, float alpha,
+                              float beta, int8_t *q, float *qs)
+{
+    if (act < ORC_ACT_GELU || act > ORC_ACT_SWIGLUOAI) return -1;
+    const int64_t I = N / 2;
+#pragma omp parallel
+    {
+        float *y = (float *)malloc(sizeof(float) * (size_t)I);
+#pragma omp for
+        for (int64_t r = 0; r < rows; ++r) {
+            float a = 0.0f;
+            for (int64_t i = 0; i < I; ++i) {
+                const float v = h2f(f2h(act_mul(h2f(h[r * N + i]), h2f(h[r * N + I + i]), act, limit, alpha, beta)));
+                y[i] = v;
+                const float b = fabsf(v);
+                a = b > a ? b : a;
+            }
+            const float s = a / 127.0f;
+            qs[r] = a == 0.0f ? 0.0f : s;
+            for (int64_t i = 0; i < I; ++i) {
+                float t = a == 0.0f ? 0.0f : rintf(y[i] / s);
+                t = t > 127.0f ? 127.0f : t;
+                t = t < -128.0f ? -128.0f : t;
+                q[r * I + i] = (int8_t)t;
+            }
+        }
+        free(y);
+    }
+    return 0;
 }
 
 /*

@@ -336,6 +336,48 @@ def dequant_swiglu_quant(x_i32, w_scale, a_scale, activate_left=True, clamp_limi
     return q, qs
 
 
+def dequant_swiglu_quant_static(x_i32, w_scale, a_scale, quant_scale, quant_offset=None, activate_left=True,
+                                clamp_limit=0.0):
+    x = np.ascontiguousarray(x_i32, dtype=np.int32)
+    rows, N = x.shape
+    ws = np.ascontiguousarray(w_scale, dtype=np.float32)
+    as_ = np.ascontiguousarray(a_scale, dtype=np.float32).reshape(-1)
+    qsc = np.ascontiguousarray(quant_scale, dtype=np.float32).reshape(-1)
+    qof = None if quant_offset is None else np.ascontiguousarray(quant_offset, dtype=np.float32).reshape(-1)
+    q = np.zeros((rows, N // 2), dtype=np.int8)
+    lib().orc_dequant_swiglu_quant_static(_p(x), _p(ws), _p(as_), _p(qsc), _i64(qsc.size), _p(qof), _i64(rows), _i64(N),
+                                          _i32(int(activate_left)), _f32(clamp_limit), _p(q))
+    return q
+
+
+ACTIVATIONS = {"gelu": 1, "gelu_tanh": 2, "swiglustep": 3, "swigluoai": 4}
+
+
+def erff(x):
+    f = lib().orc_erff
+    f.restype, f.argtypes = ctypes.c_float, [ctypes.c_float]
+    return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).reshape(-1)], dtype=np.float32)
+
+
+def tanhf(x):
+    f = lib().orc_tanhf
+    f.restype, f.argtypes = ctypes.c_float, [ctypes.c_float]
+    return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).reshape(-1)], dtype=np.float32)
+
+
+def act_mul_quant(h_bits, activation: str, limit=0.0, alpha=1.0, beta=0.0):
+    """h_bits [rows, 2I] 16-bit floats as uint16 (gate first) -> int8 [rows, I], fp32 scale [rows]."""
+    h = np.ascontiguousarray(h_bits, dtype=np.uint16)
+    rows, N = h.shape
+    q = np.zeros((rows, N // 2), dtype=np.int8)
+    qs = np.zeros((rows,), dtype=np.float32)
+    rc = lib().orc_act_mul_quant(_p(h), _i64(rows), _i64(N), _i32(ACTIVATIONS[activation]), _f32(limit), _f32(alpha),
+                                 _f32(beta), _p(q), _p(qs))
+    if rc != 0:
+        raise ValueError(f"orc_act_mul_quant rejected the arguments (rc={rc})")
+    return q, qs
+
+
 def cumsum_group_list(group_list: np.ndarray, src_list_type: int, dst_list_type: int) -> np.ndarray:
     """count <-> cumulative conversion; restates vllm_ascend/ops/fused_moe/moe_mlp.py:54-83 (types 0 and 1)."""
     if src_list_type not in (0, 1, 2):
@@ -369,16 +411,24 @@ class LayerTrace:
     extra: dict = field(default_factory=dict)
 
 
-def experts_forward(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2, *, keep_acc=True, add_bf16=None) -> LayerTrace:
+def experts_forward(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2, *, keep_acc=True, add_bf16=None,
+                    activation="silu", swiglu_limit=0.0, swiglu_alpha=1.0, swiglu_beta=0.0) -> LayerTrace:
     """dispatch -> gate_up GEMM + SwiGLU/re-quant -> down GEMM + dequant -> combine.
-    Stage order restates vllm_ascend/ops/fused_moe/moe_comm_method.py:117-162."""
+    Stage order restates vllm_ascend/ops/fused_moe/moe_comm_method.py:117-162.  An activation other than SiLU takes
+    the unfused form of vllm_ascend/ops/fused_moe/moe_mlp.py:484-549: gate_up product dequantised to 16 bits,
+    activation, dynamic quantisation."""
     E = w13.shape[0]
     tr = LayerTrace(topk_weights=topk_w_bf16, topk_ids=topk_ids)
     tr.xs, tr.expanded_row_idx, tr.expert_tokens, tr.sx = init_routing(x_bf16, topk_ids, E)
     cum = np.cumsum(tr.expert_tokens)
     acc1 = gmm_i32(tr.xs, w13, cum)
-    f = dequant_acc(acc1, tr.sx, s13, cum)
-    tr.q1, tr.s1 = swiglu_quant(f)
+    if activation == "silu":
+        f = dequant_acc(acc1, tr.sx, s13, cum)
+        tr.q1, tr.s1 = swiglu_quant(f, swiglu_limit)
+    else:
+        h = gmm2_dequant(acc1, tr.sx, s13, cum)
+        limit = (swiglu_limit or 7.0) if activation == "swiglustep" else swiglu_limit
+        tr.q1, tr.s1 = act_mul_quant(h, activation, limit, swiglu_alpha, swiglu_beta)
     acc2 = gmm_i32(tr.q1, w2, cum)
     tr.o = gmm2_dequant(acc2, tr.s1, s2, cum)
     tr.out = unpermute(tr.o, tr.expanded_row_idx, topk_w_bf16, add_bf16)

@@ -180,8 +180,10 @@ def test_unsupported_options_raise_by_name():
         disp.token_dispatch(inp)
     from vllm_ascend_amd.fused_moe.moe_mlp import quant_apply_mlp
 
-    with pytest.raises(NotImplementedError, match="gelu"):
-        quant_apply_mlp(torch.zeros(1, 8), None, None, None, None, torch.zeros(1), activation="gelu")
+    with pytest.raises(NotImplementedError, match="relu2"):
+        quant_apply_mlp(torch.zeros(1, 8), None, None, None, None, torch.zeros(1), activation="relu2")
+    with pytest.raises(NotImplementedError, match="swigluoai"):
+        quant_apply_mlp(torch.zeros(1, 8), None, None, None, None, torch.zeros(1), activation="gelu", swiglu_alpha=1.7)
 
 
 def test_bench_refuses_more_than_one_gpu():

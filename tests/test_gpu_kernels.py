@@ -491,6 +491,54 @@ def test_dequant_swiglu_quant(K, orc, rows, n, left):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,n", [(3, 192), (8, 384), (2, 8448)])
+@pytest.mark.parametrize("left", [True, False])
+def test_dequant_swiglu_quant_static_mode(K, orc, rows, n, left):
+    """quant_mode 0 through the operator (torch.ops._C_ascend.npu_dequant_swiglu_quant) and the launcher."""
+    from vllm_ascend_amd import custom_ops
+
+    custom_ops.enable_custom_op()
+    g = torch.Generator().manual_seed(rows * 31 + n)
+    x = torch.randint(-100, 100, (rows, n), generator=g, dtype=torch.int32)
+    ws = torch.randn(n, generator=g) * 0.1
+    as_ = torch.randn(rows, generator=g) * 0.5
+    qs = torch.rand(n // 2, generator=g) * 0.05 + 0.01
+    qo = torch.randn(n // 2, generator=g) * 3
+    for scale, off in ((qs, qo), (qs, None), (qs[:1], qo[:1]), (qs[:1], None)):
+        want = orc.dequant_swiglu_quant_static(x.numpy(), ws.numpy(), as_.numpy(), scale.numpy(),
+                                               None if off is None else off.numpy(), activate_left=left)
+        got, sc = torch.ops._C_ascend.npu_dequant_swiglu_quant(
+            x.to(DEV), weight_scale=ws.to(DEV), activation_scale=as_.to(DEV).reshape(rows, 1),
+            quant_scale=scale.to(DEV), quant_offset=None if off is None else off.to(DEV), activate_left=left,
+            quant_mode=0, swiglu_mode=1)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), want)
+        assert sc.shape == (rows,)
+
+
+@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "swiglustep", "swigluoai"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_act_mul_quant(K, orc, act, dtype):
+    limit, alpha, beta = (7.0, 1.0, 0.0) if act == "swiglustep" else ((3.0, 1.702, 1.0) if act == "swigluoai" else (0.0, 1.0, 0.0))
+    g = torch.Generator().manual_seed(17)
+    for rows, n in ((5, 192), (33, 1536), (2, 8320)):
+        h = (torch.randn(rows, n, generator=g) * 4).to(dtype)
+        h[0, :4] = torch.tensor([0.0, -0.0, 100.0, -100.0]).to(dtype)
+        with orc.half_kind("bf16" if dtype == torch.bfloat16 else "f16"):
+            q_want, s_want = orc.act_mul_quant(bits(h), act, limit, alpha, beta)
+        # rows beyond the group list's total stay untouched
+        cnt = torch.tensor([rows - 1, 0], dtype=torch.int64)
+        q, s_ = K.act_mul_quant(h.to(DEV), act, limit, alpha, beta)
+        torch.cuda.synchronize()
+        assert np.array_equal(q.cpu().numpy(), q_want), (act, rows, n)
+        assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+        for gl, gl_type in ((cnt, 1), (torch.cumsum(cnt, 0), 0)):
+            q2, s2 = K.act_mul_quant(h.to(DEV), act, limit, alpha, beta, gl.to(DEV), gl_type)
+            torch.cuda.synchronize()
+            assert np.array_equal(q2[: rows - 1].cpu().numpy(), q_want[: rows - 1])
+            assert np.array_equal(s2[: rows - 1].cpu().numpy().view(np.uint32), s_want[: rows - 1].view(np.uint32))
+
+
 def test_grouped_matmul_swiglu_quant_v2_against_the_reference_golden(orc):
     """A8W4 operator with per-group scales and an arbitrary assist matrix, against a numpy rendering of
     gmm_swiglu_quant_golden_a8_w4 (tests/e2e/nightly/single_node/ops/singlecard_ops/

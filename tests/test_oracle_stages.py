@@ -489,3 +489,125 @@ def test_w4_layer_matches_a_dense_float64_rendering():
             o[lo:hi] = (part * sg2[e][:, None, :]).sum(axis=0) * tr.s1[lo:hi, None].astype(np.float64)
         lo = hi
     assert rel_err(orc.bf16_to_f32(tr.o), o) <= 1e-2
+
+
+# ------------------------------------------------------------------ static quantisation mode, other activations
+def test_dequant_swiglu_quant_static_against_numpy():
+    """quant_mode 0 (dequant_swiglu_quant_static_base.hpp:266-305): y / scale[c] + offset[c] per channel,
+    y * (1 / scale) + offset per tensor, one rounding, saturation."""
+    rng = np.random.RandomState(3)
+    rows, N = 6, 192
+    x = rng.randint(-100, 100, size=(rows, N)).astype(np.int32)
+    ws = (rng.randn(N) * 0.1).astype(np.float32)
+    as_ = (rng.randn(rows) * 0.5).astype(np.float32)
+    # the SwiGLU values of the dynamic mode are the ones that get quantised
+    f = (x.astype(np.float32) * ws[None, :]) * as_[:, None]
+    _, _, y = orc.swiglu_quant(f, want_y=True)
+    qs = (rng.rand(N // 2) * 0.05 + 0.01).astype(np.float32)
+    qo = (rng.randn(N // 2) * 3).astype(np.float32)
+    for scale, off in ((qs, qo), (qs, None), (qs[:1], qo[:1]), (qs[:1], None)):
+        got = orc.dequant_swiglu_quant_static(x, ws, as_, scale, off)
+        o = np.float32(0) if off is None else off
+        if scale.size == 1:
+            v = y * (np.float32(1.0) / scale[0]) + (o if off is None else o[0])
+        else:
+            v = y / scale[None, :] + (o if off is None else o[None, :])
+        want = np.clip(np.rint(v.astype(np.float32)), -128, 127).astype(np.int8)
+        assert np.array_equal(got, want)
+    # saturation both ways
+    big = orc.dequant_swiglu_quant_static(x, ws, as_, np.array([1e-6], dtype=np.float32))
+    assert big.max() == 127 and big.min() == -128
+    # activate_left = False: the halves swap roles
+    swapped = np.concatenate([x[:, N // 2:], x[:, :N // 2]], axis=1)
+    ws_sw = np.concatenate([ws[N // 2:], ws[:N // 2]])
+    assert np.array_equal(orc.dequant_swiglu_quant_static(swapped, ws_sw, as_, qs, qo, activate_left=False),
+                          orc.dequant_swiglu_quant_static(x, ws, as_, qs, qo))
+
+
+def test_erf_and_tanh_against_libm():
+    import math
+
+    xs = np.linspace(-6.0, 6.0, 4801).astype(np.float32)
+    e = orc.erff(xs).astype(np.float64)
+    t = orc.tanhf(xs).astype(np.float64)
+    assert np.max(np.abs(e - np.array([math.erf(float(v)) for v in xs]))) <= 5e-7
+    assert np.max(np.abs(t - np.tanh(xs.astype(np.float64)))) <= 3e-7
+    assert np.array_equal(orc.erff(-xs), -orc.erff(xs))          # odd by construction (copysign)
+    assert orc.erff(np.array([0.0, 10.0, -10.0], dtype=np.float32)).tolist() == [0.0, 1.0, -1.0]
+    assert orc.tanhf(np.array([50.0, -50.0], dtype=np.float32)).tolist() == [1.0, -1.0]
+
+
+@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "swiglustep", "swigluoai"])
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+def test_activation_and_quantisation_against_float64(act, kind):
+    """The unfused activations (moe_mlp.py:484-549) against their float64 formulas: values within the rounding of
+    the 16-bit result, then exactly the dynamic quantiser's rule on those rounded values."""
+    import math
+
+    rng = np.random.RandomState(11)
+    rows, I = 5, 96
+    limit, alpha, beta = (7.0, 1.0, 0.0) if act == "swiglustep" else ((3.0, 1.702, 1.0) if act == "swigluoai" else (0.0, 1.0, 0.0))
+    with orc.half_kind(kind):
+        h = orc.f32_to_half((rng.randn(rows, 2 * I) * 4).astype(np.float32))
+        hf = orc.half_to_f32(h).astype(np.float64)
+        q, s = orc.act_mul_quant(h, act, limit, alpha, beta)
+        g, u = hf[:, :I], hf[:, I:]
+        if act == "gelu":
+            y = 0.5 * g * (1 + np.vectorize(math.erf)(g / math.sqrt(2))) * u
+        elif act == "gelu_tanh":
+            y = 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3))) * u
+        elif act == "swiglustep":
+            y = np.minimum(g / (1 + np.exp(-g)), limit) * np.clip(u, -limit, limit)
+        else:
+            gc, uc = np.minimum(g, limit), np.clip(u, -limit, limit)
+            y = gc / (1 + np.exp(-alpha * gc)) * (uc + beta)
+        y16 = orc.half_to_f32(orc.f32_to_half(y.astype(np.float32))).astype(np.float64)
+        # rebuild what the checker quantised: q * s must be within half a step of a 16-bit value near y
+        amax = np.abs(y16).max(axis=1)
+        assert np.allclose(s, amax / 127.0, rtol=2e-2)  # the row maximum may round to a neighbouring 16-bit value
+        ulp16 = 2.0 ** (-7 if kind == "bf16" else -10)
+        assert np.all(np.abs(q.astype(np.float64) * s[:, None] - y) <= 0.5 * s[:, None] + np.abs(y) * ulp16 + 2e-6)
+        assert np.abs(q).max(axis=1).tolist() == [127] * rows
+    # an all-zero row: zeros and a zero scale
+    with orc.half_kind(kind):
+        qz, sz = orc.act_mul_quant(np.zeros((1, 8), dtype=np.uint16), act, limit, alpha, beta)
+        assert not qz.any() and sz[0] == 0.0
+
+
+def test_layer_with_other_activations_matches_a_dense_float64_rendering():
+    """experts_forward(activation=...) end to end against the dense float64 layer with that activation, within the
+    quantisation noise (the same bound as the SiLU layer)."""
+    import math
+
+    from _inputs import CONFIGS, bits, make_layer
+
+    cfg = CONFIGS["c2_small"]
+    d = make_layer(cfg, seed=0)
+    y, ids, _ = orc.gating_top_k(d["logits"].numpy(), cfg.k, renorm=1, norm_type=0, x_dtype="f32")
+    w = orc.f32_to_half(y)
+    for act in ("gelu", "gelu_tanh", "swiglustep", "swigluoai"):
+        limit, alpha, beta = (7.0, 1.0, 0.0) if act == "swiglustep" else ((7.0, 1.702, 1.0) if act == "swigluoai" else (0.0, 1.0, 0.0))
+        tr = orc.experts_forward(bits(d["x"]), w, ids, d["w13"].numpy(), d["s13"].numpy(), d["w2"].numpy(),
+                                 d["s2"].numpy(), activation=act, swiglu_limit=limit, swiglu_alpha=alpha,
+                                 swiglu_beta=beta)
+        x = orc.half_to_f32(bits(d["x"])).astype(np.float64)
+        wf = orc.half_to_f32(w).astype(np.float64)
+        ref = np.zeros((cfg.T, cfg.H))
+        for e in np.unique(ids):
+            tok, slot = np.nonzero(ids == e)
+            gu = x[tok] @ (d["w13"][e].numpy().astype(np.float64) * d["s13"][e].numpy().astype(np.float64)[:, None]).T
+            g, u = gu[:, :cfg.I], gu[:, cfg.I:]
+            if act == "gelu":
+                a = 0.5 * g * (1 + np.vectorize(math.erf)(g / math.sqrt(2))) * u
+            elif act == "gelu_tanh":
+                a = 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3))) * u
+            elif act == "swiglustep":
+                a = np.minimum(g / (1 + np.exp(-g)), limit) * np.clip(u, -limit, limit)
+            else:
+                gc, uc = np.minimum(g, limit), np.clip(u, -limit, limit)
+                a = gc / (1 + np.exp(-alpha * gc)) * (uc + beta)
+            o = a @ (d["w2"][e].numpy().astype(np.float64) * d["s2"][e].numpy().astype(np.float64)[:, None]).T
+            np.add.at(ref, tok, o * wf[tok, slot][:, None])
+        got = orc.half_to_f32(tr.out).astype(np.float64)
+        err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+        assert err <= 5e-2, (act, err)

@@ -77,6 +77,10 @@ PROTOTYPES = {
                                c_void_p, c_size_t, c_void_p]),
     "moe355_dequant_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p,
                                             c_void_p, c_void_p]),
+    "moe355_dequant_swiglu_quant_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+                                                   c_int64, c_int, c_float, c_void_p, c_void_p]),
+    "moe355_act_mul_quant": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int64, c_int64, c_int, c_float,
+                                     c_float, c_float, c_void_p, c_void_p, c_void_p]),
     "moe355_silu_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "moe355_profile_next_gemm": (c_int, [c_void_p, c_void_p]),
     "moe355_gmm_kernel_name": (c_char_p, [c_int, c_int64, c_int64, c_int64, c_int]),

@@ -165,6 +165,113 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
     }
 }
 
+// Static quantisation mode of the op above: q = rint(y / quant_scale[c] + quant_offset[c]) (one scale per output
+// channel) or rint(y * (1 / quant_scale[0]) + quant_offset[0]) (one scale), saturated; no scale output.
+__global__ __launch_bounds__(256) void dequant_swiglu_quant_static_kernel(
+    const int32_t* __restrict__ x, const float* __restrict__ w_scale, const float* __restrict__ a_scale,
+    const float* __restrict__ q_scale, int per_channel, const float* __restrict__ q_offset, int64_t n,
+    int activate_left, float limit, int8_t* __restrict__ y)
+{
+    const int64_t row = blockIdx.x;
+    const int64_t half = n >> 1;
+    const int32_t* xr = x + row * n;
+    const float as = a_scale[row];
+    const int64_t goff = activate_left ? 0 : half;
+    const int64_t uoff = activate_left ? half : 0;
+    const float inv0 = 1.0f / q_scale[0];
+    for (int64_t i = threadIdx.x; i < half; i += 256) {
+        float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
+        float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
+        if (limit > 0.0f) {
+            g = g > limit ? limit : g;
+            u = u > limit ? limit : u;
+            u = u < -limit ? -limit : u;
+        }
+        const float v = m_silu(g) * u;
+        float t;
+        if (per_channel) t = v / q_scale[i] + (q_offset ? q_offset[i] : 0.0f);
+        else t = v * inv0 + (q_offset ? q_offset[0] : 0.0f);
+        y[row * half + i] = sat_rint_i8(t);
+    }
+}
+
+// erf by Abramowitz & Stegun 7.1.26 on the shared exp (absolute error below 5e-7 in fp32); the CPU checker runs the
+// same operation sequence.
+__device__ __forceinline__ float m_erff(float x)
+{
+    const float ax = __builtin_fabsf(x);
+    const float t = 1.0f / (1.0f + 0.3275911f * ax);
+    float p = 1.061405429f;
+    p = __builtin_fmaf(p, t, -1.453152027f);
+    p = __builtin_fmaf(p, t, 1.421413741f);
+    p = __builtin_fmaf(p, t, -0.284496736f);
+    p = __builtin_fmaf(p, t, 0.254829592f);
+    const float y = 1.0f - (p * t) * m_expf(-(ax * ax));
+    return __builtin_copysignf(y, x);
+}
+
+__device__ __forceinline__ float m_tanhf(float z) { return 1.0f - 2.0f / (1.0f + m_expf(2.0f * z)); }
+
+enum { ACT_GELU = 1, ACT_GELU_TANH = 2, ACT_SWIGLUSTEP = 3, ACT_SWIGLUOAI = 4 };
+
+template <int ACT>
+__device__ __forceinline__ float act_mul(float g, float u, float limit, float alpha, float beta)
+{
+    if constexpr (ACT == ACT_GELU) {
+        return ((0.5f * g) * (1.0f + m_erff(g * 0.70710678f))) * u;
+    } else if constexpr (ACT == ACT_GELU_TANH) {
+        const float inner = 0.7978845608f * (g + 0.044715f * ((g * g) * g));
+        return ((0.5f * g) * (1.0f + m_tanhf(inner))) * u;
+    } else if constexpr (ACT == ACT_SWIGLUSTEP) {
+        float sg = m_silu(g);
+        sg = sg > limit ? limit : sg;
+        u = u > limit ? limit : u;
+        u = u < -limit ? -limit : u;
+        return sg * u;
+    } else {
+        if (limit > 0.0f) {
+            g = g > limit ? limit : g;
+            u = u > limit ? limit : u;
+            u = u < -limit ? -limit : u;
+        }
+        return (g * (1.0f / (1.0f + m_expf(-(alpha * g))))) * (u + beta);
+    }
+}
+
+// h [rows, n] 16-bit (gate = first half) -> activation(gate) * up in fp32, rounded once to the 16-bit dtype ->
+// per-row dynamic int8 (scale = absmax / 127, q = rint(v / scale)).  One workgroup per row; rows at or beyond the
+// last group (gl given) are left untouched.
+template <int ACT, int DT>
+__global__ __launch_bounds__(256) void act_mul_quant_kernel(const uint16_t* __restrict__ h,
+                                                            const int64_t* __restrict__ gl, int gl_type, int E,
+                                                            int64_t n, float limit, float alpha, float beta,
+                                                            int8_t* __restrict__ q, float* __restrict__ scale)
+{
+    __shared__ float lds4[4];
+    const int64_t row = blockIdx.x;
+    if (gl) {
+        int64_t r0, total;
+        expert_rows(gl, gl_type, E - 1, threadIdx.x & 63, r0, total);
+        if (row >= total) return;
+    }
+    const int64_t half = n >> 1;
+    const uint16_t* hr = h + row * n;
+    auto value = [&](int64_t i) {
+        const float v = act_mul<ACT>(half_to_f32<DT>(hr[i]), half_to_f32<DT>(hr[half + i]), limit, alpha, beta);
+        return half_to_f32<DT>(f32_to_half<DT>(v));
+    };
+    float a = 0.0f;
+    for (int64_t i = threadIdx.x; i < half; i += 256) {
+        const float v = __builtin_fabsf(value(i));
+        a = v > a ? v : a;
+    }
+    a = block_max_256(a, lds4);
+    const float s = a / 127.0f;
+    if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
+    for (int64_t i = threadIdx.x; i < half; i += 256)
+        q[row * half + i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(value(i) / s);
+}
+
 // out[i] = silu(g[i]) by the kernels' instruction sequence (form 0) or by the IEEE quotient (form 1)
 template <int FORM>
 __global__ __launch_bounds__(256) void silu_f32_kernel(const float* __restrict__ g, float* __restrict__ out,
@@ -240,5 +347,51 @@ extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight
     else if (half <= 16 * 256) MOE355_DSQ(16);
     else MOE355_DSQ(0);
 #undef MOE355_DSQ
+    return launch_status();
+}
+
+extern "C" int moe355_dequant_swiglu_quant_static(const int32_t* x, const float* weight_scale,
+                                                  const float* activation_scale, const float* quant_scale,
+                                                  int64_t quant_scale_len, const float* quant_offset, int64_t rows,
+                                                  int64_t n, int activate_left, float clamp_limit, int8_t* y,
+                                                  void* stream)
+{
+    if (rows < 0 || n <= 0 || (n & 1)) return MOE355_E_ARG;
+    if (quant_scale_len != 1 && quant_scale_len != n / 2) return MOE355_E_SHAPE;
+    if (rows == 0) return MOE355_OK;
+    if (!x || !weight_scale || !activation_scale || !quant_scale || !y) return MOE355_E_ARG;
+    if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
+    hipLaunchKernelGGL(dequant_swiglu_quant_static_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
+                       weight_scale, activation_scale, quant_scale, quant_scale_len != 1 ? 1 : 0,
+                       quant_offset, n, activate_left, clamp_limit, y);
+    return launch_status();
+}
+
+extern "C" int moe355_act_mul_quant(const void* h, int h_dtype, const int64_t* group_list, int group_list_type,
+                                    int num_experts, int64_t rows, int64_t n, int activation, float limit, float alpha,
+                                    float beta, int8_t* q, float* scale, void* stream)
+{
+    if (rows < 0 || n <= 0 || (n & 1)) return MOE355_E_ARG;
+    if (activation < ACT_GELU || activation > ACT_SWIGLUOAI) return MOE355_E_UNSUPPORTED;
+    if (h_dtype != MOE355_DT_BF16 && h_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
+    if (group_list && (num_experts <= 0 || (group_list_type != MOE355_GL_CUMSUM && group_list_type != MOE355_GL_COUNT)))
+        return MOE355_E_ARG;
+    if (activation == ACT_SWIGLUSTEP && !(limit > 0.0f)) return MOE355_E_ARG;
+    if (rows == 0) return MOE355_OK;
+    if (!h || !q || !scale) return MOE355_E_ARG;
+    if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+#define MOE355_AMQ(A_, D_)                                                                                     \
+    hipLaunchKernelGGL((act_mul_quant_kernel<A_, D_>), dim3((unsigned)rows), dim3(256), 0, st, (const uint16_t*)h, \
+                       group_list, group_list_type, num_experts, n, limit, alpha, beta, q, scale)
+#define MOE355_AMQ_D(A_)                                 \
+    if (h_dtype == MOE355_DT_BF16) MOE355_AMQ(A_, MOE355_DT_BF16); \
+    else MOE355_AMQ(A_, MOE355_DT_F16)
+    if (activation == ACT_GELU) { MOE355_AMQ_D(ACT_GELU); }
+    else if (activation == ACT_GELU_TANH) { MOE355_AMQ_D(ACT_GELU_TANH); }
+    else if (activation == ACT_SWIGLUSTEP) { MOE355_AMQ_D(ACT_SWIGLUSTEP); }
+    else { MOE355_AMQ_D(ACT_SWIGLUOAI); }
+#undef MOE355_AMQ_D
+#undef MOE355_AMQ
     return launch_status();
 }

@@ -50,10 +50,12 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
                     swiglu_alpha: float = 1.0, swiglu_beta: float = 0.0,
                     use_w4a8_per_channel_gmm_swiglu: bool = False, output_dtype=None, **unsupported):
     act_name = getattr(activation, "value", activation) or "silu"
-    if act_name != "silu":
-        raise NotImplementedError(f"activation {act_name!r}: only 'silu' (SwiGLU) has a fused MI355X kernel")
-    if swiglu_alpha != 1.0 or swiglu_beta != 0.0:
-        raise NotImplementedError("swiglu_alpha / swiglu_beta variants are not supported")
+    from ..kernels import ACTIVATIONS
+
+    if act_name != "silu" and act_name not in ACTIVATIONS:
+        raise NotImplementedError(f"activation {act_name!r}: supported are 'silu' and {sorted(ACTIVATIONS)}")
+    if act_name not in ("swigluoai", "swigluoai_uninterleave") and (swiglu_alpha != 1.0 or swiglu_beta != 0.0):
+        raise NotImplementedError("swiglu_alpha / swiglu_beta belong to the swigluoai activation")
     if w1_offset is not None or w2_offset is not None:
         raise NotImplementedError("asymmetric weight offsets are not supported")
     if unsupported.get("use_mxfp_quant"):
@@ -67,6 +69,30 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
     else:
         pertoken_scale = dynamic_scale
 
+    if act_name != "silu":
+        # No fused op for these: gate_up product dequantised to the hidden dtype, activation * up and the dynamic
+        # quantiser in one pass, down product (the unfused branch of the reference, moe_mlp.py:484-569).
+        from ..kernels import act_mul_quant
+
+        gate_up = DeviceOperator.npu_grouped_matmul_gmm2(
+            hidden_states=hidden_states, weight=w1 if isinstance(w1, (list, tuple)) and len(w1) > 1 else _single(w1, "w1"),
+            weight_scale=(w1_scale if isinstance(w1_scale, (list, tuple)) and len(w1_scale) > 1
+                          else _single(w1_scale, "w1_scale")),
+            per_token_scale=pertoken_scale, group_list=group_list, group_list_type=group_list_type,
+            input_dtype=input_dtype)
+        limit = (swiglu_limit or 7.0) if act_name == "swiglustep" else swiglu_limit
+        gl_ok = group_list_type in (0, 1)
+        hidden_states, swiglu_out_scale = act_mul_quant(
+            gate_up, act_name, limit, swiglu_alpha, swiglu_beta,
+            group_list if gl_ok else cumsum_group_list(group_list, group_list_type, 0), group_list_type if gl_ok else 0)
+        before_gmm2_evt = torch.cuda.current_stream().record_event() if hidden_states.is_cuda else None
+        out = DeviceOperator.npu_grouped_matmul_gmm2(
+            hidden_states=hidden_states, weight=w2 if isinstance(w2, (list, tuple)) and len(w2) > 1 else _single(w2, "w2"),
+            weight_scale=(w2_scale if isinstance(w2_scale, (list, tuple)) and len(w2_scale) > 1
+                          else _single(w2_scale, "w2_scale")),
+            per_token_scale=swiglu_out_scale, group_list=group_list, group_list_type=group_list_type,
+            input_dtype=input_dtype)
+        return out, before_gmm2_evt
     if dynamic_eplb or (isinstance(w1, (list, tuple)) and len(w1) > 1):
         # per-expert weight lists (the form dynamic expert load balancing swaps in place)
         from ..kernels import ExpertTensorList, gmm1_swiglu_quant_list

@@ -403,6 +403,49 @@ def dequant_swiglu_quant(x, weight_scale, activation_scale, activate_left=True, 
     return y, s
 
 
+def dequant_swiglu_quant_static(x, weight_scale, activation_scale, quant_scale, quant_offset=None,
+                                activate_left=True, clamp_limit=0.0):
+    """quant_mode 0 of npu_dequant_swiglu_quant: one scale (and offset) per output channel or per tensor."""
+    x = _dev(x, "x")
+    lib = _lib.load()
+    n = x.shape[-1]
+    rows = x.numel() // n if n else 0
+    quant_scale = _dev(quant_scale, "quant_scale").to(torch.float32).reshape(-1)
+    if quant_offset is not None:
+        quant_offset = _dev(quant_offset, "quant_offset").to(torch.float32).reshape(-1)
+        if quant_offset.numel() != quant_scale.numel():
+            raise ValueError("quant_offset must have as many elements as quant_scale")
+    y = torch.empty(x.shape[:-1] + (n // 2,), dtype=torch.int8, device=x.device)
+    check(lib.moe355_dequant_swiglu_quant_static(_ptr(x), _ptr(_dev(weight_scale, "weight_scale")),
+                                                 _ptr(_dev(activation_scale, "activation_scale")), _ptr(quant_scale),
+                                                 quant_scale.numel(), _ptr(quant_offset), rows, n,
+                                                 int(bool(activate_left)), float(clamp_limit), _ptr(y), _stream(x)),
+          "moe355_dequant_swiglu_quant_static")
+    return y
+
+
+ACTIVATIONS = {"gelu": 1, "gelu_tanh": 2, "swiglustep": 3, "swigluoai": 4, "swigluoai_uninterleave": 4}
+
+
+def act_mul_quant(h, activation: str, limit=0.0, alpha=1.0, beta=0.0, group_list=None, group_list_type=1):
+    """activation(gate) * up on a 16-bit [rows, 2I] tensor (gate first) + per-row dynamic int8 quantisation."""
+    h = _dev(h, "hidden_states")
+    lib = _lib.load()
+    rows, n = h.shape
+    q = torch.empty((rows, n // 2), dtype=torch.int8, device=h.device)
+    s = torch.empty((rows,), dtype=torch.float32, device=h.device)
+    E = 0
+    if group_list is not None:
+        group_list = _dev(group_list, "group_list")
+        if group_list.dtype != torch.int64:
+            group_list = group_list.to(torch.int64)
+        E = group_list.numel()
+    check(lib.moe355_act_mul_quant(_ptr(h), _dt(h, "hidden_states"), _ptr(group_list), int(group_list_type), E, rows, n,
+                                   ACTIVATIONS[activation], float(limit), float(alpha), float(beta), _ptr(q), _ptr(s),
+                                   _stream(h)), "moe355_act_mul_quant")
+    return q, s
+
+
 def token_unpermute(permuted, sorted_indices, probs, residual=None):
     permuted = _dev(permuted, "permuted_tokens")
     sorted_indices = _dev(sorted_indices, "sorted_indices")
