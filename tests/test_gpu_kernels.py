@@ -679,15 +679,18 @@ def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
-# Skewed histograms: the host picks a kernel family from the mean rows per expert and the device splits the
-# experts between that family and the 128-row tiles.  Mean below 48 with at least 1024 rows: streaming up to 32
-# rows, tiles above (rows at 31 / 32 / 33 sit on the border).  The other two cases keep one family (the
-# weight-streaming tiles) over experts far above and below its range: 255 / 256 / 257 / 511 / 513 rows.
+# Skewed histograms: the host picks a kernel family from the mean rows per expert and, for a large product (a GiB
+# of weights) with 12 to 19 rows per expert on average, the device splits the experts between streaming (up to 32
+# rows: 31 / 32 / 33 sit on the border) and the 128-row tiles.  Small products with the same histogram run on the
+# tiles alone.  The last two cases keep one family (the weight-streaming tiles) over experts far above and below
+# its range: 255 / 256 / 257 / 511 / 513 rows.   name -> (rows per expert, K, N)
+_HOT = [0, 1, 31, 32, 33, 2, 64, 65, 700, 3, 0, 5, 129, 7, 1, 0]
 SKEWED = {
-    "stream+tiled": ([0, 1, 31, 32, 33, 2, 64, 65, 700, 3, 0, 5, 129, 7, 1, 0] + [4] * 48, 256),
-    "stream+tiled, nothing above the border": ([16] * 40 + [32] * 24, 192),
-    "wide": ([255, 256, 257, 511, 513, 1, 0, 33, 128, 160, 161, 192, 193, 40, 90, 100], 1024),
-    "wide, K 4096": ([300, 20, 256, 257, 47, 150, 0, 90], 4096),
+    "stream+tiled": (_HOT + [12] * 240, 4096, 1024),
+    "stream+tiled, nothing above the border": ([16] * 224 + [32] * 32, 4096, 1024),
+    "tiled": (_HOT + [12] * 240, 256, 256),
+    "wide": ([255, 256, 257, 511, 513, 1, 0, 33, 128, 160, 161, 192, 193, 40, 90, 100], 1024, 256),
+    "wide, K 4096": ([300, 20, 256, 257, 47, 150, 0, 90], 4096, 256),
 }
 
 
@@ -696,8 +699,7 @@ SKEWED = {
 def test_grouped_gemms_on_skewed_histograms(K, orc, name, gl_type):
     from vllm_ascend_amd._lib import W_ENK, load
 
-    counts, Kd = SKEWED[name]
-    N = 256
+    counts, Kd, N = SKEWED[name]
     cnt = torch.tensor(counts, dtype=torch.int64)
     E, R = len(counts), int(cnt.sum())
     print(f"skewed gemm {name}: E={E} R={R} K={Kd} N={N} gl_type={gl_type}", flush=True)

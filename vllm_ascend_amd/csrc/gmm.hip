@@ -12,6 +12,7 @@
 // LDS (integer addition: exact, order free).
 #include <hip/hip_ext.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "gmm_common.h"
 #include "gmm_tiled.h"
@@ -50,7 +51,11 @@ __global__ __launch_bounds__(256) void format_cast_nz_kernel(const int8_t* __res
 // ------------------------------------------------------------------ streaming GEMM
 // SLABS: K is cut into gridDim.y slabs (the dense few-row int32 product only; reading gridDim costs every
 // wavefront a scalar load in front of its first weight request, 4 us per launch of the decode down GEMM)
-template <int EPI, int KSPLIT, int UN, int OCC, bool SLABS = false>
+// EARLY: the first weight tiles are requested before the group list is read (decode batches: nearly every expert
+// has rows, and the lookup hides behind the HBM latency).  A launch that covers only some of the experts of a
+// large batch reads the group list first: a unit whose expert is empty or belongs to the other kernel of the call
+// would otherwise fetch 32 KiB for nothing, times thousands of units.
+template <int EPI, int KSPLIT, int UN, int OCC, bool SLABS = false, bool EARLY = true>
 __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
 {
     static_assert(KSPLIT == 1 || KSPLIT == 4, "workgroup barriers need all four wavefronts on one unit");
@@ -98,13 +103,14 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
             }
         }
     };
-    load_weights(kb_begin);
+    if constexpr (EARLY) load_weights(kb_begin);
 
     int64_t row0, row1;
     expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
     if (!expert_in_launch(a, row1 - row0)) return;  // another kernel of this operator call covers the expert
     if (row1 > a.R) row1 = a.R;
     if (row1 <= row0) return;
+    if constexpr (!EARLY) load_weights(kb_begin);
 
     const int tok = lane & 31;
     const int kh = lane >> 5;
@@ -365,7 +371,18 @@ static int tiled_bm(const GmmArgs& a)
     if (force && force[0] == 'u') return 64;
 #endif
     const int64_t avg = a.R / a.E;
-    if (avg < 48) return 0;
+    if (avg < 48) {
+        // Streaming wants every expert inside one 32-row pass.  Measured with uniform routing (the friendliest
+        // case for it) at K = 7168 / 2048: 24 rows per expert on average 1407 / 84 us streaming against 1288 / 74 us
+        // on the tiles, 32 rows 1957 / 115 against 1311 / 75, 16 rows 1223 / 73 against 1266 / 73, 8 rows 1119
+        // against 1244; under Zipf(1.1) routing at 16 rows on average the tiles win as well (1260 against 1521).
+        // Decode batches (fewer than 1024 rows) always stream.
+        if (a.R < 1024 || avg < 12) return 0;
+        if (avg >= 20) return 128;
+        // 12..19 rows per expert: large products split the experts between both families (gemm_plan); for small
+        // ones the second launch costs more than it brings and the tiles alone are as fast as streaming
+        return (int64_t)a.E * a.N * a.K >= (1ll << 30) ? 0 : 128;
+    }
     // the list of 256-row tiles is built from 16-bit counters (tile_map_kernel, by_length)
     const bool wide_ok = a.R / 256 + a.E < 32768;
     if (avg <= 256 && a.K >= 4096 && wide_ok) return 256;
@@ -377,28 +394,39 @@ static int tiled_bm(const GmmArgs& a)
 
 // What one operator call launches: the family chosen from the mean rows per expert, restricted to the experts it
 // is good at, and (split > 0) the 128-row tiles for the experts above that range.
-//   mean < 48 and at least 1024 rows: streaming for experts of at most 32 rows (one pass over their weights),
-//     tiles for the others -- a 500-row expert would otherwise stream its weights 16 times while the units of
-//     the cold experts have long finished.  Below 1024 rows (decode batches) a second launch costs more than the
-//     few extra passes of a hot expert.
+//   mean < 20 (12..19 for products of a GiB of weights and more, see tiled_bm) and at least 1024 rows: streaming
+//     for experts of at most 32 rows (one pass over their weights, and no request before the group list says that
+//     the expert is theirs), tiles for the others -- a 500-row expert would otherwise stream its weights 16 times
+//     while the units of the cold experts have long finished.  Measured at the DeepSeek-V3 shape with Zipf(1.1)
+//     routing, 4096 rows: 1154 us against 1260 (tiles alone) and 1521 (streaming alone) over 244 touched experts;
+//     533 against 568 and 1190 over the 90 touched experts of the benchmark's batch.
 //   The weight-streaming tiles (mean 48..256) keep every expert: sending those above 256 rows to the 128-row
 //     tiles measured the same on a Zipf(1.1) batch of 32,768 rows (2149 against 2180 us for the gate_up product,
 //     1136 against 1119 us for the down product) and would cost the uniform batches an empty launch.
 struct GemmPlan {
-    int bm;     // 0 streaming, 64 / 128 LDS-tiled, 256 weight-streaming tiles
-    int split;  // > 0: experts with more than `split` rows run on the 128-row tiles instead
+    int bm;        // 0 streaming, 64 / 128 LDS-tiled, 256 weight-streaming tiles
+    int split;     // > 0: experts with more than `split` rows run on another family instead
+    int split_bm;  // that family: 128 LDS-tiled, 256 weight-streaming tiles
 };
 
 static GemmPlan gemm_plan(const GmmArgs& a, bool have_tile_ws)
 {
-    GemmPlan p = {have_tile_ws ? tiled_bm(a) : 0, 0};
+    GemmPlan p = {have_tile_ws ? tiled_bm(a) : 0, 0, 128};
     if (a.E == 1 && a.R <= 64) p.bm = 0;  // dense, few rows: the streaming kernel, one workgroup per 64 channels
     if (!have_tile_ws || a.K % 64 != 0 || a.E == 1) return p;
 #ifdef MOE355_DEV_KNOBS
     static const char* force = getenv("MOE355_GEMM");
     if (force && force[0]) return p;
+    static const char* sp = getenv("MOE355_SPLIT");  // "<rows>:<family>", e.g. 32:256
+    if (sp && sp[0] && p.bm == 0 && a.R >= 1024) {  // experiments only
+        p.split = atoi(sp);
+        const char* c = strchr(sp, ':');
+        p.split_bm = c ? atoi(c + 1) : 128;
+        return p;
+    }
 #endif
-    if (p.bm == 0 && a.R >= 1024) p.split = 32;
+    // a large product (a GiB of weights and more) over many experts with few rows on average
+    if (p.bm == 0 && a.R >= 1024 && (int64_t)a.E * a.N * a.K >= (1ll << 30)) p.split = 32;
     return p;
 }
 
@@ -481,6 +509,8 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
         // itself (no K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K (from
         // K = 2048 on that measured 1.5 % faster on the whole layer, below it the same or slower).
         if (done) {
+        } else if (plan.split > 0) {
+            launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, false, false>, dim3((unsigned)units), st, a, ev0, first_stop);
         } else if (EPI != EPI_SWIGLU && units >= 2048 && a.K < 2048) {
             launch_gemm(gmm_stream_kernel<EPI, 1, 4, 2>, dim3((unsigned)((units + 3) / 4)), st, a, ev0, first_stop);
         } else {
@@ -490,7 +520,7 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
     if (plan.split > 0) {
         a.rows_min = plan.split + 1;
         a.rows_max = 0;
-        launch_tiled_any(EPI, 128, a, tile_ws2, st, nullptr, ev1);
+        launch_tiled_any(EPI, plan.split_bm, a, tile_ws2, st, nullptr, ev1);
     }
     return launch_status();
 }
