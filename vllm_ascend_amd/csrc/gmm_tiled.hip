@@ -480,7 +480,7 @@ template <int EPI, bool WIDE, int NBLK = 4>
 __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
                                                  int8_t* lds)
 {
-    static_assert(NBLK == 4 || (WIDE && NBLK > 4 && NBLK <= 8), "tall tiles have two halves of four blocks");
+    static_assert(WIDE ? (NBLK >= 1 && NBLK <= 8) : NBLK == 4, "tall tiles have two halves of four blocks");
     constexpr int GROUPS = WIDE ? 8 : 4;            // channel groups (two storage tiles each) per workgroup
     constexpr int A_BYTES = GROUPS * 4096;          // weights of a stage
     constexpr int X_BYTES = WIDE ? NBLK * 2048 : 16384;  // tokens of a stage
@@ -753,7 +753,13 @@ __global__ __launch_bounds__(512, 1) void gmm_wide_kernel(GmmArgs a, TileMap tm,
     if (mt >= count) return;
     if (row_end > a.R) row_end = a.R;
     if (row0 >= row_end) return;
-    if (row_end - row0 <= 128) {
+    // An expert of a few rows (the cold ones of a skewed batch) runs the same body with one or two token blocks:
+    // the matrix units draw their power whether a block's rows exist or not, and the kernel's clock follows it.
+    if (row_end - row0 <= 32) {
+        stream_tile_body<EPI, true, 1>(a, e, row0, row_end, col, wide_lds);
+    } else if (row_end - row0 <= 64) {
+        stream_tile_body<EPI, true, 2>(a, e, row0, row_end, col, wide_lds);
+    } else if (row_end - row0 <= 128) {
         stream_tile_body<EPI, true>(a, e, row0, row_end, col, wide_lds);
     } else if (row_end - row0 <= 160) {
         stream_tile_body<EPI, true, 5>(a, e, row0, row_end, col, wide_lds);
