@@ -67,6 +67,14 @@ const char *moe355_strerror(int code);
 int moe355_dynamic_quant(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q, float *scale,
                          void *stream);
 
+/* The same operator with the division chosen by the caller.  form 0: what moe355_dynamic_quant and every other
+ * token quantiser of this library run (one reciprocal per row, the product corrected once; rows whose scale lies
+ * outside [2^-100, 2^100] divide); form 1: the general IEEE division on every value, which is the definition above.
+ * No operator of the reference stands behind it: a bf16 / fp16 row holds values of 2^16 patterns below a maximum
+ * of 2^15, so a test can run every (maximum, value) pair through both forms and find the same int8. */
+int moe355_dynamic_quant_form(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q, float *scale,
+                              int form, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Router gate: logits = x.float() @ weight.T (+ bias) in fp32.
  * Stands in for AscendGateLinear.forward (vllm_ascend/ops/fused_moe/gate_linear.py:55-63) and the

@@ -23,6 +23,7 @@ PROTOTYPES = {
     "moe355_abi_version": (c_int, []),
     "moe355_strerror": (c_char_p, [c_int]),
     "moe355_dynamic_quant": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
+    "moe355_dynamic_quant_form": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p]),
     "moe355_router_gate_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "moe355_router_gate": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p,
                                    c_size_t, c_void_p]),

@@ -129,6 +129,43 @@ __device__ __forceinline__ int8_t sat_rint_i8(float v)
     return (int8_t)(int)r;
 }
 
+// The token quantiser on 16-bit inputs: int8(rint(x / s)) for the values x of a row and the row's s = amax / 127.
+// The definition divides (torch_npu.npu_dynamic_quant as the reference calls it,
+// vllm_ascend/ops/fused_moe/moe_mlp.py:211-214: x / scale, rounded, then rounded to an integer); a row shares its
+// divisor, so the kernels take the reciprocal once per row and correct the product once: q0 = x r,
+// q1 = q0 + r (x - s q0) with fused operations.  That is not the correctly rounded quotient for every pair of
+// binary32 numbers, but here x is a bf16 or fp16 value with |x| <= amax and amax is one too: about 2^31 pairs per
+// type, and a test runs all of them through this sequence and through the division and finds the same int8
+// (without the clamp to [-128, 127], which |x| <= amax makes idle: the quotient stays within +-127.00001).
+// Rows whose divisor lies outside [2^-100, 2^100] (bf16 rows of all but vanishing or of astronomic values, where
+// the reciprocal or the residual would leave the normal range) divide.
+struct RowDivisor {
+    float s, r;
+    bool fast;
+};
+
+__device__ __forceinline__ RowDivisor row_divisor(float s, bool ieee_only = false)
+{
+    RowDivisor d;
+    d.s = s;
+    d.r = 1.0f / s;
+    d.fast = !ieee_only && s >= 0x1p-100f && s <= 0x1p100f;
+    return d;
+}
+
+template <bool FAST>
+__device__ __forceinline__ int8_t quantise_by_row(float x, const RowDivisor& d)
+{
+    if constexpr (FAST) {
+        const float q0 = x * d.r;
+        const float e = __builtin_fmaf(-d.s, q0, x);
+        // |x| <= amax keeps the quotient within +-127.00001: nothing to clamp
+        return (int8_t)(int)__builtin_rintf(__builtin_fmaf(e, d.r, q0));
+    } else {
+        return sat_rint_i8(x / d.s);
+    }
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll

@@ -3,6 +3,8 @@
 // One workgroup (256 lanes = 4 wavefronts) per row.  The row absmax is reduced
 // with wavefront shuffles, then across the four wavefronts through LDS; the
 // row is read twice (the second read hits L2) in 16-byte vectors.
+#include <type_traits>
+
 #include "moe355_common.h"
 
 namespace moe355 {
@@ -25,7 +27,8 @@ __device__ __forceinline__ float block_max_256(float v, float* lds4)
 // NV > 0 (VEC only): rows of at most NV x 2048 values stay in registers between the two passes.
 template <bool VEC, int DT, int NV = 0>
 __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __restrict__ x, int64_t cols,
-                                                                 int8_t* __restrict__ q, float* __restrict__ scale)
+                                                                 int8_t* __restrict__ q, float* __restrict__ scale,
+                                                                 int ieee_only)
 {
     __shared__ float lds4[4];
     const int64_t row = blockIdx.x;
@@ -50,19 +53,25 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __re
             }
         a = block_max_256(a, lds4);
         const float s = a / 127.0f;
+        const RowDivisor d = row_divisor(s, ieee_only != 0);
         if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
         uint2* qv = (uint2*)qr;
+        auto emit = [&](auto fast) {
 #pragma unroll
-        for (int n = 0; n < NV; ++n) {
-            const int64_t i = threadIdx.x + 256 * n;
-            uint32_t w[2] = {0u, 0u};
+            for (int n = 0; n < NV; ++n) {
+                const int64_t i = threadIdx.x + 256 * n;
+                uint32_t w[2] = {0u, 0u};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(held[n][j]) / s);
-                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                for (int j = 0; j < 8; ++j) {
+                    int8_t b = (a == 0.0f) ? (int8_t)0
+                                           : quantise_by_row<decltype(fast)::value>(half_to_f32<DT>(held[n][j]), d);
+                    w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                }
+                if (i < nv) qv[i] = make_uint2(w[0], w[1]);
             }
-            if (i < nv) qv[i] = make_uint2(w[0], w[1]);
-        }
+        };
+        if (d.fast) emit(std::true_type{});
+        else emit(std::false_type{});
         return;
     }
     if constexpr (VEC) {
@@ -84,25 +93,31 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __re
     }
     a = block_max_256(a, lds4);
     const float s = a / 127.0f;
+    const RowDivisor d = row_divisor(s, ieee_only != 0);
     if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
-    if constexpr (VEC) {
-        const int64_t nv = cols >> 3;
-        const v8u16* xv = (const v8u16*)xr;
-        uint2* qv = (uint2*)qr;
-        for (int64_t i = threadIdx.x; i < nv; i += 256) {
-            v8u16 v = xv[i];
-            uint32_t w[2] = {0u, 0u};
+    auto emit = [&](auto fast) {
+        constexpr bool F = decltype(fast)::value;
+        if constexpr (VEC) {
+            const int64_t nv = cols >> 3;
+            const v8u16* xv = (const v8u16*)xr;
+            uint2* qv = (uint2*)qr;
+            for (int64_t i = threadIdx.x; i < nv; i += 256) {
+                v8u16 v = xv[i];
+                uint32_t w[2] = {0u, 0u};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(v[j]) / s);
-                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                for (int j = 0; j < 8; ++j) {
+                    int8_t b = (a == 0.0f) ? (int8_t)0 : quantise_by_row<F>(half_to_f32<DT>(v[j]), d);
+                    w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                }
+                qv[i] = make_uint2(w[0], w[1]);
             }
-            qv[i] = make_uint2(w[0], w[1]);
+        } else {
+            for (int64_t i = threadIdx.x; i < cols; i += 256)
+                qr[i] = (a == 0.0f) ? (int8_t)0 : quantise_by_row<F>(half_to_f32<DT>(xr[i]), d);
         }
-    } else {
-        for (int64_t i = threadIdx.x; i < cols; i += 256)
-            qr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(xr[i]) / s);
-    }
+    };
+    if (d.fast) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 // x [rows, n] int32 -> dequant (weight scale, then activation scale) -> SwiGLU -> dynamic int8.
@@ -297,8 +312,8 @@ extern "C" int moe355_silu_f32(const float* g, float* out, int64_t n, int form, 
     return launch_status();
 }
 
-extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q, float* scale,
-                                    void* stream)
+static int dynamic_quant_impl(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q, float* scale,
+                              int ieee_only, void* stream)
 {
     if (rows < 0 || cols <= 0) return MOE355_E_ARG;
     if (rows == 0) return MOE355_OK;
@@ -309,10 +324,10 @@ extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, in
     const bool vec = (cols % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)q & 7) == 0);
 #define MOE355_DQ(V_, D_)                                                                                      \
     hipLaunchKernelGGL((dynamic_quant_kernel<V_, D_>), dim3((unsigned)rows), dim3(256), 0, st, (const uint16_t*)x, \
-                       cols, q, scale)
+                       cols, q, scale, ieee_only)
 #define MOE355_DQH(D_, N_)                                                                                        \
     hipLaunchKernelGGL((dynamic_quant_kernel<true, D_, N_>), dim3((unsigned)rows), dim3(256), 0, st,                \
-                       (const uint16_t*)x, cols, q, scale)
+                       (const uint16_t*)x, cols, q, scale, ieee_only)
     if (x_dtype == MOE355_DT_BF16) {
         if (vec && cols <= 2048) MOE355_DQH(MOE355_DT_BF16, 1);
         else if (vec && cols <= 4096) MOE355_DQH(MOE355_DT_BF16, 2);
@@ -329,6 +344,19 @@ extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, in
 #undef MOE355_DQH
 #undef MOE355_DQ
     return launch_status();
+}
+
+extern "C" int moe355_dynamic_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q, float* scale,
+                                    void* stream)
+{
+    return dynamic_quant_impl(x, x_dtype, rows, cols, q, scale, 0, stream);
+}
+
+extern "C" int moe355_dynamic_quant_form(const void* x, int x_dtype, int64_t rows, int64_t cols, int8_t* q,
+                                         float* scale, int form, void* stream)
+{
+    if (form != 0 && form != 1) return MOE355_E_ARG;
+    return dynamic_quant_impl(x, x_dtype, rows, cols, q, scale, form, stream);
 }
 
 extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight_scale, const float* activation_scale,

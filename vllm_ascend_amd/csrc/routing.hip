@@ -16,6 +16,7 @@
 // destination rows.  Batches of at most 2048 pairs take one launch for all of it
 // (route_gather_small_kernel).
 #include <mutex>
+#include <type_traits>
 
 #include "moe355_common.h"
 
@@ -242,19 +243,25 @@ __device__ __forceinline__ void gather_token_row(const uint16_t* __restrict__ xr
         a = lds4[2] > a ? lds4[2] : a;
         a = lds4[3] > a ? lds4[3] : a;
         const float s = a / 127.0f;
+        const RowDivisor d = row_divisor(s);
         if (threadIdx.x < top_k && drow[threadIdx.x] >= 0) sx[drow[threadIdx.x]] = (a == 0.0f) ? 0.0f : s;
-        for (int64_t i = threadIdx.x; i < nv; i += 256) {
-            v8u16 v = i < 256 ? held : xv[i];
-            uint32_t w[2] = {0u, 0u};
+        auto emit = [&](auto fast) {
+            for (int64_t i = threadIdx.x; i < nv; i += 256) {
+                v8u16 v = i < 256 ? held : xv[i];
+                uint32_t w[2] = {0u, 0u};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                int8_t b = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(v[j]) / s);
-                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                for (int j = 0; j < 8; ++j) {
+                    int8_t b = (a == 0.0f) ? (int8_t)0
+                                           : quantise_by_row<decltype(fast)::value>(half_to_f32<DT>(v[j]), d);
+                    w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+                }
+                const uint2 pk = make_uint2(w[0], w[1]);
+                for (int j = 0; j < top_k; ++j)
+                    if (drow[j] >= 0) ((uint2*)((int8_t*)xs + (int64_t)drow[j] * H))[i] = pk;
             }
-            const uint2 pk = make_uint2(w[0], w[1]);
-            for (int j = 0; j < top_k; ++j)
-                if (drow[j] >= 0) ((uint2*)((int8_t*)xs + (int64_t)drow[j] * H))[i] = pk;
-        }
+        };
+        if (d.fast) emit(std::true_type{});
+        else emit(std::false_type{});
     }
 }
 

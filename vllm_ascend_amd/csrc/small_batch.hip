@@ -4,7 +4,7 @@
 // quantisation), and the expert GEMM reads the gathered copy.  For a few hundred (token, slot) pairs that is two
 // launches of a few microseconds each in front of a weight stream of some tens of microseconds.  Here one launch
 // does both:
-//   - the first ceil(T / 4) workgroups gate four token rows each (one per wavefront, the arithmetic of the gating
+//   - ceil(T / 4) workgroups (every fifth of the grid) gate four token rows each (one per wavefront, the arithmetic of the gating
 //     kernel) and then count themselves on a counter; the one that finds all the others done sorts the T * k pairs
 //     by expert, stably: per-chunk histograms in LDS (a chunk = 64 consecutive pairs), a scan over (chunk, expert),
 //     ballot-matched ranks inside a chunk.  Nobody waits for anybody: a workgroup that is not the last one ends;
@@ -68,18 +68,24 @@ __device__ __forceinline__ void quantise_token_row(const SmallRouteArgs& a, int 
 #pragma unroll
     for (int w = 1; w < kSmallWaves; ++w) amax = lds16[w] > amax ? lds16[w] : amax;
     const float s = amax / 127.0f;
+    const RowDivisor d = row_divisor(s);
     if (tid == 0) a.x_scale[t] = (amax == 0.0f) ? 0.0f : s;
     uint2* qv = (uint2*)(a.xq + (int64_t)t * a.H);
-    for (int64_t i = tid; i < nv; i += kSmallThreads) {
-        const v8u16 v = i < kSmallThreads ? held : xv[i];
-        uint32_t w[2] = {0u, 0u};
+    auto emit = [&](auto fast) {
+        for (int64_t i = tid; i < nv; i += kSmallThreads) {
+            const v8u16 v = i < kSmallThreads ? held : xv[i];
+            uint32_t w[2] = {0u, 0u};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int8_t b = (amax == 0.0f) ? (int8_t)0 : sat_rint_i8(half_to_f32<DT>(v[j]) / s);
-            w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+            for (int j = 0; j < 8; ++j) {
+                const int8_t b = (amax == 0.0f) ? (int8_t)0
+                                                : quantise_by_row<decltype(fast)::value>(half_to_f32<DT>(v[j]), d);
+                w[j >> 2] |= (uint32_t)(uint8_t)b << (8 * (j & 3));
+            }
+            qv[i] = make_uint2(w[0], w[1]);
         }
-        qv[i] = make_uint2(w[0], w[1]);
-    }
+    };
+    if (d.fast) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 // LDT: dtype of the logits; XDT: dtype of the hidden states (and of the weights that are returned)
