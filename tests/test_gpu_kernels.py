@@ -648,8 +648,10 @@ TILE_COUNTS = [128, 64, 65, 129, 192, 193, 1, 0, 256, 63, 127, 320, 160, 161, 14
 
 # K >= 1024 at about 128 rows per expert selects the weight-streaming tiles (tall ones and wide ones of four and of
 # five token blocks occur in TILE_COUNTS); the K values leave every remainder of the three-, four- and five-stage
-# rings
-@pytest.mark.parametrize("Kd,N", [(256, 256), (192, 128), (512, 320), (1024, 256), (2112, 128), (4096, 256),
+# rings; below K = 1024 the 128-row tiles run, whose closing steps are compiled per remainder of K / 64 by three
+# (64 and 128: fewer K blocks than the ring is deep)
+@pytest.mark.parametrize("Kd,N", [(64, 128), (128, 256), (256, 256), (192, 128), (320, 128), (384, 192), (512, 320),
+                                  (768, 256), (1024, 256), (2112, 128), (4096, 256),
                                   (4160, 320), (4224, 128), (4288, 256), (4352, 192), (4416, 1152)])
 def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
     print(f"tiled gemms at tile boundaries K={Kd} N={N}", flush=True)

@@ -12,6 +12,8 @@
 #include <hip/hip_ext.h>
 
 #include "gmm_common.h"
+#include <type_traits>
+
 #include "gmm_tiled.h"
 
 namespace moe355 {
@@ -261,7 +263,8 @@ __device__ __forceinline__ void tiled_epilogue(const GmmArgs& a, int e, v16i (&a
 // One tile of BMT token blocks: rows [row0, row_end) of expert e (at most 32 * BMT of them are computed),
 // column block nt.
 // RING = depth of the operand ring in registers: weights are requested RING - 1 K blocks ahead, tokens RING.
-template <int EPI, int BMT, int RING>  // BMT = token blocks of 32 per tile (BM = 32 * BMT)
+// REM: K / 64 modulo RING when K / 64 >= RING (the closing steps are then specialised), -1 for any K.
+template <int EPI, int BMT, int RING, int REM>  // BMT = token blocks of 32 per tile (BM = 32 * BMT)
 __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0, int64_t row_end, int nt,
                                            int8_t* lds_raw)
 {
@@ -372,8 +375,9 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
     __syncthreads();
     read_frags(bf0, 0, 0);
 
-    // One pipeline step on stage U (compile-time ring position) for K block I.
-#define MOE355_STEP(U, I)                                                                        \
+    // One pipeline step on stage U (compile-time ring position) for K block I.  LA / LB: request the weights of
+    // K block I + RING - 1 / the tokens of K block I + RING; SB: move the tokens of K block I + 1 to LDS.
+#define MOE355_STEP(U, I, LA, LB, SB)                                                            \
     {                                                                                            \
         /* first K step: its MFMAs go first; the LDS traffic of the second K step and of the */  \
         /* next stage is issued in the gaps while the matrix pipe is busy                    */  \
@@ -382,7 +386,7 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
             acc[0][b] = mfma_i8(Areg[(U)][0][0], bf0[b], acc[0][b]);                             \
             acc[1][b] = mfma_i8(Areg[(U)][1][0], bf0[b], acc[1][b]);                             \
             bf1[b] = *(const v4i*)(&Bs[(U)][((BMT + b) * 64 + lane) * 16]);                      \
-            if (b == 0) store_B(((U) + 1) % RING); /* B(I+1): registers -> LDS */                \
+            if ((SB) && b == 0) store_B(((U) + 1) % RING); /* B(I+1): registers -> LDS */        \
             __builtin_amdgcn_sched_barrier(0);                                                   \
         }                                                                                        \
         __syncthreads(); /* B(I+1) visible to all wavefronts */                                  \
@@ -390,24 +394,43 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
         {                                                                                        \
             acc[0][b] = mfma_i8(Areg[(U)][0][1], bf1[b], acc[0][b]);                             \
             acc[1][b] = mfma_i8(Areg[(U)][1][1], bf1[b], acc[1][b]);                             \
-            bf0[b] = *(const v4i*)(&Bs[((U) + 1) % RING][(b * 64 + lane) * 16]);                 \
-            if (b == 0) load_A((I) + RING - 1, ((U) + RING - 1) % RING);                         \
-            if (b == (BMT > 1 ? 1 : 0)) load_B((I) + RING, (U));                                 \
+            if (SB) bf0[b] = *(const v4i*)(&Bs[((U) + 1) % RING][(b * 64 + lane) * 16]);         \
+            if ((LA) && b == 0) load_A((I) + RING - 1, ((U) + RING - 1) % RING);                 \
+            if ((LB) && b == (BMT > 1 ? 1 : 0)) load_B((I) + RING, (U));                         \
             __builtin_amdgcn_sched_barrier(0);                                                   \
         }                                                                                        \
     }
-    // whole passes through the ring run without any condition inside (exact wait counts); the remainder is peeled
-    const int n_full = (n_iter / RING) * RING;
-    for (int i0 = 0; i0 < n_full; i0 += RING) {
-        MOE355_STEP(0, i0)
-        MOE355_STEP(1, i0 + 1)
-        MOE355_STEP(2, i0 + 2)
-        if constexpr (RING > 3) MOE355_STEP(3, i0 + 3)
-    }
-    if (n_iter - n_full >= 1) MOE355_STEP(0, n_full)
-    if (n_iter - n_full >= 2) MOE355_STEP(1, n_full + 1)
-    if constexpr (RING > 3) {
-        if (n_iter - n_full >= 3) MOE355_STEP(2, n_full + 2)
+    if constexpr (REM < 0) {
+        // any K: whole passes through the ring run without any condition inside (exact wait counts), the remainder
+        // is peeled; requests past the last K block are redirected to it (load_A, load_B)
+        const int n_full = (n_iter / RING) * RING;
+        for (int i0 = 0; i0 < n_full; i0 += RING) {
+            MOE355_STEP(0, i0, 1, 1, 1)
+            MOE355_STEP(1, i0 + 1, 1, 1, 1)
+            MOE355_STEP(2, i0 + 2, 1, 1, 1)
+        }
+        if (n_iter - n_full >= 1) MOE355_STEP(0, n_full, 1, 1, 1)
+        if (n_iter - n_full >= 2) MOE355_STEP(1, n_full + 1, 1, 1, 1)
+    } else {
+        // K / 64 = 3 q + REM with q >= 1 (the host picks the instantiation).  The last RING steps request nothing
+        // that lies past the last K block (the weights of the last block are requested RING - 1 steps before it,
+        // its tokens RING steps before); their ring positions follow from REM, so every step is written out with
+        // its requests decided at compile time: no condition inside a step, exact waits, and a tile of 12 K blocks
+        // issues 66 loads per wavefront instead of 80.
+        static_assert(RING == 3, "the closing steps are written for a ring of three");
+        const int n_pass = (n_iter - RING - REM) / RING;  // whole passes that request both operands
+        int it = 0;
+        for (int ps = 0; ps < n_pass; ++ps, it += RING) {
+            MOE355_STEP(0, it, 1, 1, 1)
+            MOE355_STEP(1, it + 1, 1, 1, 1)
+            MOE355_STEP(2, it + 2, 1, 1, 1)
+        }
+        if constexpr (REM >= 1) MOE355_STEP(0, it, 1, 1, 1)
+        if constexpr (REM >= 2) MOE355_STEP(1, it + 1, 1, 1, 1)
+        it += REM;
+        MOE355_STEP(REM % RING, it, 1, 0, 1)
+        MOE355_STEP((REM + 1) % RING, it + 1, 0, 0, 1)
+        MOE355_STEP((REM + 2) % RING, it + 2, 0, 0, 0)
     }
 #undef MOE355_STEP
 
@@ -419,7 +442,7 @@ __device__ __forceinline__ void tiled_body(const GmmArgs& a, int e, int64_t row0
 // The last tile of an expert is usually short.  Tiles of at most 64 rows run the two-block body (half the
 // MFMAs and half the token traffic of a full tile) inside the same launch, next to the full tiles of their
 // expert, so that they still find the expert's weights in the L2 of their XCD.
-template <int EPI, int BMT, int RING>
+template <int EPI, int BMT, int RING, int REM>
 __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : 2)) void gmm_tiled_kernel(GmmArgs a, TileMap tm, int max_tiles, int n_col_blocks)
 {
     __shared__ __attribute__((aligned(16))) int8_t lds_raw[TiledLds<EPI, BMT, RING>::BYTES];
@@ -439,11 +462,11 @@ __global__ __launch_bounds__(256, (BMT <= 2 ? 3 : 2)) void gmm_tiled_kernel(GmmA
     if (row0 >= row_end) return;
     if constexpr (BMT > 2) {
         if (row_end - row0 <= 64) {
-            tiled_body<EPI, 2, RING>(a, e, row0, row_end, nt, lds_raw);
+            tiled_body<EPI, 2, RING, REM>(a, e, row0, row_end, nt, lds_raw);
             return;
         }
     }
-    tiled_body<EPI, BMT, RING>(a, e, row0, row_end, nt, lds_raw);
+    tiled_body<EPI, BMT, RING, REM>(a, e, row0, row_end, nt, lds_raw);
 }
 
 // ------------------------------------------------------------------ weight-streaming tiles
@@ -616,20 +639,43 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
         load_weights(j + SW - 1, j + SW - 1);
     }
 
-    constexpr int NAFTER = (SW > SX) ? NA : 0;  // the weights requested right behind a step's tokens
-    const int n_full = (n_iter / CYCLE) * CYCLE;
+    // Requests that may still be in flight when the step d before the last one (d = kSteady: any step that is at
+    // least SW - 1 before it) waits for the stage `ahead` steps after its own: everything requested behind that
+    // stage's tokens.  The last SW - 1 steps request no weights and the last SX - 1 no tokens (nothing lies past the
+    // last K block), so the counts shrink towards the end; each of those steps is compiled with its own.
+    constexpr int kSteady = 1 << 20;
+    auto in_flight = [](int d, int ahead, int nx) constexpr {
+        int n = (SW > SX && d >= SW - SX + ahead) ? NA : 0;  // the weights requested right behind those tokens
+        for (int m = 1; m <= SX - 2 - ahead; ++m) n += (d + m >= SX - 1 ? nx : 0) + (d + m >= SW - 1 ? NA : 0);
+        return n;
+    };
+    // the steps d = SW - 2 .. 0 before the end (those that exist), each with its distance as a type
+    auto closing_steps = [&](auto& step_fn, auto dfirst) {
+        auto one = [&](auto self, auto dtag) -> void {
+            constexpr int D = decltype(dtag)::value;
+            if (D < n_iter) {
+                const int it = last_it - D;
+                step_fn(dtag, it % SW, it % SX, it);
+            }
+            if constexpr (D > 0) self(self, std::integral_constant<int, D - 1>{});
+        };
+        one(one, dfirst);
+    };
+    const int n_main = n_iter > SW - 1 ? n_iter - (SW - 1) : 0;  // steps that request both operands
+    const int n_full = (n_main / CYCLE) * CYCLE;
     if constexpr (WIDE) {
         // One K block on stage uw of the weights and ux of the tokens.  Requests retire in order.  The younger of
         // the two requests that this step needs is its tokens (its weights, in the same step, if the rings are
         // equally deep): what was requested after it may still be in flight.  The barrier then covers the other
         // wavefronts and also says that everybody is done reading the stages that the next requests overwrite.
-        auto step = [&](int uw, int ux, int it) {
-            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
-            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
-            else wait_vmcnt<NAFTER + NA * (SX - 2)>();
+        auto step = [&](auto dtag, int uw, int ux, int it) {
+            constexpr int D = decltype(dtag)::value;
+            if (n_xloads == 2) wait_vmcnt<in_flight(D, 0, 2)>();
+            else if (n_xloads == 1) wait_vmcnt<in_flight(D, 0, 1)>();
+            else wait_vmcnt<in_flight(D, 0, 0)>();
             __builtin_amdgcn_s_barrier();
-            load_tokens(it + SX - 1, (ux + SX - 1) % SX);
-            load_weights(it + SW - 1, (uw + SW - 1) % SW);
+            if constexpr (D >= SX - 1) load_tokens(it + SX - 1, (ux + SX - 1) % SX);
+            if constexpr (D >= SW - 1) load_weights(it + SW - 1, (uw + SW - 1) % SW);
             if (active) {
                 const int8_t* wbase = lds + uw * A_BYTES;
                 const int8_t* xbase = lds + ux * X_BYTES;
@@ -646,13 +692,16 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
                 }
             }
         };
+        constexpr std::integral_constant<int, kSteady> steady{};
         for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
 #pragma unroll
-            for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
+            for (int u = 0; u < CYCLE; ++u) step(steady, u % SW, u % SX, i0 + u);
         }
 #pragma unroll
         for (int u = 0; u + 1 < CYCLE; ++u)
-            if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
+            if (n_full + u < n_main) step(steady, u % SW, u % SX, n_full + u);
+        // the closing steps: ring positions known at run time only (three or four steps of a tile's dozens)
+        closing_steps(step, std::integral_constant<int, SW - 2>{});
     } else {
         // Tall tiles are bound by the matrix units, and every wavefront meets the others at the barrier of every K
         // block: operand reads that start behind that barrier leave all eight wavefronts, both of each SIMD, without
@@ -677,15 +726,17 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
         // the stage of K block 0 has landed (for everybody): its first operands
         auto wait_stage = [&]() {
             // the younger request of the stage waited for is its tokens; behind them: the weights of that step and
-            // every request of the later steps
-            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 2)>();
-            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 2)>();
-            else wait_vmcnt<NAFTER + NA * (SX - 2)>();
+            // every request of the later steps (the steps before the first have requested everything, redirected
+            // to the last K block where a tile has fewer blocks than the rings are deep)
+            if (n_xloads == 2) wait_vmcnt<in_flight(kSteady, 0, 2)>();
+            else if (n_xloads == 1) wait_vmcnt<in_flight(kSteady, 0, 1)>();
+            else wait_vmcnt<in_flight(kSteady, 0, 0)>();
         };
-        auto wait_next_stage = [&]() {
-            if (n_xloads == 2) wait_vmcnt<NAFTER + (NA + 2) * (SX - 3)>();
-            else if (n_xloads == 1) wait_vmcnt<NAFTER + (NA + 1) * (SX - 3)>();
-            else wait_vmcnt<NAFTER + NA * (SX - 3)>();
+        auto wait_next_stage = [&](auto dtag) {
+            constexpr int D = decltype(dtag)::value;
+            if (n_xloads == 2) wait_vmcnt<in_flight(D, 1, 2)>();
+            else if (n_xloads == 1) wait_vmcnt<in_flight(D, 1, 1)>();
+            else wait_vmcnt<in_flight(D, 1, 0)>();
         };
         static_assert(SX >= 4, "a block reads the stage after its own: three stages in flight plus the one overwritten");
         wait_stage();
@@ -694,11 +745,12 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
 #pragma unroll
             for (int part = 0; part < NBLK; ++part) read_operands(0, 0, 0, 0, part);
         }
-        auto step = [&](int uw, int ux, int it) {
-            wait_next_stage();  // stage it + 1 has landed
+        auto step = [&](auto dtag, int uw, int ux, int it) {
+            constexpr int D = decltype(dtag)::value;
+            if constexpr (D > 0) wait_next_stage(dtag);  // stage it + 1 has landed
             __builtin_amdgcn_s_barrier();
-            load_tokens(it + SX - 1, (ux + SX - 1) % SX);
-            load_weights(it + SW - 1, (uw + SW - 1) % SW);
+            if constexpr (D >= SX - 1) load_tokens(it + SX - 1, (ux + SX - 1) % SX);
+            if constexpr (D >= SW - 1) load_weights(it + SW - 1, (uw + SW - 1) % SW);
             if (active) {
                 // K step 0 on set 0, reading K step 1 into set 1
 #pragma unroll
@@ -713,18 +765,20 @@ __device__ __forceinline__ void stream_tile_body(const GmmArgs& a, int e, int64_
                 for (int b = 0; b < NBLK; ++b) {
                     acc[0][b] = mfma_i8(fa[1][0], fb[1][b], acc[0][b]);
                     acc[1][b] = mfma_i8(fa[1][1], fb[1][b], acc[1][b]);
-                    read_operands(0, (uw + 1) % SW, (ux + 1) % SX, 0, b);
+                    if constexpr (D > 0) read_operands(0, (uw + 1) % SW, (ux + 1) % SX, 0, b);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
+        constexpr std::integral_constant<int, kSteady> steady{};
         for (int i0 = 0; i0 < n_full; i0 += CYCLE) {
 #pragma unroll
-            for (int u = 0; u < CYCLE; ++u) step(u % SW, u % SX, i0 + u);
+            for (int u = 0; u < CYCLE; ++u) step(steady, u % SW, u % SX, i0 + u);
         }
 #pragma unroll
         for (int u = 0; u + 1 < CYCLE; ++u)
-            if (n_full + u < n_iter) step(u % SW, u % SX, n_full + u);
+            if (n_full + u < n_main) step(steady, u % SW, u % SX, n_full + u);
+        closing_steps(step, std::integral_constant<int, SW - 2>{});
     }
 
     wait_vmcnt<0>();  // the redirected loads past the end still write LDS
@@ -822,12 +876,18 @@ static void launch_tiled(const GmmArgs& a, void* workspace, hipStream_t st, hipE
     const int n_col_blocks = (channels + per_block - 1) / per_block;
     const int total = max_tiles * n_col_blocks;
     const int grid = ((total + 7) / 8) * 8;
-    if (ev0 || ev1)
-        hipExtLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT, RING>), dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm,
-                              max_tiles, n_col_blocks);
-    else
-        hipLaunchKernelGGL((gmm_tiled_kernel<EPI, BMT, RING>), dim3(grid), dim3(256), 0, st, a, tm, max_tiles,
-                           n_col_blocks);
+    auto launch = [&](auto kernel) {
+        if (ev0 || ev1)
+            hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, st, ev0, ev1, 0, a, tm, max_tiles, n_col_blocks);
+        else
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, st, a, tm, max_tiles, n_col_blocks);
+    };
+    // the closing steps of the K loop are compiled for K / 64 modulo the ring depth
+    const int n_iter = a.K / kBK;
+    if (n_iter < RING) launch(gmm_tiled_kernel<EPI, BMT, RING, -1>);
+    else if (n_iter % RING == 0) launch(gmm_tiled_kernel<EPI, BMT, RING, 0>);
+    else if (n_iter % RING == 1) launch(gmm_tiled_kernel<EPI, BMT, RING, 1>);
+    else launch(gmm_tiled_kernel<EPI, BMT, RING, 2>);
 }
 
 template <int EPI>
