@@ -326,7 +326,9 @@ GMM_CASES = [(8, 128, 256, 128), (128, 2, 1024, 2816), (500, 32, 512, 512), (100
              (64, 1, 7168, 256), (33, 1, 2048, 1024), (1, 1, 4096, 128),
              # one expert with thousands of rows (the shared expert of a prefill batch): the dense kernel's 256 x 256
              # tiles, with a ragged last row tile and a last column block of 64 channels
-             (3000, 1, 128, 4096), (2049, 1, 192, 6464)]
+             # (K of one to seven blocks of 64: fewer than, as many as and more than the closing steps of its K loop)
+             (3000, 1, 128, 4096), (2049, 1, 192, 6464), (2100, 1, 64, 4096), (2050, 1, 384, 4096),
+             (2300, 1, 448, 4096)]
 
 
 @pytest.mark.parametrize("R,E,Kd,N", GMM_CASES)
