@@ -161,6 +161,12 @@ SMALL_ROUTE_CASES = [
     (33, 6, 96, 9216, 1, 0, True, 4, 2, 1.5, torch.float16, torch.float16),      # rows longer than one pass
     (17, 2, 3, 72, 0, 1, False, 1, 1, 1.0, torch.float32, torch.float16),
     (100, 4, 256, 128, 0, 1, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
+    # a handful of tokens: fewer gating workgroups than wavefronts in one, groups that do not divide 64
+    (16, 8, 256, 7168, 1, 1, True, 8, 4, 2.5, torch.float32, torch.bfloat16),
+    (8, 8, 128, 2048, 0, 1, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
+    (5, 4, 64, 256, 1, 0, True, 4, 2, 1.0, torch.bfloat16, torch.bfloat16),
+    (13, 6, 160, 512, 0, 1, False, 5, 3, 1.0, torch.float16, torch.float16),
+    (2, 2, 2, 64, 0, 1, False, 1, 1, 1.0, torch.float32, torch.bfloat16),
 ]
 
 
