@@ -74,6 +74,31 @@ def test_gating_top_k(K, orc, case):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), no.view(np.uint32))
 
 
+# Group-limited routing over every group length: powers of two up to 64 (the group scores come from a butterfly
+# over the lanes of a group), others (one lane per group walks its experts), with logits from a set of five values
+# so that ties inside and between groups are the rule, and with zeros of both signs.
+@pytest.mark.parametrize("E,G,k_group,k", [(8, 8, 3, 2), (16, 8, 4, 4), (64, 16, 5, 6), (128, 8, 3, 8), (256, 16, 4, 8),
+                                           (256, 8, 4, 8), (512, 8, 2, 8), (96, 4, 2, 6), (160, 5, 3, 8), (384, 2, 1, 4),
+                                           (256, 64, 9, 8)])
+@pytest.mark.parametrize("mode,norm_type", [(1, 1), (0, 0)])
+def test_gating_groups_with_ties(K, orc, E, G, k_group, k, mode, norm_type):
+    print(f"gating groups with ties E={E} G={G} k_group={k_group} k={k} mode={mode} norm={norm_type}", flush=True)
+    T = 37
+    g = torch.Generator().manual_seed(E * 31 + G)
+    levels = torch.tensor([-1.5, -0.0, 0.0, 0.75, 2.0])
+    x = levels[torch.randint(0, 5, (T, E), generator=g)]
+    x[1::3] = (torch.rand(T, E, generator=g) * 4 - 2)[1::3]   # some rows without ties
+    bias = levels[torch.randint(0, 5, (E,), generator=g)] * 0.5
+    y, idx, out = K.gating_top_k(x.to(DEV), k, k_group, G, mode, 1, norm_type, True, 1.0, 1e-20, bias.to(DEV))
+    torch.cuda.synchronize()
+    yo, io, no = orc.gating_top_k(bits(x), k, bias=bits(bias), k_group=k_group, group_count=G, group_select_mode=mode,
+                                  renorm=1, norm_type=norm_type, routed_scaling_factor=1.0, eps=1e-20, x_dtype="f32",
+                                  want_norm=True)
+    assert np.array_equal(idx.cpu().numpy(), io)
+    assert np.array_equal(bits(y).view(np.uint32), yo.view(np.uint32))
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), no.view(np.uint32))
+
+
 @pytest.mark.parametrize("T,k,E,H", [(3, 2, 2, 64), (64, 8, 128, 2048), (1, 1, 8, 64), (700, 8, 256, 512),
                                      (2000, 4, 16, 128), (40, 6, 2048, 64),
                                      # the single-launch path ends at 2048 rows; 64 slots per token is its widest

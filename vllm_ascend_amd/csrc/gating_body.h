@@ -91,6 +91,56 @@ __device__ __forceinline__ float group_score(const float* s, int gs, int mode)
     return (mode != 0 && gs >= 2) ? v1 + v2 : v1;
 }
 
+// The scores of all groups of one row at once, for groups of a power of two of at most 64 experts: such a group is
+// a run of gs lanes in one of the row's registers (expert e = lane + 64 i), so a butterfly over the lanes of the
+// run leaves the group's two largest selection scores in every one of them.  The same two values as the pass of
+// group_score (a tie is two equal values either way; the order of a +0 and a -0 does not change their sum), the
+// same sum; a row that holds a NaN takes group_score instead, whose treatment of it depends on the position.
+// Lane g (< G) returns the score of group g, the other lanes anything.
+template <int PER>
+__device__ __forceinline__ float group_scores_butterfly(const float (&sel)[PER], int gs, int mode, int lane)
+{
+    float t1[PER], t2[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        t1[i] = sel[i];
+        t2[i] = -__builtin_inff();
+    }
+    for (int m = 1; m < gs; m <<= 1) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const float p1 = __shfl_xor(t1[i], m);
+            const float p2 = __shfl_xor(t2[i], m);
+            const bool gt = t1[i] > p1;
+            const float hi = gt ? t1[i] : p1;
+            const float lo = gt ? p1 : t1[i];
+            const float second = t2[i] > p2 ? t2[i] : p2;
+            t1[i] = hi;
+            t2[i] = lo > second ? lo : second;
+        }
+    }
+    const int runs = 64 / gs;  // groups per register
+    const int src = (lane % runs) * gs;
+    float out = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const float sc = (mode != 0 && gs >= 2) ? t1[i] + t2[i] : t1[i];
+        const float v = __shfl(sc, src);
+        if (lane / runs == i) out = v;
+    }
+    return out;
+}
+
+template <int PER>
+__device__ __forceinline__ bool butterfly_groups(const float (&sel)[PER], int gs)
+{
+    if (gs > 64 || (gs & (gs - 1)) != 0) return false;
+    bool nan = false;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) nan = nan || (sel[i] != sel[i]);
+    return __ballot(nan) == 0ull;
+}
+
 // One token row by one wavefront.  Every wavefront of the workgroup calls this the same number of times (it
 // contains workgroup barriers); a call with live == false computes a valid row and stores nothing.
 // sc_lds: E floats, w_lds: 64 floats, both private to the wavefront.  y may be null (only y_alt wanted);
@@ -153,7 +203,10 @@ __device__ __forceinline__ void gate_row(const void* __restrict__ x, const void*
         }
         __syncthreads();
         unsigned long long gkey = 0ull;
-        if (lane < G) {
+        if (butterfly_groups<PER>(sel, gs)) {
+            const float sc = group_scores_butterfly<PER>(sel, gs, mode, lane);
+            if (lane < G) gkey = make_key(sc, lane);
+        } else if (lane < G) {
             const float* s = sc_lds + lane * gs;
             gkey = make_key(group_score(s, gs, mode), lane);
         }
@@ -280,7 +333,10 @@ __device__ __forceinline__ void gate_rows(const void* __restrict__ x, const void
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             gkey[r] = 0ull;
-            if (lane < G) {
+            if (butterfly_groups<PER>(sel[r], gs)) {
+                const float sc = group_scores_butterfly<PER>(sel[r], gs, mode, lane);
+                if (lane < G) gkey[r] = make_key(sc, lane);
+            } else if (lane < G) {
                 gkey[r] = make_key(group_score(grp_lds + r * E + lane * gs, gs, mode), lane);
             }
         }
