@@ -17,26 +17,33 @@ namespace moe355 {
 // without a source keep their own value, which is harmless for max.
 #define MOE355_DPP(v, ctrl, rmask) __builtin_amdgcn_update_dpp((int)(v), (int)(v), ctrl, rmask, 0xf, false)
 
-// Maximum of a 64-bit key over the wavefront; every lane returns it.
+// Maximum of an unsigned value over the wavefront; every lane returns it.  Six DPP steps, each one v_max_u32 that
+// reads its first operand through the lane permutation (the compiler keeps the permutation and the maximum apart:
+// copy, v_mov_dpp, compare, select).  A lane without a source in a step (shifted in from outside its row, or a row
+// outside the row mask) is left as it is.  The s_nop in front of every step is the wait that a DPP read of a
+// register needs after a vector instruction has written it.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v)
+{
+    asm volatile(
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(v));
+    return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// Maximum of a 64-bit key over the wavefront; every lane returns it: the largest high word, and the largest low
+// word among the lanes that hold it.
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
 {
-#define MOE355_STEP(ctrl, rmask)                                                             \
-    {                                                                                        \
-        unsigned lo = (unsigned)MOE355_DPP((unsigned)v, ctrl, rmask);                        \
-        unsigned hi = (unsigned)MOE355_DPP((unsigned)(v >> 32), ctrl, rmask);                \
-        unsigned long long o = ((unsigned long long)hi << 32) | lo;                          \
-        v = o > v ? o : v;                                                                   \
-    }
-    MOE355_STEP(0x111, 0xf)  // row_shr:1
-    MOE355_STEP(0x112, 0xf)  // row_shr:2
-    MOE355_STEP(0x114, 0xf)  // row_shr:4
-    MOE355_STEP(0x118, 0xf)  // row_shr:8
-    MOE355_STEP(0x142, 0xa)  // row_bcast:15
-    MOE355_STEP(0x143, 0xc)  // row_bcast:31
-#undef MOE355_STEP
-    unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)v, 63);
-    unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(v >> 32), 63);
-    return ((unsigned long long)hi << 32) | lo;
+    const unsigned hi = (unsigned)(v >> 32);
+    const unsigned m = wave_max_u32(hi);
+    const unsigned lo = wave_max_u32(hi == m ? (unsigned)v : 0u);
+    return ((unsigned long long)m << 32) | lo;
 }
 
 __device__ __forceinline__ float wave_max_dpp(float v)
