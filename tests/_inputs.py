@@ -28,7 +28,7 @@ class LayerCfg:
 
 
 CONFIGS = {
-    # BASELINE configs (full sizes) and reduced variants for CPU-checkable parity
+    # the benchmark configurations (full sizes) and reduced variants for CPU-checkable parity
     "c1_tiny": LayerCfg("c1_tiny", 64, 1024, 8, 2, 1408),
     "c2_qwen3_decode": LayerCfg("c2_qwen3_decode", 64, 2048, 128, 8, 768),
     "c3_qwen3_prefill": LayerCfg("c3_qwen3_prefill", 8192, 2048, 128, 8, 768),
