@@ -49,12 +49,12 @@ WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_
 # kernel of known size), taken from the committed summaries: NOT measured in this run.
 TRAFFIC_FROM_PROFILES = {
     "c2_qwen3_decode": (401_500_000, "profiles/moe_layer_qwen3_decode_kernel_trace.md"),
-    "c3_qwen3_prefill": (953_600_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
-    "c4_dsv3_prefill": (8_031_800_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
-    "c5_w4a8_zipf": (1_677_300_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
+    "c3_qwen3_prefill": (955_400_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
+    "c4_dsv3_prefill": (8_031_500_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
+    "c5_w4a8_zipf": (1_673_400_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
     "c6_dsv3_decode": (6_628_300_000, "profiles/moe_layer_dsv3_decode_kernel_trace.md"),
-    "c7_w8a8_zipf": (3_089_500_000, "profiles/moe_layer_w8a8_zipf_kernel_trace.md"),
-    "c7_w8a8_zipf_4096": (8_312_500_000, "profiles/moe_layer_w8a8_zipf_4096_kernel_trace.md"),
+    "c7_w8a8_zipf": (3_089_300_000, "profiles/moe_layer_w8a8_zipf_kernel_trace.md"),
+    "c7_w8a8_zipf_4096": (8_312_900_000, "profiles/moe_layer_w8a8_zipf_4096_kernel_trace.md"),
 }
 
 
@@ -245,9 +245,10 @@ def run_workload(name, args, lib, torch, np):
             step()
         torch.cuda.synchronize()
         hooked = {"i": 0, "fired": 0}
-        # the launchers of the routed gate_up GEMM (small batches read their rows through a row -> token map)
+        # the launchers of the routed gate_up GEMM (batches past a decode batch read their rows through a
+        # row -> token map, decode batches run in pair order)
         hook_names = (["gmm1_swiglu_quant_w4", "gmm1_swiglu_quant_w4_gather"] if cfg.w4_group >= 0
-                      else ["gmm1_swiglu_quant", "gmm1_swiglu_quant_gather"])
+                      else ["gmm1_swiglu_quant", "gmm1_swiglu_quant_gather", "gmm1_swiglu_quant_pairs"])
         origs = {h: getattr(K, h) for h in hook_names}
 
         def make_timed(orig, routed):
@@ -264,7 +265,7 @@ def run_workload(name, args, lib, torch, np):
             return timed_gmm1
 
         for h in hook_names:
-            setattr(K, h, make_timed(origs[h], (lambda x_: True) if h.endswith("gather")
+            setattr(K, h, make_timed(origs[h], (lambda x_: True) if h.endswith(("gather", "pairs"))
                                      else (lambda x_: x_.shape[0] == R)))
         try:
             torch.cuda.synchronize()

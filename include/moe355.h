@@ -416,6 +416,36 @@ int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorte
                            const void *residual, void *out, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Pair order: the expert MLP of a decode batch without a sorted activation.
+ * No counterpart of their own in the reference: together with moe355_gate_quant they compute what
+ * torch.ops._C_ascend.moe_gating_top_k + torch_npu.npu_moe_init_routing_v2 + grouped_matmul_swiglu_quant +
+ * npu_grouped_matmul + npu_moe_token_unpermute compute (vllm_ascend/ops/fused_moe/routed_experts.py:496-609,
+ * moe_mlp.py:174-570, token_dispatcher.py:367-461), bit for bit, for at most 1024 (token, slot) pairs
+ * (moe355_gmm_pairs_supported() != 0) whose ids all lie in [0, num_experts).  The sort of the pairs by expert,
+ * which for such a batch is a hand-off between workgroups through memory in front of the first weight request,
+ * disappears: row f = token * top_k + slot of every intermediate tensor belongs to pair f, a workgroup of the
+ * weight-streaming GEMM collects the pairs of its expert from topk_ids itself, and the combine reads the k rows of
+ * a token where they lie.  A pair whose id is out of range is computed by nobody: its rows are left untouched.
+ *   gmm1: x int8 [T, K] and x_scale [T] in token order (moe355_gate_quant) -> out int8 [T*k, N/2], out_scale [T*k]
+ *   gmm2: x int8 [T*k, K], per_token_scale [T*k] -> out bf16 / fp16 [T*k, N]
+ *   unpermute: out[t] = sum over the slots of token t, in slot order, of probs[t, s] * rows[t*k + s] (+ residual),
+ *   the arithmetic of moe355_token_unpermute; expert_tokens [num_experts] int64 receives the number of pairs of
+ *   every expert (what moe355_init_routing returns as counts), counted by one more workgroup of the same launch.
+ *   num_experts <= 2048. */
+int moe355_gmm_pairs_supported(int64_t num_tokens, int top_k, int64_t n, int64_t k);
+size_t moe355_gmm1_swiglu_quant_pairs_workspace(int64_t num_tokens, int top_k, int64_t n);
+int moe355_gmm1_swiglu_quant_pairs(const int8_t *x, const float *x_scale, const int32_t *topk_ids, int64_t num_tokens,
+                                   int top_k, const int8_t *weight_nz, const float *weight_scale, int64_t k,
+                                   int64_t n, int num_experts, float swiglu_limit, int8_t *out, float *out_scale,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+int moe355_gmm2_dequant_pairs(const int8_t *x, const int8_t *weight_nz, const float *scale,
+                              const float *per_token_scale, const int32_t *topk_ids, int64_t num_tokens, int top_k,
+                              int64_t k, int64_t n, int num_experts, void *out, int out_dtype, void *stream);
+int moe355_token_unpermute_pairs(const void *rows, int dtype, const void *probs, const int32_t *topk_ids,
+                                 int64_t num_tokens, int top_k, int64_t hidden, int num_experts, const void *residual,
+                                 void *out, int64_t *expert_tokens, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement hook (no counterpart in the reference; for benchmarks).  The one piece of per-thread host
  * state in the library: the armed pair of events is kept in thread-local storage until the next GEMM launch
  * of the same thread takes it.

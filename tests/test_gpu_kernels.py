@@ -957,3 +957,45 @@ def test_grouped_gemms_on_random_problems(K, orc, seed):
     torch.cuda.synchronize()
     assert np.array_equal(q.cpu().numpy(), q_want)
     assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
+# The expert MLP of a decode batch in pair order (no sort): every stage against the sorted form of the checker,
+# rows moved to pair order through the checker's own expanded_row_idx.
+@pytest.mark.parametrize("T,k,E,H,I", [(64, 8, 128, 2048, 768), (8, 8, 128, 2048, 768), (1, 1, 8, 64, 32),
+                                       (128, 8, 64, 512, 128), (33, 6, 96, 256, 96), (64, 8, 256, 1024, 256),
+                                       (100, 4, 256, 128, 64), (300, 2, 16, 192, 160)])
+def test_expert_mlp_in_pair_order(K, orc, T, k, E, H, I):
+    from vllm_ascend_amd._lib import W_ENK
+
+    print(f"pair order T={T} k={k} E={E} H={H} I={I}", flush=True)
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if E >= 8:
+        ids[:, 0] = ids[0, 0]  # one popular expert: more than 32 rows (several passes) when T allows
+    tw = torch.rand(T, k, generator=g).to(torch.bfloat16)
+    w13 = torch.randint(-128, 128, (E, 2 * I, H), generator=g, dtype=torch.int8)
+    w2 = torch.randint(-128, 128, (E, H, I), generator=g, dtype=torch.int8)
+    s13 = torch.rand(E, 2 * I, generator=g) * 0.009 + 0.001
+    s2 = torch.rand(E, H, generator=g) * 0.009 + 0.001
+    # checker, sorted form
+    xs_o, dst_o, cnt_o, sx_o = orc.init_routing(bits(x), ids.numpy(), E, quant=True)
+    cum = np.cumsum(cnt_o)
+    acc1 = orc.gmm_i32(xs_o, w13.numpy(), cum)
+    q1_o, s1_o = orc.swiglu_quant(orc.dequant_acc(acc1, sx_o, s13.numpy(), cum))
+    acc2 = orc.gmm_i32(q1_o, w2.numpy(), cum)
+    y2_o = orc.gmm2_dequant(acc2, s1_o, s2.numpy(), cum)
+    out_o = orc.unpermute(y2_o, dst_o, bits(tw))
+    # GPU, pair order
+    xq, xsc = K.dynamic_quant(x.to(DEV))
+    w13nz, w2nz = K.format_cast_nz(w13.to(DEV), W_ENK), K.format_cast_nz(w2.to(DEV), W_ENK)
+    q1, s1 = K.gmm1_swiglu_quant_pairs(xq, xsc, ids.to(DEV), w13nz, s13.to(DEV), 2 * I, H)
+    y2 = K.gmm2_dequant_pairs(q1, w2nz, s2.to(DEV), s1, ids.to(DEV), H, I)
+    out, cnt = K.token_unpermute_pairs(y2, tw.to(DEV), ids.to(DEV), E)
+    torch.cuda.synchronize()
+    dst = dst_o.astype(np.int64)
+    assert np.array_equal(q1.cpu().numpy(), q1_o[dst])
+    assert np.array_equal(s1.cpu().numpy().view(np.uint32), s1_o[dst].view(np.uint32))
+    assert np.array_equal(bits(y2.cpu()), y2_o[dst])
+    assert np.array_equal(bits(out.cpu()), out_o)
+    assert np.array_equal(cnt.cpu().numpy(), cnt_o)

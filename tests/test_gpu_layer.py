@@ -11,9 +11,10 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-# fused: small batches take the four-launch form (gating + dispatch in one kernel) unless it is switched off;
-# c3_small (2560 pairs) is beyond it either way
-@pytest.mark.parametrize("fused", [True, False])
+# fused: batches of at most 1024 pairs run in pair order (nothing sorted: gating + quantisation, the GEMMs collect
+# their pairs themselves); "sorted": the form before it, gating + dispatch in one kernel and GEMMs on the sorted
+# order; False: op by op.  c3_small (2560 pairs) is beyond the first two either way
+@pytest.mark.parametrize("fused", [True, "sorted", False])
 @pytest.mark.parametrize("name", ["c1_tiny", "c2_small", "c3_small", "c4_small", "c7_small", "c2_qwen3_decode"])
 def test_layer_bit_exact(name, fused):
     from oracle import oracle as orc
@@ -22,7 +23,8 @@ def test_layer_bit_exact(name, fused):
     print(f"layer {name} fused={fused}", flush=True)
     d = make_layer(cfg, seed=0)
     layer = build_layer(cfg, d, DEV)
-    layer.use_fused_small_batch = fused
+    layer.use_fused_small_batch = bool(fused)
+    layer.use_pair_order = fused is True
     takes_fused = layer.quant_method.supports_small_batch(layer, d["x"].to(DEV), d["logits"].to(DEV), layer.router)
     assert takes_fused  # every plain W8A8 call has a router-fused form (one launch up to 1024 pairs)
     x, logits = d["x"].to(DEV), d["logits"].to(DEV)

@@ -83,6 +83,15 @@ PROTOTYPES = {
     "moe355_act_mul_quant": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int64, c_int64, c_int, c_float,
                                      c_float, c_float, c_void_p, c_void_p, c_void_p]),
     "moe355_silu_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "moe355_gmm_pairs_supported": (c_int, [c_int64, c_int, c_int64, c_int64]),
+    "moe355_gmm1_swiglu_quant_pairs_workspace": (c_size_t, [c_int64, c_int, c_int64]),
+    "moe355_gmm1_swiglu_quant_pairs": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int64,
+                                               c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p, c_size_t,
+                                               c_void_p]),
+    "moe355_gmm2_dequant_pairs": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
+                                          c_int64, c_int, c_void_p, c_int, c_void_p]),
+    "moe355_token_unpermute_pairs": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int,
+                                             c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe355_profile_next_gemm": (c_int, [c_void_p, c_void_p]),
     "moe355_gmm_kernel_name": (c_char_p, [c_int, c_int64, c_int64, c_int64, c_int]),
     "moe355_token_unpermute": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p,

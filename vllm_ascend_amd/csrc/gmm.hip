@@ -55,11 +55,21 @@ __global__ __launch_bounds__(256) void format_cast_nz_kernel(const int8_t* __res
 // has rows, and the lookup hides behind the HBM latency).  A launch that covers only some of the experts of a
 // large batch reads the group list first: a unit whose expert is empty or belongs to the other kernel of the call
 // would otherwise fetch 32 KiB for nothing, times thousands of units.
-template <int EPI, int KSPLIT, int UN, int OCC, bool SLABS = false, bool EARLY = true>
+// PAIRS: the rows of an expert are not a range of a sorted activation but the (token, slot) pairs that chose it,
+// found here from the ids of all pairs (at most 1024: a decode batch).  The four wavefronts of a workgroup work on
+// one expert (KSPLIT == 1: four units of it; the host picks that form only when the units of an expert come in
+// fours), scan a quarter of the ids each and leave the expert's pairs, in ascending order, in LDS.  The routing
+// launch in front of the GEMM then is gating and quantisation only: no sort, no hand-off between workgroups.
+constexpr int kPairMax = 1024;
+
+template <int EPI, int KSPLIT, int UN, int OCC, bool SLABS = false, bool EARLY = true, bool PAIRS = false>
 __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
 {
     static_assert(KSPLIT == 1 || KSPLIT == 4, "workgroup barriers need all four wavefronts on one unit");
+    static_assert(!PAIRS || (!SLABS && EARLY && EPI != EPI_I32), "pair order: the two GEMMs of a decode layer");
     __shared__ int32_t red[(KSPLIT > 1) ? 32 * 64 : 1];
+    __shared__ uint16_t plist[PAIRS ? kPairMax : 1];
+    __shared__ int32_t pcount[4];
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int NB = a.N >> 5, KB = a.K >> 5;
@@ -105,11 +115,42 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     };
     if constexpr (EARLY) load_weights(kb_begin);
 
-    int64_t row0, row1;
-    expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
-    if (!expert_in_launch(a, row1 - row0)) return;  // another kernel of this operator call covers the expert
-    if (row1 > a.R) row1 = a.R;
-    if (row1 <= row0) return;
+    int64_t row0 = 0, row1 = 0;
+    if constexpr (PAIRS) {
+        // wavefront w scans pairs [w Q, (w + 1) Q), Q a multiple of 64 and at most 256
+        const int R = (int)a.R;
+        const int Q = ((R + 255) >> 8) << 6;
+        const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+        bool mine[4];
+        int cnt = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int f = wave * Q + c * 64 + lane;
+            mine[c] = c * 64 < Q && f < R && a.pair_ids[f] == e;
+            cnt += __popcll(__ballot(mine[c]));
+        }
+        if (lane == 0) pcount[wave] = cnt;
+        __syncthreads();
+        int base = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) base += pcount[w];
+            row1 += pcount[w];
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const unsigned long long m = __ballot(mine[c]);
+            if (mine[c]) plist[base + __popcll(m & below)] = (uint16_t)(wave * Q + c * 64 + lane);
+            base += __popcll(m);
+        }
+        __syncthreads();
+        if (row1 == 0) return;  // the whole workgroup: nobody chose this expert
+    } else {
+        expert_rows(a.gl, a.gl_type, e, lane, row0, row1);
+        if (!expert_in_launch(a, row1 - row0)) return;  // another kernel of this operator call covers the expert
+        if (row1 > a.R) row1 = a.R;
+        if (row1 <= row0) return;
+    }
     if constexpr (!EARLY) load_weights(kb_begin);
 
     const int tok = lane & 31;
@@ -138,12 +179,18 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     if constexpr (KSPLIT > 1) load_channel_scales(0);
 
     for (int64_t r0 = row0; r0 < row1; r0 += 32) {
-        const int64_t row = r0 + tok;
-        const bool valid = row < row1;
-        const int64_t src = a.row_src ? (int64_t)a.row_src[valid ? row : row0] : row;  // where the row's values lie
+        const bool valid = r0 + tok < row1;
+        int64_t row, src;  // where the row's result goes, where its values lie
+        if constexpr (PAIRS) {
+            row = plist[valid ? r0 + tok : 0];
+            src = a.pair_gather ? row / a.pair_k : row;
+        } else {
+            row = r0 + tok;
+            src = a.row_src ? (int64_t)a.row_src[valid ? row : row0] : row;
+        }
         const int8_t* xr = a.x + src * a.K + kh * 16;
         float rs = 0.0f;
-        if constexpr (EPI != EPI_I32) rs = a.row_scale[a.row_src ? src : (valid ? row : row0)];
+        if constexpr (EPI != EPI_I32) rs = a.row_scale[(PAIRS || a.row_src) ? src : (valid ? row : row0)];
         v16i c0 = {0}, c1 = {0};
         if (r0 != row0) load_weights(kb_begin);
         for (int kb = kb_begin; kb < kb_end; kb += UN) {
@@ -228,9 +275,11 @@ __global__ __launch_bounds__(256) void swiglu_requant_kernel(const float* __rest
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (row >= R) return;
-    int64_t r0, total;
-    expert_rows(gl, gl_type, E - 1, lane, r0, total);
-    if (row >= total) return;
+    if (gl) {  // without a group list (pair order) every row is a row of some expert
+        int64_t r0, total;
+        expert_rows(gl, gl_type, E - 1, lane, r0, total);
+        if (row >= total) return;
+    }
     const v4f* yr = (const v4f*)(y + row * I);
     const int nvec = I >> 2;
     float amax = 0.0f;
@@ -748,4 +797,98 @@ extern "C" int moe355_gmm2_dequant_list(const int8_t* x, const int8_t* const* we
     if (!weight_nz_list || !scale_list) return MOE355_E_ARG;
     return gmm2_impl(x, nullptr, weight_nz_list, nullptr, scale_list, per_token_scale, group_list, group_list_type,
                      rows, k, n, num_experts, out, out_dtype, workspace, workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------------ pair order (decode batches)
+extern "C" int moe355_gmm_pairs_supported(int64_t num_tokens, int top_k, int64_t n, int64_t k)
+{
+    return num_tokens > 0 && top_k > 0 && num_tokens * top_k <= kPairMax && n > 0 && k > 0 && n % 64 == 0 && k % 32 == 0;
+}
+
+extern "C" size_t moe355_gmm1_swiglu_quant_pairs_workspace(int64_t num_tokens, int top_k, int64_t n)
+{
+    if (num_tokens <= 0 || top_k <= 0 || n <= 0) return 256;
+    return (((size_t)num_tokens * top_k * (size_t)(n / 2) * 4 + 255) & ~(size_t)255);
+}
+
+extern "C" int moe355_gmm1_swiglu_quant_pairs(const int8_t* x, const float* x_scale, const int32_t* topk_ids,
+                                              int64_t num_tokens, int top_k, const int8_t* weight_nz,
+                                              const float* weight_scale, int64_t k, int64_t n, int num_experts,
+                                              float swiglu_limit, int8_t* out, float* out_scale, void* workspace,
+                                              size_t workspace_bytes, void* stream)
+{
+    if (num_tokens < 0 || top_k <= 0 || k <= 0 || n <= 0 || num_experts <= 0) return MOE355_E_ARG;
+    if (num_tokens == 0) return MOE355_OK;
+    if (!moe355_gmm_pairs_supported(num_tokens, top_k, n, k)) return MOE355_E_SHAPE;
+    if ((int64_t)num_experts * (n / 64) >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (!x || !x_scale || !topk_ids || !weight_nz || !weight_scale || !out || !out_scale) return MOE355_E_ARG;
+    if (((uintptr_t)x & 15) || ((uintptr_t)weight_nz & 15) || ((uintptr_t)weight_scale & 15) || ((uintptr_t)out & 3))
+        return MOE355_E_SHAPE;
+    if (!workspace || ((uintptr_t)workspace & 255) ||
+        workspace_bytes < moe355_gmm1_swiglu_quant_pairs_workspace(num_tokens, top_k, n))
+        return MOE355_E_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t rows = num_tokens * top_k;
+    const int I = (int)(n / 2);
+    GmmArgs a = {};
+    a.x = x;
+    a.w = weight_nz;
+    a.R = rows;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    a.row_scale = x_scale;
+    a.ch_scale = weight_scale;
+    a.limit = swiglu_limit;
+    a.y = (float*)workspace;
+    a.pair_ids = topk_ids;
+    a.pair_k = top_k;
+    a.pair_gather = 1;
+    hipEvent_t ev0, ev1;
+    take_profile_events(ev0, ev1);
+    const int64_t units = (int64_t)num_experts * (n / 64);
+    launch_gemm(gmm_stream_kernel<EPI_SWIGLU, 4, 4, 3, false, true, true>, dim3((unsigned)units), st, a, ev0, ev1);
+    launch_swiglu_requant(a.y, nullptr, 0, num_experts, rows, I, out, out_scale, st);
+    return launch_status();
+}
+
+extern "C" int moe355_gmm2_dequant_pairs(const int8_t* x, const int8_t* weight_nz, const float* scale,
+                                         const float* per_token_scale, const int32_t* topk_ids, int64_t num_tokens,
+                                         int top_k, int64_t k, int64_t n, int num_experts, void* out, int out_dtype,
+                                         void* stream)
+{
+    if (num_tokens < 0 || top_k <= 0 || k <= 0 || n <= 0 || num_experts <= 0) return MOE355_E_ARG;
+    if (out_dtype != MOE355_DT_BF16 && out_dtype != MOE355_DT_F16) return MOE355_E_UNSUPPORTED;
+    if (num_tokens == 0) return MOE355_OK;
+    if (!moe355_gmm_pairs_supported(num_tokens, top_k, n, k)) return MOE355_E_SHAPE;
+    if ((int64_t)num_experts * (n / 64) >= 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (!x || !weight_nz || !scale || !per_token_scale || !topk_ids || !out) return MOE355_E_ARG;
+    if (((uintptr_t)x & 15) || ((uintptr_t)weight_nz & 15) || ((uintptr_t)scale & 15) || ((uintptr_t)out & 15))
+        return MOE355_E_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    GmmArgs a = {};
+    a.x = x;
+    a.w = weight_nz;
+    a.R = num_tokens * top_k;
+    a.K = (int)k;
+    a.N = (int)n;
+    a.E = num_experts;
+    a.row_scale = per_token_scale;
+    a.ch_scale = scale;
+    a.out = (uint16_t*)out;
+    a.out_f16 = out_dtype == MOE355_DT_F16;
+    a.pair_ids = topk_ids;
+    a.pair_k = top_k;
+    a.pair_gather = 0;
+    hipEvent_t ev0, ev1;
+    take_profile_events(ev0, ev1);
+    const int64_t units = (int64_t)num_experts * (n / 64);
+    // as the sorted form chooses: a wavefront per unit when there are enough units and K is short, and the units
+    // of an expert come in fours (a workgroup collects the pairs of one expert)
+    if (units >= 2048 && k < 2048 && (n / 64) % 4 == 0)
+        launch_gemm(gmm_stream_kernel<EPI_DEQUANT, 1, 4, 2, false, true, true>, dim3((unsigned)((units + 3) / 4)), st, a,
+                    ev0, ev1);
+    else
+        launch_gemm(gmm_stream_kernel<EPI_DEQUANT, 4, 4, 3, false, true, true>, dim3((unsigned)units), st, a, ev0, ev1);
+    return launch_status();
 }

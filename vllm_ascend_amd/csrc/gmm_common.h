@@ -32,6 +32,12 @@ struct GmmArgs {
     // when set they replace w / ch_scale
     const int8_t* const* w_list;
     const float* const* s_list;
+    // Pair order (small batches, streaming kernel only): no group list and no sorted copy.  pair_ids[f] is the
+    // expert of pair f = token * pair_k + slot; R pairs.  Every workgroup collects the pairs of its expert itself;
+    // row i of the expert is pair f: its values lie in row f / pair_k of x (pair_gather: x and row_scale in token
+    // order) or in row f, and its result goes to row f.
+    const int32_t* pair_ids;
+    int pair_k, pair_gather;
     float limit;            // swiglu clamp
     // A launch may cover only the experts whose row count lies in [rows_min, rows_max] (rows_max 0: no upper
     // bound): a batch with a skewed histogram is split over kernel families by expert, on the device.

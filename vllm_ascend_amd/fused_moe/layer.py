@@ -38,6 +38,9 @@ class AscendRoutedExperts(torch.nn.Module):
         self.log2phy = None
         # small batches (decode): gating and dispatch in one launch when the scheme has the fused form
         self.use_fused_small_batch = True
+        # ... and, for at most 1024 (token, slot) pairs, without sorting them: every intermediate row belongs to a
+        # pair, the GEMMs' workgroups collect the pairs of their expert themselves (W8A8 scheme)
+        self.use_pair_order = True
         specs = dict(quant_method.get_weight(moe_config.num_experts, moe_config.intermediate_size_per_partition,
                                              moe_config.hidden_dim, params_dtype))
         specs.update(quant_method.get_dynamic_quant_param(moe_config.num_experts,

@@ -472,6 +472,88 @@ def token_unpermute(permuted, sorted_indices, probs, residual=None):
     return out
 
 
+# ------------------------------------------------------------------ pair order (decode batches)
+def gmm_pairs_supported(num_tokens: int, top_k: int, n: int, k: int) -> bool:
+    return bool(_lib.load().moe355_gmm_pairs_supported(num_tokens, top_k, n, k))
+
+
+def _check_pair_operands(name, x, x_rows, k, scale_rows, row_scale, topk_ids, weight_nz, n, ch_scale):
+    for t, what in ((x, "x"), (row_scale, "row scale"), (topk_ids, "topk_ids"), (weight_nz, "weight"),
+                    (ch_scale, "scale")):
+        _dev(t, what)
+    E = weight_nz.shape[0]
+    if x.dtype != torch.int8 or x.numel() != x_rows * k:
+        raise ValueError(f"{name}: x must be int8 with {x_rows} rows of {k} values, got {x.dtype} {tuple(x.shape)}")
+    if row_scale.dtype != torch.float32 or row_scale.numel() != scale_rows:
+        raise ValueError(f"{name}: {scale_rows} float32 row scales expected, got {row_scale.dtype} "
+                         f"{tuple(row_scale.shape)}")
+    if topk_ids.dtype != torch.int32:
+        raise TypeError(f"{name}: topk_ids must be int32, got {topk_ids.dtype}")
+    if weight_nz.dtype != torch.int8 or weight_nz.numel() != E * n * k:
+        raise ValueError(f"{name}: weight must be int8 with E x N x K = {E * n * k} values")
+    if ch_scale.dtype != torch.float32 or ch_scale.numel() != E * n:
+        raise ValueError(f"{name}: scale must be float32 with E x N = {E * n} values")
+    return E
+
+
+def gmm1_swiglu_quant_pairs(xq, x_scale, topk_ids, weight_nz, weight_scale, n, k, swiglu_limit=0.0):
+    """gate_up GEMM + SwiGLU + re-quantisation in pair order: xq int8 [T, K] and x_scale [T] in token order,
+    topk_ids [T, top_k] -> (int8 [T*top_k, n/2], fp32 [T*top_k]); row t*top_k + s belongs to slot s of token t."""
+    lib = _lib.load()
+    T, top_k = topk_ids.shape
+    E = _check_pair_operands("gmm1_swiglu_quant_pairs", xq, T, k, T, x_scale, topk_ids, weight_nz, n, weight_scale)
+    dev = xq.device
+    out = torch.empty((T * top_k, n // 2), dtype=torch.int8, device=dev)
+    out_scale = torch.empty((T * top_k,), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.moe355_gmm1_swiglu_quant_pairs_workspace(T, top_k, n), dev)
+    check(lib.moe355_gmm1_swiglu_quant_pairs(_ptr(xq), _ptr(x_scale), _ptr(topk_ids), T, top_k, _ptr(weight_nz),
+                                             _ptr(weight_scale), k, n, E, float(swiglu_limit), _ptr(out),
+                                             _ptr(out_scale), _ptr(ws), ws.numel(), _stream(xq)),
+          "moe355_gmm1_swiglu_quant_pairs")
+    return out, out_scale
+
+
+def gmm2_dequant_pairs(x, weight_nz, scale, per_token_scale, topk_ids, n, k, out_dtype=torch.bfloat16):
+    """down GEMM + dequant in pair order: x int8 [T*top_k, K], per_token_scale [T*top_k] -> [T*top_k, n]."""
+    lib = _lib.load()
+    T, top_k = topk_ids.shape
+    E = _check_pair_operands("gmm2_dequant_pairs", x, T * top_k, k, T * top_k, per_token_scale, topk_ids, weight_nz, n,
+                             scale)
+    out = torch.empty((T * top_k, n), dtype=_half_dtype(out_dtype), device=x.device)
+    check(lib.moe355_gmm2_dequant_pairs(_ptr(x), _ptr(weight_nz), _ptr(scale), _ptr(per_token_scale), _ptr(topk_ids),
+                                        T, top_k, k, n, E, _ptr(out), _dt(out, "out"), _stream(x)),
+          "moe355_gmm2_dequant_pairs")
+    return out
+
+
+def token_unpermute_pairs(rows, probs, topk_ids, num_experts, residual=None):
+    """Weighted sum of the top_k rows of every token, rows in pair order.  -> (out [T, H], expert_tokens [E] int64
+    counts of the pairs of every expert)."""
+    rows = _dev(rows, "rows")
+    probs = _dev(probs, "probs")
+    topk_ids = _dev(topk_ids, "topk_ids")
+    if topk_ids.dtype != torch.int32:
+        raise TypeError(f"topk_ids must be int32, got {topk_ids.dtype}")
+    if probs.dtype != rows.dtype:
+        probs = probs.to(rows.dtype)
+    T, k = probs.shape
+    H = rows.shape[1]
+    if rows.shape[0] != T * k or tuple(topk_ids.shape) != (T, k):
+        raise ValueError(f"rows {tuple(rows.shape)} / topk_ids {tuple(topk_ids.shape)} do not match {T} x {k} pairs")
+    if residual is not None:
+        residual = _dev(residual, "residual")
+        if residual.dtype != rows.dtype or tuple(residual.shape) != (T, H):
+            raise ValueError(f"residual must be {rows.dtype} of shape {(T, H)}, got {residual.dtype} "
+                             f"{tuple(residual.shape)}")
+    lib = _lib.load()
+    out = torch.empty((T, H), dtype=rows.dtype, device=rows.device)
+    tokens = torch.empty((num_experts,), dtype=torch.int64, device=rows.device)
+    check(lib.moe355_token_unpermute_pairs(_ptr(rows), _dt(rows, "rows"), _ptr(probs), _ptr(topk_ids), T, k, H,
+                                           num_experts, _ptr(residual), _ptr(out), _ptr(tokens), _stream(rows)),
+          "moe355_token_unpermute_pairs")
+    return out, tokens
+
+
 # ------------------------------------------------------------------ W4A8 (int4 weights)
 def format_cast_nz_int4(w: torch.Tensor, source: int, n: int, k: int) -> torch.Tensor:
     """source 0: int8 [E, N, K] with one int4 value per byte; source 1: packed bytes [E, K, N/2]

@@ -189,6 +189,9 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         Same results, bit for bit, as ``router.select_experts`` followed by ``apply``
         (``vllm_ascend/ops/fused_moe/routed_experts.py:496-609``, ``w8a8_dynamic.py:224-301``)."""
         before_dispatch_evt = torch.cuda.current_stream().record_event()
+        if self._pair_order(layer, x, router_logits, router):
+            return self._experts_in_pair_order(layer, x, router_logits, router, shared_experts, shared_experts_input,
+                                               before_dispatch_evt)
         topk_weights, topk_ids, xq, x_scale, expanded_row_idx, row_token, expert_tokens = \
             route_and_quantize(layer, x, router_logits, router)
         shared_out = None
@@ -199,6 +202,64 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
                 shared_out = shared_experts(shared_experts_input)
         return self._experts_on_row_map(layer, x, xq, x_scale, row_token, expanded_row_idx, expert_tokens,
                                         topk_weights, shared_experts, shared_out, before_dispatch_evt)
+
+    # ------------------------------------------------------------------ decode batches: no sort at all
+    @staticmethod
+    def _pair_order(layer, x: torch.Tensor, router_logits: torch.Tensor, router) -> bool:
+        """At most 1024 (token, slot) pairs that the grouped GEMMs would stream the weights for anyway, ids
+        straight from the gate (always in range)."""
+        from .. import kernels
+
+        if getattr(layer, "log2phy", None) is not None or not getattr(layer, "use_pair_order", True):
+            return False
+        T, k, E = x.shape[0], router.top_k, router_logits.shape[1]
+        w13, w2 = layer.w13_weight, layer.w2_weight
+        if not (kernels.gmm_pairs_supported(T, k, w13.shape[2], w13.shape[1])
+                and kernels.gmm_pairs_supported(T, k, w2.shape[2], w2.shape[1])):
+            return False
+        if not kernels.gate_quant_supported(T, k, E) or E > 2048:
+            return False
+        return T * k < 1024 or (T * k) // E < 12  # where the sorted form streams as well (csrc/gmm.hip: tiled_bm)
+
+    def _experts_in_pair_order(self, layer, x, router_logits, router, shared_experts, shared_experts_input,
+                               before_dispatch_evt):
+        """Five launches and no hand-off between workgroups: gating + token quantisation, the gate_up GEMM (its
+        workgroups collect the pairs of their expert from the ids themselves), the re-quantisation, the down GEMM,
+        and the combine, which also counts the pairs per expert.  Every intermediate row t * k + s belongs to slot
+        s of token t; nothing is sorted.  Same results, bit for bit, as the sorted form."""
+        from .. import kernels
+        from ..fused_moe.contracts import FusedExpertsResult
+
+        stream = torch.cuda.current_stream()
+        bias = router.e_score_correction_bias
+        if bias is not None and bias.dtype != router_logits.dtype:
+            bias = router.e_score_correction_bias = bias.to(router_logits.dtype)
+        topk_weights, topk_ids, xq, x_scale = kernels.gate_quant(
+            x, router_logits, router.top_k, router.topk_group if router.topk_group is not None else 1,
+            router.num_expert_group if router.num_expert_group is not None else 1, 1, int(router.renormalize),
+            0 if router.scoring_func == "softmax" else 1, router.routed_scaling_factor, 1e-20, bias)
+        shared_out = None
+        if shared_experts is not None:
+            if shared_experts_input is None:
+                shared_out = shared_experts(x, quantized=(xq, x_scale))
+            else:
+                shared_out = shared_experts(shared_experts_input)
+        w13, w2 = layer.w13_weight, layer.w2_weight
+        cfg = getattr(layer, "moe_config", None)
+        swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
+        q1, q1_scale = kernels.gmm1_swiglu_quant_pairs(xq, x_scale, topk_ids, w13, layer.w13_weight_scale_fp32,
+                                                       w13.shape[2], w13.shape[1], swiglu_limit)
+        before_gmm2_evt = stream.record_event()
+        out = kernels.gmm2_dequant_pairs(q1, w2, layer.w2_weight_scale_fp32, q1_scale, topk_ids, w2.shape[2],
+                                         w2.shape[1], out_dtype=x.dtype)
+        before_combine_evt = stream.record_event()
+        if shared_experts is not None and shared_out is not None:
+            shared_experts.wait()
+        routed_out, expert_tokens = kernels.token_unpermute_pairs(out, topk_weights, topk_ids, router_logits.shape[1],
+                                                                  shared_out)
+        return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
+                                  before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
+                                  group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
 
     @staticmethod
     def get_eplb_weight_views(layer) -> list:
