@@ -113,20 +113,28 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
             }
         }
     };
+    // pair order: wavefront w scans pairs [w Q, (w + 1) Q), Q a multiple of 64 and at most 256.  The ids are
+    // requested in front of the weights: answers come back in the order of the requests, and the list of the
+    // expert's pairs (which the token loads wait for) should not queue behind the first weight tiles from HBM.
+    const int Q = PAIRS ? (((int)a.R + 255) >> 8) << 6 : 0;
+    int pid[PAIRS ? 4 : 1];
+    if constexpr (PAIRS) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int f = wave * Q + c * 64 + lane;
+            pid[c] = (c * 64 < Q && f < (int)a.R) ? a.pair_ids[f] : -1;
+        }
+    }
     if constexpr (EARLY) load_weights(kb_begin);
 
     int64_t row0 = 0, row1 = 0;
     if constexpr (PAIRS) {
-        // wavefront w scans pairs [w Q, (w + 1) Q), Q a multiple of 64 and at most 256
-        const int R = (int)a.R;
-        const int Q = ((R + 255) >> 8) << 6;
         const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
         bool mine[4];
         int cnt = 0;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const int f = wave * Q + c * 64 + lane;
-            mine[c] = c * 64 < Q && f < R && a.pair_ids[f] == e;
+            mine[c] = pid[c] == e;
             cnt += __popcll(__ballot(mine[c]));
         }
         if (lane == 0) pcount[wave] = cnt;
