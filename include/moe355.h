@@ -425,7 +425,8 @@ int moe355_token_unpermute(const void *permuted, int dtype, const int32_t *sorte
  * which for such a batch is a hand-off between workgroups through memory in front of the first weight request,
  * disappears: row f = token * top_k + slot of every intermediate tensor belongs to pair f, a workgroup of the
  * weight-streaming GEMM collects the pairs of its expert from topk_ids itself, and the combine reads the k rows of
- * a token where they lie.  A pair whose id is out of range is computed by nobody: its rows are left untouched.
+ * a token where they lie.  A pair whose id is out of range is computed by nobody: its rows are left untouched, and
+ * the combine leaves it out of the token's sum and of the counts (a dropped pair, as in the sorted form).
  *   gmm1: x int8 [T, K] and x_scale [T] in token order (moe355_gate_quant) -> out int8 [T*k, N/2], out_scale [T*k]
  *   gmm2: x int8 [T*k, K], per_token_scale [T*k] -> out bf16 / fp16 [T*k, N]
  *   unpermute: out[t] = sum over the slots of token t, in slot order, of probs[t, s] * rows[t*k + s] (+ residual),

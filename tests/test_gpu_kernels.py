@@ -999,3 +999,18 @@ def test_expert_mlp_in_pair_order(K, orc, T, k, E, H, I):
     assert np.array_equal(bits(y2.cpu()), y2_o[dst])
     assert np.array_equal(bits(out.cpu()), out_o)
     assert np.array_equal(cnt.cpu().numpy(), cnt_o)
+    if T >= 8:
+        # dropped pairs (ids outside the range): nobody computes them, the combine and the counts leave them out
+        bad = ids.clone()
+        bad[1, 0], bad[3, k - 1] = E, -1
+        xs_b, dst_b, cnt_b, sx_b = orc.init_routing(bits(x), bad.numpy(), E, quant=True)
+        cum_b = np.cumsum(cnt_b)
+        q1_b, s1_b = orc.swiglu_quant(orc.dequant_acc(orc.gmm_i32(xs_b, w13.numpy(), cum_b), sx_b, s13.numpy(), cum_b))
+        y2_b = orc.gmm2_dequant(orc.gmm_i32(q1_b, w2.numpy(), cum_b), s1_b, s2.numpy(), cum_b)
+        out_b = orc.unpermute(y2_b, dst_b, bits(tw))
+        q1, s1 = K.gmm1_swiglu_quant_pairs(xq, xsc, bad.to(DEV), w13nz, s13.to(DEV), 2 * I, H)
+        y2 = K.gmm2_dequant_pairs(q1, w2nz, s2.to(DEV), s1, bad.to(DEV), H, I)
+        out, cnt = K.token_unpermute_pairs(y2, tw.to(DEV), bad.to(DEV), E)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out.cpu()), out_b)
+        assert np.array_equal(cnt.cpu().numpy(), cnt_b)

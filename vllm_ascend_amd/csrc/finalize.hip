@@ -43,6 +43,10 @@ __global__ __launch_bounds__(256) void token_unpermute_kernel(const uint16_t* __
     if (threadIdx.x < top_k) {
         int32_t d = idx ? idx[t * top_k + threadIdx.x] : (int32_t)(t * top_k + threadIdx.x);
         d = d < 0 ? -d : d;
+        if (!idx && hist_ids) {  // pair order: a pair whose expert id is out of range was computed by nobody
+            const int32_t e = hist_ids[t * top_k + threadIdx.x];
+            if (e < 0 || e >= hist_experts) d = 0x7fffffff;
+        }
         srow[threadIdx.x] = ((int64_t)d < permuted_rows) ? d : -1;
         sw[threadIdx.x] = probs ? half_to_f32<DT>(probs[t * top_k + threadIdx.x]) : 1.0f;
     }
