@@ -324,7 +324,7 @@ def test_expert_load_collection(fused):
 
 
 @pytest.mark.parametrize("name", ["c2_small", "c5_small"])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, "sorted", False])
 def test_redundant_experts_through_log2phy(name, fused):
     """Two physical copies of logical experts behind the logical -> physical map: the router scores the logical
     experts, the dispatch runs over the physical ones, the output is the one of the layer without copies, and
@@ -336,7 +336,8 @@ def test_redundant_experts_through_log2phy(name, fused):
     plain = build_layer(cfg, d, DEV)
     want = plain.forward_impl(x, logits)
     layer = build_layer(cfg, d, DEV, redundant=(3, 1))
-    layer.use_fused_small_batch = fused
+    layer.use_fused_small_batch = bool(fused)
+    layer.use_pair_order = fused is True
     log2phy = torch.arange(cfg.E, dtype=torch.int32, device=DEV)
     log2phy[3] = cfg.E  # every token of logical expert 3 goes to its copy; the copy of expert 1 stays idle
     layer.log2phy = log2phy

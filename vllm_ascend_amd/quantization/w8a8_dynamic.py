@@ -210,16 +210,17 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         straight from the gate (always in range)."""
         from .. import kernels
 
-        if getattr(layer, "log2phy", None) is not None or not getattr(layer, "use_pair_order", True):
+        if not getattr(layer, "use_pair_order", True):
             return False
         T, k, E = x.shape[0], router.top_k, router_logits.shape[1]
         w13, w2 = layer.w13_weight, layer.w2_weight
         if not (kernels.gmm_pairs_supported(T, k, w13.shape[2], w13.shape[1])
                 and kernels.gmm_pairs_supported(T, k, w2.shape[2], w2.shape[1])):
             return False
-        if not kernels.gate_quant_supported(T, k, E) or E > 2048:
+        experts = layer.w13_weight.shape[0]  # physical experts (more than E with redundant copies behind log2phy)
+        if not kernels.gate_quant_supported(T, k, E) or experts > 2048:
             return False
-        return T * k < 1024 or (T * k) // E < 12  # where the sorted form streams as well (csrc/gmm.hip: tiled_bm)
+        return T * k < 1024 or (T * k) // experts < 12  # where the sorted form streams as well (csrc/gmm.hip: tiled_bm)
 
     def _experts_in_pair_order(self, layer, x, router_logits, router, shared_experts, shared_experts_input,
                                before_dispatch_evt):
@@ -238,6 +239,11 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
             x, router_logits, router.top_k, router.topk_group if router.topk_group is not None else 1,
             router.num_expert_group if router.num_expert_group is not None else 1, 1, int(router.renormalize),
             0 if router.scoring_func == "softmax" else 1, router.routed_scaling_factor, 1e-20, bias)
+        log2phy = getattr(layer, "log2phy", None)
+        if log2phy is not None:
+            # logical -> physical expert ids (redundant experts of dynamic load balancing,
+            # vllm_ascend/ops/fused_moe/routed_experts.py:452-453): the experts run over the physical ones
+            topk_ids = log2phy[topk_ids.long()].to(torch.int32)
         shared_out = None
         if shared_experts is not None:
             if shared_experts_input is None:
@@ -255,8 +261,7 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         before_combine_evt = stream.record_event()
         if shared_experts is not None and shared_out is not None:
             shared_experts.wait()
-        routed_out, expert_tokens = kernels.token_unpermute_pairs(out, topk_weights, topk_ids, router_logits.shape[1],
-                                                                  shared_out)
+        routed_out, expert_tokens = kernels.token_unpermute_pairs(out, topk_weights, topk_ids, w13.shape[0], shared_out)
         return FusedExpertsResult(routed_out=routed_out, before_dispatch_evt=before_dispatch_evt,
                                   before_gmm2_evt=before_gmm2_evt, before_combine_evt=before_combine_evt,
                                   group_list_type=1, expert_tokens=expert_tokens, shared_out=shared_out)
