@@ -248,7 +248,7 @@ def run_workload(name, args, lib, torch, np):
         # the launchers of the routed gate_up GEMM (batches past a decode batch read their rows through a
         # row -> token map, decode batches run in pair order)
         hook_names = (["gmm1_swiglu_quant_w4", "gmm1_swiglu_quant_w4_gather"] if cfg.w4_group >= 0
-                      else ["gmm1_swiglu_quant", "gmm1_swiglu_quant_gather", "gmm1_swiglu_quant_pairs"])
+                      else ["gmm1_swiglu_quant", "gmm1_swiglu_quant_gather", "gmm1_swiglu_quant_pairs", "gmm1_swiglu_pairs"])
         origs = {h: getattr(K, h) for h in hook_names}
 
         def make_timed(orig, routed):

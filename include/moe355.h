@@ -442,6 +442,19 @@ int moe355_gmm1_swiglu_quant_pairs(const int8_t *x, const float *x_scale, const 
 int moe355_gmm2_dequant_pairs(const int8_t *x, const int8_t *weight_nz, const float *scale,
                               const float *per_token_scale, const int32_t *topk_ids, int64_t num_tokens, int top_k,
                               int64_t k, int64_t n, int num_experts, void *out, int out_dtype, void *stream);
+/* The same two GEMMs with the re-quantisation inside the second: gmm1 leaves the fp32 SwiGLU values y [T*k, N/2],
+ * gmm2 takes them as its activation (K = N/2 of gmm1) and every workgroup quantises the rows of its expert itself
+ * (the arithmetic of the re-quantisation of moe355_gmm1_swiglu_quant), so that a decode layer is four launches.
+ * moe355_gmm2_requant_pairs_supported() != 0: many units of work, a short K (k < 2048, 32 rows of k + 16 bytes
+ * in LDS) and at most three pairs per expert on average -- a small decode batch over many small experts, where a
+ * launch costs more than the repeated quantisation. */
+int moe355_gmm1_swiglu_pairs(const int8_t *x, const float *x_scale, const int32_t *topk_ids, int64_t num_tokens,
+                             int top_k, const int8_t *weight_nz, const float *weight_scale, int64_t k, int64_t n,
+                             int num_experts, float swiglu_limit, float *y, void *stream);
+int moe355_gmm2_requant_pairs_supported(int64_t num_tokens, int top_k, int64_t n, int64_t k, int num_experts);
+int moe355_gmm2_requant_dequant_pairs(const float *y, const int8_t *weight_nz, const float *scale,
+                                      const int32_t *topk_ids, int64_t num_tokens, int top_k, int64_t k, int64_t n,
+                                      int num_experts, void *out, int out_dtype, void *stream);
 int moe355_token_unpermute_pairs(const void *rows, int dtype, const void *probs, const int32_t *topk_ids,
                                  int64_t num_tokens, int top_k, int64_t hidden, int num_experts, const void *residual,
                                  void *out, int64_t *expert_tokens, void *stream);

@@ -961,7 +961,8 @@ def test_grouped_gemms_on_random_problems(K, orc, seed):
 
 # The expert MLP of a decode batch in pair order (no sort): every stage against the sorted form of the checker,
 # rows moved to pair order through the checker's own expanded_row_idx.
-@pytest.mark.parametrize("T,k,E,H,I", [(64, 8, 128, 2048, 768), (8, 8, 128, 2048, 768), (1, 1, 8, 64, 32),
+@pytest.mark.parametrize("T,k,E,H,I", [(64, 8, 128, 2048, 768), (8, 8, 128, 2048, 768), (48, 8, 128, 2048, 768),
+                                       (40, 8, 256, 1024, 256), (1, 1, 8, 64, 32),
                                        (128, 8, 64, 512, 128), (33, 6, 96, 256, 96), (64, 8, 256, 1024, 256),
                                        (100, 4, 256, 128, 64), (300, 2, 16, 192, 160)])
 def test_expert_mlp_in_pair_order(K, orc, T, k, E, H, I):
@@ -999,6 +1000,14 @@ def test_expert_mlp_in_pair_order(K, orc, T, k, E, H, I):
     assert np.array_equal(bits(y2.cpu()), y2_o[dst])
     assert np.array_equal(bits(out.cpu()), out_o)
     assert np.array_equal(cnt.cpu().numpy(), cnt_o)
+    if K.gmm2_requant_pairs_supported(T, k, H, I, E):
+        # the form of four launches: fp32 SwiGLU values out of the first GEMM, re-quantised inside the second
+        _, _, y_o = orc.swiglu_quant(orc.dequant_acc(acc1, sx_o, s13.numpy(), cum), want_y=True)
+        y = K.gmm1_swiglu_pairs(xq, xsc, ids.to(DEV), w13nz, s13.to(DEV), 2 * I, H)
+        y2f = K.gmm2_requant_dequant_pairs(y, w2nz, s2.to(DEV), ids.to(DEV), H, I)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), y_o[dst].view(np.uint32))
+        assert np.array_equal(bits(y2f.cpu()), y2_o[dst])
     if T >= 8:
         # dropped pairs (ids outside the range): nobody computes them, the combine and the counts leave them out
         bad = ids.clone()

@@ -90,6 +90,11 @@ PROTOTYPES = {
                                                c_void_p]),
     "moe355_gmm2_dequant_pairs": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
                                           c_int64, c_int, c_void_p, c_int, c_void_p]),
+    "moe355_gmm1_swiglu_pairs": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64,
+                                         c_int, c_float, c_void_p, c_void_p]),
+    "moe355_gmm2_requant_pairs_supported": (c_int, [c_int64, c_int, c_int64, c_int64, c_int]),
+    "moe355_gmm2_requant_dequant_pairs": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
+                                                  c_int64, c_int, c_void_p, c_int, c_void_p]),
     "moe355_token_unpermute_pairs": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int,
                                              c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe355_profile_next_gemm": (c_int, [c_void_p, c_void_p]),

@@ -38,6 +38,9 @@ struct GmmArgs {
     // order) or in row f, and its result goes to row f.
     const int32_t* pair_ids;
     int pair_k, pair_gather;
+    // pair order, down GEMM with the re-quantisation inside (REQ): the SwiGLU values [R, K] fp32 that the gate_up
+    // GEMM wrote; the workgroup quantises the rows of its expert itself (x and row_scale are not read)
+    const float* y_in;
     float limit;            // swiglu clamp
     // A launch may cover only the experts whose row count lies in [rows_min, rows_max] (rows_max 0: no upper
     // bound): a batch with a skewed histogram is split over kernel families by expert, on the device.

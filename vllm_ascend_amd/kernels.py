@@ -526,6 +526,44 @@ def gmm2_dequant_pairs(x, weight_nz, scale, per_token_scale, topk_ids, n, k, out
     return out
 
 
+def gmm2_requant_pairs_supported(num_tokens: int, top_k: int, n: int, k: int, num_experts: int) -> bool:
+    return bool(_lib.load().moe355_gmm2_requant_pairs_supported(num_tokens, top_k, n, k, num_experts))
+
+
+def gmm1_swiglu_pairs(xq, x_scale, topk_ids, weight_nz, weight_scale, n, k, swiglu_limit=0.0):
+    """gate_up GEMM + SwiGLU in pair order, no re-quantisation: -> fp32 [T*top_k, n/2]."""
+    lib = _lib.load()
+    T, top_k = topk_ids.shape
+    E = _check_pair_operands("gmm1_swiglu_pairs", xq, T, k, T, x_scale, topk_ids, weight_nz, n, weight_scale)
+    y = torch.empty((T * top_k, n // 2), dtype=torch.float32, device=xq.device)
+    check(lib.moe355_gmm1_swiglu_pairs(_ptr(xq), _ptr(x_scale), _ptr(topk_ids), T, top_k, _ptr(weight_nz),
+                                       _ptr(weight_scale), k, n, E, float(swiglu_limit), _ptr(y), _stream(xq)),
+          "moe355_gmm1_swiglu_pairs")
+    return y
+
+
+def gmm2_requant_dequant_pairs(y, weight_nz, scale, topk_ids, n, k, out_dtype=torch.bfloat16):
+    """Re-quantisation + down GEMM + dequant in pair order: y fp32 [T*top_k, K] -> [T*top_k, n]."""
+    lib = _lib.load()
+    y = _dev(y, "y")
+    T, top_k = topk_ids.shape
+    E = weight_nz.shape[0]
+    if y.dtype != torch.float32 or tuple(y.shape) != (T * top_k, k):
+        raise ValueError(f"gmm2_requant_dequant_pairs: y must be float32 {(T * top_k, k)}, got {y.dtype} "
+                         f"{tuple(y.shape)}")
+    if _dev(topk_ids, "topk_ids").dtype != torch.int32:
+        raise TypeError(f"gmm2_requant_dequant_pairs: topk_ids must be int32, got {topk_ids.dtype}")
+    if _dev(weight_nz, "weight").dtype != torch.int8 or weight_nz.numel() != E * n * k:
+        raise ValueError(f"gmm2_requant_dequant_pairs: weight must be int8 with E x N x K = {E * n * k} values")
+    if _dev(scale, "scale").dtype != torch.float32 or scale.numel() != E * n:
+        raise ValueError(f"gmm2_requant_dequant_pairs: scale must be float32 with E x N = {E * n} values")
+    out = torch.empty((T * top_k, n), dtype=_half_dtype(out_dtype), device=y.device)
+    check(lib.moe355_gmm2_requant_dequant_pairs(_ptr(y), _ptr(weight_nz), _ptr(scale), _ptr(topk_ids), T, top_k, k, n,
+                                                E, _ptr(out), _dt(out, "out"), _stream(y)),
+          "moe355_gmm2_requant_dequant_pairs")
+    return out
+
+
 def token_unpermute_pairs(rows, probs, topk_ids, num_experts, residual=None):
     """Weighted sum of the top_k rows of every token, rows in pair order.  -> (out [T, H], expert_tokens [E] int64
     counts of the pairs of every expert)."""

@@ -253,11 +253,20 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         w13, w2 = layer.w13_weight, layer.w2_weight
         cfg = getattr(layer, "moe_config", None)
         swiglu_limit = (getattr(cfg, "swiglu_limit", 0.0) or 0.0) if cfg is not None else 0.0
-        q1, q1_scale = kernels.gmm1_swiglu_quant_pairs(xq, x_scale, topk_ids, w13, layer.w13_weight_scale_fp32,
-                                                       w13.shape[2], w13.shape[1], swiglu_limit)
-        before_gmm2_evt = stream.record_event()
-        out = kernels.gmm2_dequant_pairs(q1, w2, layer.w2_weight_scale_fp32, q1_scale, topk_ids, w2.shape[2],
-                                         w2.shape[1], out_dtype=x.dtype)
+        T, k = topk_ids.shape
+        if kernels.gmm2_requant_pairs_supported(T, k, w2.shape[2], w2.shape[1], w2.shape[0]):
+            # four launches: the down GEMM re-quantises the SwiGLU values of its expert's rows itself
+            y = kernels.gmm1_swiglu_pairs(xq, x_scale, topk_ids, w13, layer.w13_weight_scale_fp32, w13.shape[2],
+                                          w13.shape[1], swiglu_limit)
+            before_gmm2_evt = stream.record_event()
+            out = kernels.gmm2_requant_dequant_pairs(y, w2, layer.w2_weight_scale_fp32, topk_ids, w2.shape[2],
+                                                     w2.shape[1], out_dtype=x.dtype)
+        else:
+            q1, q1_scale = kernels.gmm1_swiglu_quant_pairs(xq, x_scale, topk_ids, w13, layer.w13_weight_scale_fp32,
+                                                           w13.shape[2], w13.shape[1], swiglu_limit)
+            before_gmm2_evt = stream.record_event()
+            out = kernels.gmm2_dequant_pairs(q1, w2, layer.w2_weight_scale_fp32, q1_scale, topk_ids, w2.shape[2],
+                                             w2.shape[1], out_dtype=x.dtype)
         before_combine_evt = stream.record_event()
         if shared_experts is not None and shared_out is not None:
             shared_experts.wait()
