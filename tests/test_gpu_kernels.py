@@ -716,13 +716,14 @@ def test_tiled_gemms_at_tile_boundaries(K, orc, Kd, N):
 
 # Skewed histograms: the host picks a kernel family from the mean rows per expert and, for a large product (a GiB
 # of weights) with 12 to 19 rows per expert on average, the device splits the experts between streaming (up to 32
-# rows: 31 / 32 / 33 sit on the border) and the 128-row tiles.  Small products with the same histogram run on the
-# tiles alone.  The last two cases keep one family (the weight-streaming tiles) over experts far above and below
+# rows: 31 / 32 / 33 sit on the border) and, above it, the weight-streaming tiles (K from 4096 on) or the 128-row
+# tiles.  Small products with the same histogram run on the tiles alone.  The last two cases keep one family (the weight-streaming tiles) over experts far above and below
 # its range: 255 / 256 / 257 / 511 / 513 rows.   name -> (rows per expert, K, N)
 _HOT = [0, 1, 31, 32, 33, 2, 64, 65, 700, 3, 0, 5, 129, 7, 1, 0]
 SKEWED = {
-    "stream+tiled": (_HOT + [12] * 240, 4096, 1024),
-    "stream+tiled, nothing above the border": ([16] * 224 + [32] * 32, 4096, 1024),
+    "stream+wide": (_HOT + [12] * 240, 4096, 1024),
+    "stream+wide, nothing above the border": ([16] * 224 + [32] * 32, 4096, 1024),
+    "stream+tiled": (_HOT + [12] * 240, 2048, 2048),
     "tiled": (_HOT + [12] * 240, 256, 256),
     "wide": ([255, 256, 257, 511, 513, 1, 0, 33, 128, 160, 161, 192, 193, 40, 90, 100], 1024, 256),
     "wide, K 4096": ([300, 20, 256, 257, 47, 150, 0, 90], 4096, 256),
@@ -741,7 +742,10 @@ def test_grouped_gemms_on_skewed_histograms(K, orc, name, gl_type):
     lib = load()
     for epi in (0, 1, 2):
         kn = lib.moe355_gmm_kernel_name(epi, R, Kd, N, E).decode()
-        assert name.split(",")[0].split("+")[0] in kn and ("+ gmm_tiled_kernel" in kn) == ("+" in name)
+        families = name.split(",")[0].split("+")
+        assert families[0] in kn and (" + " in kn) == (len(families) == 2)
+        if len(families) == 2:
+            assert f"+ gmm_{families[1]}_kernel" in kn
     g = torch.Generator().manual_seed(len(counts) + Kd)
     cum = torch.cumsum(cnt, 0)
     gl = (cum if gl_type == 0 else cnt).to(DEV)

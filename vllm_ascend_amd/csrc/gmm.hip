@@ -535,7 +535,14 @@ static GemmPlan gemm_plan(const GmmArgs& a, bool have_tile_ws)
     }
 #endif
     // a large product (a GiB of weights and more) over many experts with few rows on average
-    if (p.bm == 0 && a.R >= 1024 && (int64_t)a.E * a.N * a.K >= (1ll << 30)) p.split = 32;
+    if (p.bm == 0 && a.R >= 1024 && (int64_t)a.E * a.N * a.K >= (1ll << 30)) {
+        p.split = 32;
+        // the experts above the border: weight-streaming tiles when K is long (an expert of up to 256 rows fetches
+        // its weights once), 128-row tiles otherwise.  Measured on 512 tokens of Zipf(1.1) routing at the
+        // DeepSeek-V3 shape: K = 7168 518 against 532 us for the pair of launches, K = 2048 the other way round
+        // by as much; a border of 16 or 64 rows instead of 32 costs 70 / 40 us.
+        if (a.K >= 4096 && a.R / 256 + a.E < 32768) p.split_bm = 256;
+    }
     return p;
 }
 
@@ -658,7 +665,9 @@ extern "C" const char* moe355_gmm_kernel_name(int epilogue, int64_t rows, int64_
     const GemmPlan p = gemm_plan(a, true);  // as launch_gemm_auto decides
     if (p.bm == 256) return "gmm_wide_kernel";
     if (p.bm != 0) return "gmm_tiled_kernel";
-    return p.split ? "gmm_stream_kernel + gmm_tiled_kernel above 32 rows" : "gmm_stream_kernel";
+    if (!p.split) return "gmm_stream_kernel";
+    return p.split_bm == 256 ? "gmm_stream_kernel + gmm_wide_kernel above 32 rows"
+                             : "gmm_stream_kernel + gmm_tiled_kernel above 32 rows";
 }
 
 extern "C" int moe355_format_cast_nz(const int8_t* w, int layout, int64_t num_experts, int64_t n, int64_t k,
