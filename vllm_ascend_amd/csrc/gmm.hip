@@ -487,9 +487,16 @@ static int tiled_bm(const GmmArgs& a)
         // against 1244; under Zipf(1.1) routing at 16 rows on average the tiles win as well (1260 against 1521).
         // Decode batches (fewer than 1024 rows) always stream.
         if (a.R < 1024 || avg < 12) return 0;
-        if (avg >= 20) return 128;
-        // 12..19 rows per expert: large products split the experts between both families (gemm_plan); for small
-        // ones the second launch costs more than it brings and the tiles alone are as fast as streaming
+        // the list of 256-row tiles is built from 16-bit counters (tile_map_kernel, by_length)
+        const bool wide_small = a.K >= 4096 && a.R / 256 + a.E < 32768;
+        // 24..47 rows per expert: tiles.  With a long K the weight-streaming tiles (their one- and two-block forms
+        // for the experts of up to 32 / 64 rows): uniform routing over 256 experts, K = 7168, 24 / 32 / 48 rows
+        // 1255 / 1270 / 1286 us against 1283 / 1305 / 1322 us on the 128-row tiles (streaming 1373 / 1938 / 2706);
+        // at K = 2048 the two kinds of tiles measure the same (664 / 677 / 697 against 664 / 680 / 703).
+        if (avg >= 24) return wide_small ? 256 : 128;
+        // 12..23 rows per expert: large products split the experts between both families (gemm_plan; streaming
+        // alone leads the tiles up to 20 rows at K = 7168 and up to 24 at K = 2048: 612 against 654 us at 20); for
+        // small ones the second launch costs more than it brings and the tiles alone are as fast as streaming
         return (int64_t)a.E * a.N * a.K >= (1ll << 30) ? 0 : 128;
     }
     // the list of 256-row tiles is built from 16-bit counters (tile_map_kernel, by_length)
@@ -503,7 +510,7 @@ static int tiled_bm(const GmmArgs& a)
 
 // What one operator call launches: the family chosen from the mean rows per expert, restricted to the experts it
 // is good at, and (split > 0) the 128-row tiles for the experts above that range.
-//   mean < 20 (12..19 for products of a GiB of weights and more, see tiled_bm) and at least 1024 rows: streaming
+//   mean < 24 (12..23 for products of a GiB of weights and more, see tiled_bm) and at least 1024 rows: streaming
 //     for experts of at most 32 rows (one pass over their weights, and no request before the group list says that
 //     the expert is theirs), tiles for the others -- a 500-row expert would otherwise stream its weights 16 times
 //     while the units of the cold experts have long finished.  Measured at the DeepSeek-V3 shape with Zipf(1.1)
