@@ -300,8 +300,10 @@ def test_gmm1_swiglu_quant_gather(K, orc, R, E, Kd, N, T):
     assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(qs.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
+# up to 4096 pairs of at most 1024 tokens: one launch; beyond: histogram, scan, scatter
 @pytest.mark.parametrize("T,k,E,bad", [(3, 2, 2, False), (64, 8, 128, False), (300, 8, 256, True), (4096, 8, 256, False),
-                                       (1000, 6, 40, True), (2500, 1, 7, False)])
+                                       (1000, 6, 40, True), (2500, 1, 7, False), (512, 8, 256, True), (513, 8, 256, False),
+                                       (1024, 4, 2048, False), (64, 64, 64, False)])
 def test_route_map_equals_init_routing_maps(K, T, k, E, bad):
     """The maps alone (nothing moved) against the ones of the init-routing op; row -> token inverts pair -> row."""
     g = torch.Generator().manual_seed(T + 5 * k + E)

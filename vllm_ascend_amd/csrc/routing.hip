@@ -322,6 +322,62 @@ __global__ __launch_bounds__(256) void route_gather_small_kernel(const int32_t* 
     gather_token_row<QUANT, DT>(x + (int64_t)t * H, H, top_k, drow, lds4, xs, sx, held);
 }
 
+// The index maps alone for at most 4096 pairs, in ONE launch of num_tokens + 1 workgroups: workgroup t finds the
+// destinations of its token's k pairs by counting (as above) and writes them and the row -> token map; the last
+// workgroup the per-expert counts.  Nobody waits for anybody.
+constexpr int kMapSmallIters = 16;  // 16 * 256 = 4096 pairs
+
+__global__ __launch_bounds__(256) void route_map_small_kernel(const int32_t* __restrict__ ids, int R, int E,
+                                                              int tokens_num_type, int32_t* __restrict__ off,
+                                                              int64_t* __restrict__ expert_tokens,
+                                                              int32_t* __restrict__ dst, int32_t* __restrict__ row_token,
+                                                              int top_k)
+{
+    extern __shared__ int32_t sm[];  // the counting workgroup: [E] counts, [256] scan scratch
+    __shared__ int32_t wsum[4][64];
+    const int num_tokens = (int)gridDim.x - 1;
+    if ((int)blockIdx.x == num_tokens) {
+        small_hist_scan(ids, R, E, tokens_num_type, off, expert_tokens, sm);
+        return;
+    }
+    const int t = blockIdx.x;
+    const int tid = threadIdx.x;
+    int my_e[kMapSmallIters];
+#pragma unroll
+    for (int it = 0; it < kMapSmallIters; ++it) {
+        const int f = it * 256 + tid;
+        int e = kInvalidExpert;
+        if (f < R) {
+            e = ids[f];
+            if (e < 0 || e >= E) e = kInvalidExpert;
+        }
+        my_e[it] = e;
+    }
+    const int iters = (R + 255) >> 8;
+    for (int j = 0; j < top_k; ++j) {
+        const int fj = t * top_k + j;
+        const int ej = ids[fj];
+        int c = 0;
+#pragma unroll
+        for (int it = 0; it < kMapSmallIters; ++it) {
+            if (it < iters) {
+                const int f = it * 256 + tid;
+                c += (my_e[it] < ej || (my_e[it] == ej && f < fj)) ? 1 : 0;
+            }
+        }
+        c = wave_sum_i32(c);
+        if ((tid & 63) == 0) wsum[tid >> 6][j] = c;
+    }
+    __syncthreads();
+    if (tid < top_k) {
+        const int ej = ids[t * top_k + tid];
+        const bool valid = ej >= 0 && ej < E;
+        const int d = wsum[0][tid] + wsum[1][tid] + wsum[2][tid] + wsum[3][tid];
+        dst[t * top_k + tid] = valid ? d : R;  // a dropped pair points one past the last row
+        if (valid) row_token[d] = t;
+    }
+}
+
 // One workgroup per token: quantise the row once, write it to its k destinations.
 template <bool QUANT, int DT = MOE355_DT_BF16>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x, int64_t H, int top_k,
@@ -479,6 +535,14 @@ extern "C" int moe355_route_map(const int32_t* expert_idx, int64_t num_tokens, i
     if (R > 0 && (!expert_idx || !expanded_row_idx || !row_token)) return MOE355_E_ARG;
     int nch, parts, cpp, nbits;
     const RouteWs ws = route_ws_of(workspace, R, num_experts, nch, parts, cpp, nbits);
+    if (R > 0 && R <= kMapSmallIters * 256 && num_tokens <= 1024) {
+        // one launch instead of three short ones that wait for each other (every workgroup reads all ids: not for
+        // thousands of tokens with one slot each)
+        hipLaunchKernelGGL(route_map_small_kernel, dim3((unsigned)num_tokens + 1), dim3(256),
+                           ((size_t)num_experts + 256) * 4, (hipStream_t)stream, expert_idx, (int)R, num_experts,
+                           tokens_num_type, ws.off, expert_tokens, expanded_row_idx, row_token, top_k);
+        return launch_status();
+    }
     launch_maps(expert_idx, R, num_experts, top_k, tokens_num_type, ws, nch, parts, cpp, nbits, expanded_row_idx,
                 row_token, expert_tokens, (hipStream_t)stream);
     return launch_status();
