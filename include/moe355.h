@@ -83,8 +83,9 @@ int moe355_dynamic_quant_form(const void *x, int x_dtype, int64_t rows, int64_t 
  * fused multiply-add chain over ascending k from +0 inside a chunk, chunk results added in ascending order to
  * a total that starts at +0, bias last.
  * x [T, hidden] bf16, fp16 or fp32; weight [E, hidden] fp32; bias [E] fp32 or NULL -> logits [T, E] fp32.
- * hidden must be a multiple of 64.  Few tokens (fewer than 128 output tiles of 32 x 128) run one workgroup
- * per K chunk and need the workspace (256-byte aligned); otherwise the workspace size is 0 and it may be NULL.
+ * hidden must be a multiple of 64 and below 2^22, num_experts * hidden below 2^30 (MOE355_E_SHAPE otherwise).
+ * Few tokens (fewer than 192 output tiles of 32 x 32) run one workgroup per K chunk and need the workspace
+ * (256-byte aligned); otherwise the workspace size is 0 and it may be NULL.
  */
 size_t moe355_router_gate_workspace(int64_t num_tokens, int hidden, int num_experts);
 int moe355_router_gate(const void *x, int x_dtype, const float *weight, const float *bias, int64_t num_tokens,

@@ -1,6 +1,7 @@
-"""Router gate kernel against the checker, bit for bit (fp32 logits), both launch forms (one workgroup per K
-chunk for few tokens, one workgroup over all chunks otherwise), ragged token and expert counts, the order-pin
-cases of the CPU suite, and the layer computing its own logits."""
+"""Router gate kernel against the checker, bit for bit (fp32 logits), every launch form (one workgroup per K
+chunk for few tokens; two or four wavefronts sharing an output tile and taking its chunks in turn; one wavefront
+per tile over all chunks), ragged token and expert counts, the order-pin cases of the CPU suite, and the layer
+computing its own logits."""
 import numpy as np
 import pytest
 import torch
@@ -31,19 +32,22 @@ def _same_bits(a: torch.Tensor, b: np.ndarray):
 
 
 # (T, H, E): decode (split over chunks), ragged everything, tail chunk of 64, more than 128 experts per row of
-# workgroups, enough tiles for the single-pass form, DeepSeek-V3's K
+# workgroups, enough tiles for the single-pass form, DeepSeek-V3's K; then the forms in which the wavefronts of a
+# workgroup share a tile: four per tile (256 tiles; fp32 tokens: two), two per tile with a last group of one
+# chunk that is 64 long, at most 32 experts with two and with four per tile
 @pytest.mark.parametrize("T,H,E", [(64, 2048, 128), (5, 192, 40), (1, 64, 8), (33, 320, 288), (4200, 256, 256),
-                                   (4100, 192, 130), (96, 7168, 256)])
-@pytest.mark.parametrize("x_dtype", ["bf16", "f32"])
+                                   (4100, 192, 130), (96, 7168, 256), (1000, 2112, 256), (2000, 1088, 250),
+                                   (16001, 1088, 24), (9000, 2112, 20)])
+@pytest.mark.parametrize("x_dtype", ["bf16", "f32", "f16"])
 def test_router_gate_matches_the_checker(K, orc, T, H, E, x_dtype):
     print(f"router gate T={T} H={H} E={E} x={x_dtype}", flush=True)
     g = torch.Generator().manual_seed(T * 7 + E)
     x = torch.randn(T, H, generator=g)
     w = torch.randn(E, H, generator=g) * 0.05
     b = torch.randn(E, generator=g)
-    if x_dtype == "bf16":
-        xb = x.to(torch.bfloat16)
-        x_np = bits(xb)
+    if x_dtype in ("bf16", "f16"):
+        xb = x.to(torch.bfloat16 if x_dtype == "bf16" else torch.float16)
+        x_np = bits(xb) if x_dtype == "bf16" else xb.float().numpy()  # fp16 -> fp32 is exact
         x_dev = xb.to(DEV)
     else:
         x_np = x.numpy()
@@ -61,40 +65,47 @@ def test_router_gate_matches_the_checker(K, orc, T, H, E, x_dtype):
 
 
 def test_router_gate_order_cases_on_the_gpu(K, orc):
-    """The cases that tell the summation order apart, on both launch forms (1 token: split; 4200: single pass)."""
+    """The cases that tell the summation order apart, on every launch form: with 32 experts, 5 tokens run one
+    workgroup per chunk (8 at the longer K), 4200 one wavefront per tile; at 17 chunks (the last 64 long) 9000 tokens run four
+    wavefronts per tile, 16000 two and 30000 one."""
     big = F(2.0 ** 24)
-    H = 320
-    rows = []
-    for pairs in ({0: big, 128: 1, 129: 1}, {0: big, 64: 1, 65: 1}, {0: 1, 1: 1, 2: big}, {5: 1, 130: 1, 260: big},
-                  {5: big, 130: 1, 260: 1}):
-        r = np.zeros(H, dtype=F)
-        for k, v in pairs.items():
-            r[k] = v
-        rows.append(r)
-    want_col = np.array([big + 2, big, big + 2, big + 2, big], dtype=F)
-    a = F(1.0) + F(2.0 ** -12)
-    fma_row = np.zeros(H, dtype=F)
-    fma_w = np.ones(H, dtype=F)
-    fma_row[0], fma_w[0] = 1.0, -(F(1.0) + F(2.0 ** -11))
-    fma_row[1], fma_w[1] = a, a
-    for T in (5, 4200):
+    for H, T in ((320, 5), (320, 4200), (2112, 8), (2112, 9000), (2112, 16000), (2112, 30000)):
+        rows = []
+        cases = [({0: big, 128: 1, 129: 1}, big + 2), ({0: big, 64: 1, 65: 1}, big), ({0: 1, 1: 1, 2: big}, big + 2),
+                 ({5: 1, 130: 1, 260: big}, big + 2), ({5: big, 130: 1, 260: 1}, big)]
+        if H > 2100:  # chunks of different groups of two and of four, and the short last chunk
+            cases += [({0: big, 517: 1, 1027: 1}, big), ({517: 1, 1027: 1, 2100: big}, big + 2),
+                      ({700: big, 2050: 1, 2111: 1}, big + 2)]
+        for pairs, _ in cases:
+            r = np.zeros(H, dtype=F)
+            for k, v in pairs.items():
+                r[k] = v
+            rows.append(r)
+        n = len(rows)
+        want_col = np.array([v for _, v in cases], dtype=F)
+        a = F(1.0) + F(2.0 ** -12)
+        fma_row = np.zeros(H, dtype=F)
+        fma_w = np.ones(H, dtype=F)
+        fma_row[0], fma_w[0] = 1.0, -(F(1.0) + F(2.0 ** -11))
+        fma_row[1], fma_w[1] = a, a
+        print(f"gate order cases H={H} T={T}", flush=True)
         x = np.zeros((T, H), dtype=F)
-        x[:5] = np.stack(rows)
+        x[:n] = np.stack(rows)
         w = np.ones((32, H), dtype=F)
         got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV))
         torch.cuda.synchronize()
-        assert np.array_equal(got[:5, 0].cpu().numpy(), want_col), T
+        assert np.array_equal(got[:n, 0].cpu().numpy(), want_col), (H, T)
         assert _same_bits(got, orc.router_gate(x, w))
         x[0] = fma_row
         w[3] = fma_w
         got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV))
-        assert got[0, 3].item() == 2.0 ** -24, T
+        assert got[0, 3].item() == 2.0 ** -24, (H, T)
         # bias last: (1 + 2^24) + 1
         x[1] = 0
         x[1, 0], x[1, 128] = 1, big
         w[3] = 1
         got = K.router_gate(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV), torch.ones(32, device=DEV))
-        assert got[1, 3].item() == float(big), T
+        assert got[1, 3].item() == float(big), (H, T)
 
 
 def test_router_gate_argument_checks(K):
