@@ -34,10 +34,11 @@ def _same_bits(a: torch.Tensor, b: np.ndarray):
 # (T, H, E): decode (split over chunks), ragged everything, tail chunk of 64, more than 128 experts per row of
 # workgroups, enough tiles for the single-pass form, DeepSeek-V3's K; then the forms in which the wavefronts of a
 # workgroup share a tile: four per tile (256 tiles; fp32 tokens: two), two per tile with a last group of one
-# chunk that is 64 long, at most 32 experts with two and with four per tile
+# chunk that is 64 long, at most 32 experts with two and with four per tile; more than one round of workgroups,
+# the rest of the tokens in a launch of their own (two and four wavefronts per tile)
 @pytest.mark.parametrize("T,H,E", [(64, 2048, 128), (5, 192, 40), (1, 64, 8), (33, 320, 288), (4200, 256, 256),
                                    (4100, 192, 130), (96, 7168, 256), (1000, 2112, 256), (2000, 1088, 250),
-                                   (16001, 1088, 24), (9000, 2112, 20)])
+                                   (16001, 1088, 24), (9000, 2112, 20), (5000, 1088, 256), (4600, 2112, 256)])
 @pytest.mark.parametrize("x_dtype", ["bf16", "f32", "f16"])
 def test_router_gate_matches_the_checker(K, orc, T, H, E, x_dtype):
     print(f"router gate T={T} H={H} E={E} x={x_dtype}", flush=True)

@@ -294,34 +294,44 @@ __global__ __launch_bounds__(256) void router_gate_reduce_kernel(const float* __
 }
 
 // How a launch spreads the product over the chip: EW wavefronts of a workgroup side by side along the experts,
-// KW sharing a tile, and whether every chunk gets workgroups of its own.  Measured on MI355X (DeepSeek-V3 and
-// Qwen3 gate shapes): with fewer than 192 output tiles of 32 x 32 the chunk-per-workgroup form wins, up to 384
-// four wavefronts per tile, up to 768 two; from there on a wavefront per tile fills the 1024 SIMDs.
+// KW sharing a tile, or every chunk with workgroups of its own (split).  One workgroup fits a compute unit, so a
+// launch runs in rounds of 256 workgroups; `cost` is its length in rounds of the one-wavefront-per-tile form
+// (measured on MI355X, DeepSeek-V3 and Qwen3 gate shapes: a stage of two wavefronts per tile takes 1.2 to 1.45
+// times as long, of four 1.5 to 1.7 times, for half and a quarter of the stages).
 struct GatePlan {
     int ew, kw;
     bool split;
+    int64_t wgs;
+    double cost;
     int tw() const { return 4 / (ew * kw); }
 };
-static GatePlan gate_plan(int64_t T, int E, int n_chunks, int x_dtype)
+static GatePlan gate_form(int64_t T, int E, int kw)
 {
     GatePlan g;
+    g.kw = kw;
+    g.ew = kw == 4 ? 1 : (E > 32 ? 2 : 1);
+    g.split = false;
+    g.wgs = ((T + 32 * g.tw() - 1) / (32 * g.tw())) * ((E + 32 * g.ew - 1) / (32 * g.ew));
+    const double stage = kw == 1 ? 1.0 : kw == 2 ? 1.4 : 1.7;
+    g.cost = (double)((g.wgs + 255) / 256) * stage / kw;
+    return g;
+}
+// Fewer than 192 output tiles of 32 x 32: the chunk-per-workgroup form (when the caller can take it: it needs
+// the scratch).  Otherwise the cheapest of one, two and four wavefronts per tile; sharing a tile pays from four
+// chunks per wavefront on, and fp32 tokens are twice the loads, so four wavefronts on one tile would not fit
+// their LDS writes in a stage.
+static GatePlan gate_plan(int64_t T, int E, int n_chunks, int x_dtype, bool may_split = true)
+{
     const int64_t tiles = ((T + 31) / 32) * ((E + 31) / 32);
-    g.ew = E > 32 ? 2 : 1;
-    g.kw = 1;
-    g.split = tiles < 192;
-    if (!g.split && tiles < 384) {
-        g.kw = 4;
-        g.ew = 1;
-    } else if (!g.split && tiles < 768) {
-        g.kw = 2;
+    GatePlan g = gate_form(T, E, 1);
+    if (may_split && tiles < 192) {
+        g.split = true;
+        return g;
     }
-    // sharing a tile pays from four chunks per wavefront on
-    while (g.kw > 1 && n_chunks < 4 * g.kw) g.kw /= 2;
-    if (g.kw < 4) g.ew = E > 32 ? 2 : 1;
-    // fp32 tokens are twice the loads: four wavefronts on one tile would not fit their LDS writes in a stage
-    if (g.kw == 4 && x_dtype == MOE355_DT_F32) {
-        g.kw = 2;
-        g.ew = E > 32 ? 2 : 1;
+    for (int kw = 2; kw <= 4; kw *= 2) {
+        if (n_chunks < 4 * kw || (kw == 4 && x_dtype == MOE355_DT_F32)) break;
+        const GatePlan c = gate_form(T, E, kw);
+        if (c.cost < g.cost) g = c;
     }
     return g;
 }
@@ -357,7 +367,7 @@ using namespace moe355;
 extern "C" size_t moe355_router_gate_workspace(int64_t num_tokens, int hidden, int num_experts)
 {
     if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0) return 0;
-    if (!gate_plan(num_tokens, num_experts, 1, MOE355_DT_BF16).split) return 0;  // splitting depends on the tile count alone
+    if (!gate_plan(num_tokens, num_experts, 1, MOE355_DT_BF16).split) return 0;  // depends on the tile count alone
     const size_t chunks = (size_t)((hidden + kGateChunk - 1) / kGateChunk);
     return ((chunks * (size_t)num_tokens * (size_t)num_experts * 4 + 255) / 256) * 256;
 }
@@ -385,9 +395,34 @@ extern "C" int moe355_router_gate(const void* x, int x_dtype, const float* weigh
         out = (float*)workspace;
         b = nullptr;
     }
-    if (x_dtype == MOE355_DT_BF16) launch_gate<MOE355_DT_BF16>(g, x, weight, b, out, num_tokens, hidden, num_experts, n_chunks, st);
-    else if (x_dtype == MOE355_DT_F16) launch_gate<MOE355_DT_F16>(g, x, weight, b, out, num_tokens, hidden, num_experts, n_chunks, st);
-    else launch_gate<MOE355_DT_F32>(g, x, weight, b, out, num_tokens, hidden, num_experts, n_chunks, st);
+    auto launch = [&](const GatePlan& pl, int64_t t_first, int64_t t_count) {
+        const int xb = x_dtype == MOE355_DT_F32 ? 4 : 2;
+        const void* xp = (const char*)x + t_first * hidden * xb;
+        float* op = out + t_first * num_experts;
+        if (x_dtype == MOE355_DT_BF16) launch_gate<MOE355_DT_BF16>(pl, xp, weight, b, op, t_count, hidden, num_experts, n_chunks, st);
+        else if (x_dtype == MOE355_DT_F16) launch_gate<MOE355_DT_F16>(pl, xp, weight, b, op, t_count, hidden, num_experts, n_chunks, st);
+        else launch_gate<MOE355_DT_F32>(pl, xp, weight, b, op, t_count, hidden, num_experts, n_chunks, st);
+    };
+    // More than one round: the full rounds run one wavefront per tile; a last round that would leave most SIMDs
+    // idle becomes a launch of its own over the remaining tokens when sharing its tiles makes it shorter.
+    int64_t main_tokens = num_tokens;
+    GatePlan first = g, rest = g;
+    const GatePlan one = gate_form(num_tokens, num_experts, 1);
+    if (!g.split && one.wgs > 256 && one.wgs % 256 != 0) {
+        const int64_t wg_cols = (num_experts + 32 * one.ew - 1) / (32 * one.ew);
+        const int64_t wg_rows = one.wgs / 256 * 256 / wg_cols;
+        const int64_t n_first = wg_rows * 32 * one.tw();
+        if (wg_rows > 0 && n_first < num_tokens) {
+            const GatePlan r = gate_plan(num_tokens - n_first, num_experts, n_chunks, x_dtype, false);
+            if ((double)((wg_rows * wg_cols + 255) / 256) + r.cost < g.cost - 0.05) {
+                main_tokens = n_first;
+                first = one;
+                rest = r;
+            }
+        }
+    }
+    launch(first, 0, main_tokens);
+    if (main_tokens < num_tokens) launch(rest, main_tokens, num_tokens - main_tokens);
     if (g.split) {
         const int64_t n = num_tokens * num_experts;
         hipLaunchKernelGGL(router_gate_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
