@@ -400,6 +400,27 @@ int moe355_dequant_swiglu_quant_static(const int32_t *x, const float *weight_sca
                                        int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t *y,
                                        void *stream);
 
+/* The general form of the same op, as the reference's grouped kernel computes it
+ * (csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant.h; Python call site
+ * vllm_ascend/ops/fused_moe/moe_mlp.py:340-359 with group_index = the per-expert row counts):
+ *   group_index [num_groups] int64 row COUNTS (NULL: one group owning every row); group g owns the next
+ *     group_index[g] rows and brings weight_scale[g][n], bias[g][n], quant_scale[g] or [g][n/2]; rows past the
+ *     sum get y = 0, scale = 0 (the reference leaves them unwritten)                                (:211-242)
+ *   bias_kind 1: int32 bias added to x; 2: fp32 bias added after the scales; 0: none (bias NULL)    (:380-424)
+ *   activation_scale may be NULL (no per-row scale)
+ *   swiglu_mode 0: lin * silu(act), clamp_limit ignored; 1: lin = clamp(lin, +-clamp_limit) + glu_bias,
+ *     act = min(act, clamp_limit) (clamps only when clamp_limit > 0), lin * act / (1 + exp(-glu_alpha * act))  (:627-677)
+ *   quant_mode 1: scale = max|v| * (float)(1.0 / 127.0), y = rint(v / scale)                       (:681-738)
+ *   quant_mode 0: quant_scale_len == num_groups: y = rint(v * (1 / quant_scale[g]) + quant_offset[g]);
+ *     == num_groups * n/2: y = rint(v / quant_scale[g][c] + quant_offset[g][c]); scale is not written (:741-790)
+ * A quant_scale in quant_mode 1 (the smooth scale) is MOE355_E_UNSUPPORTED. */
+int moe355_dequant_swiglu_quant_grouped(const int32_t *x, const float *weight_scale, const float *activation_scale,
+                                        const void *bias, int bias_kind, const int64_t *group_index, int num_groups,
+                                        int64_t rows, int64_t n, int activate_left, int swiglu_mode,
+                                        float clamp_limit, float glu_alpha, float glu_bias, int quant_mode,
+                                        const float *quant_scale, int64_t quant_scale_len, const float *quant_offset,
+                                        int8_t *y, float *scale, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Weighted un-permute (finalize routing).
  * Stands in for torch_npu.npu_moe_token_unpermute as called from

@@ -47,6 +47,11 @@
  *                         "swap the halves of x and of the weight scale")
  *   orc_dequant_swiglu_quant_static : the dynamic mode's SwiGLU values (orc_swiglu_quant's y) pushed through
  *                         numpy's y / scale + offset and rint, per-channel and per-tensor, with and without offset
+ *   orc_dequant_swiglu_quant_grouped : with one group, no bias and swiglu_mode 0 the SwiGLU values of
+ *                         orc_dequant_swiglu_quant; with groups, the same function called per row range with that
+ *                         group's scales (numpy slicing); int32 bias = the op on x + bias; float64 closed form of
+ *                         the swiglu_mode 1 expression (clamps, alpha, bias) within fp32 rounding; the quantiser's
+ *                         own arithmetic (max * (1/127), v / scale) against numpy float32
  *   orc_erff, orc_tanhf : math.erf within 5e-7, math.tanh within 3e-7 absolute on a dense grid, odd symmetry, the limits
  *   orc_act_mul_quant   : float64 formulas of the four activations within 16-bit rounding, clamp closed forms,
  *                         the quantiser of orc_dynamic_quant on the rounded values; which intermediate roundings
@@ -706,6 +711,109 @@ ORC_API int orc_dequant_swiglu_quant_static(const int32_t *x, const float *w_sca
             t = t < -128.0f ? -128.0f : t;
             q[r * I + i] = (int8_t)t;
         }
+    return 0;
+}
+
+/*
+ * The general form of npu_dequant_swiglu_quant: rows in groups with a weight scale (bias, quant scale) per group,
+ * int32 or float bias, the clamped / scaled SwiGLU of swiglu_mode 1.  Restates the kernel class every grouped
+ * call runs, csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant.h (dispatch:
+ * dequant_swiglu_quant.cpp:77-171):
+ *   groups      group_index holds row COUNTS (negative = 0); group g owns the next count rows; rows past the sum
+ *               are not processed (here: y = 0, scale = 0)                                         (:211-242)
+ *   dequant     int32 bias is added to x first; f = float(x) * weight_scale[g][c], then * activation_scale[row]
+ *               when there is one; a float bias is added after both                               (:380-424)
+ *   swiglu 0    lin * (act / (1 + exp(-act))), no clamp                                             (:432-470)
+ *   swiglu 1    lin = clamp(lin, -L, L) + glu_bias;  act = min(act, L)  (both only when L > 0);
+ *               lin * (act / (1 + exp(act * -glu_alpha)))                                           (:627-677)
+ *   dynamic     scale = max|v| * (float)(1.0 / 127.0);  q = rint(v / scale)                         (:681-738)
+ *   static      one scale per group: q = rint(v * (1 / quant_scale[g]) + quant_offset[g]);
+ *               per channel: q = rint(v / quant_scale[g][c] + quant_offset[g][c])                   (:277-324, :741-790)
+ * "act" is the left half when activate_left, else the right one.  bias_kind: 0 none, 1 int32, 2 float.
+ * An all-zero row has scale 0 and q = 0 (fixed by build: the kernel divides by zero there).
+ */
+ORC_API int orc_dequant_swiglu_quant_grouped(const int32_t *x, const float *w_scale, const float *a_scale,
+                                             const void *bias, int bias_kind, const int64_t *group_index,
+                                             int64_t num_groups, int64_t rows, int64_t N, int activate_left,
+                                             int swiglu_mode, float clamp_limit, float glu_alpha, float glu_bias,
+                                             int quant_mode, const float *quant_scale, int quant_per_channel,
+                                             const float *quant_offset, int8_t *q, float *qs)
+{
+    const int64_t I = N / 2;
+    const float factor = (float)(1.0 / 127.0);
+    float *v = (float *)malloc(sizeof(float) * (size_t)(I > 0 ? I : 1));
+    int64_t g = 0, left = (group_index && num_groups > 0) ? (group_index[0] < 0 ? 0 : group_index[0]) : rows;
+    for (int64_t r = 0; r < rows; ++r) {
+        if (group_index) {
+            while (g < num_groups && left == 0) {
+                ++g;
+                if (g < num_groups) left = group_index[g] < 0 ? 0 : group_index[g];
+            }
+            if (g >= num_groups) { /* past the last group */
+                memset(q + r * I, 0, (size_t)I);
+                if (qs) qs[r] = 0.0f;
+                continue;
+            }
+            --left;
+        }
+        const float *ws = w_scale + g * N;
+        float amax = 0.0f;
+        for (int64_t i = 0; i < I; ++i) {
+            const int64_t ai = activate_left ? i : i + I, li = activate_left ? i + I : i;
+            int32_t xa = x[r * N + ai], xl = x[r * N + li];
+            if (bias_kind == 1) {
+                xa = (int32_t)((uint32_t)xa + (uint32_t)((const int32_t *)bias)[g * N + ai]);
+                xl = (int32_t)((uint32_t)xl + (uint32_t)((const int32_t *)bias)[g * N + li]);
+            }
+            float act = (float)xa * ws[ai], lin = (float)xl * ws[li];
+            if (a_scale) {
+                act = act * a_scale[r];
+                lin = lin * a_scale[r];
+            }
+            if (bias_kind == 2) {
+                act = act + ((const float *)bias)[g * N + ai];
+                lin = lin + ((const float *)bias)[g * N + li];
+            }
+            float e;
+            if (swiglu_mode == 1) {
+                if (clamp_limit > 0.0f) {
+                    lin = lin > clamp_limit ? clamp_limit : lin;
+                    lin = lin < -clamp_limit ? -clamp_limit : lin;
+                }
+                lin = lin + glu_bias;
+                if (clamp_limit > 0.0f) act = act > clamp_limit ? clamp_limit : act;
+                e = orc_expf(act * -glu_alpha);
+            } else {
+                e = orc_expf(act * -1.0f);
+            }
+            v[i] = lin * (act / (1.0f + e));
+            const float a = fabsf(v[i]);
+            amax = a > amax ? a : amax;
+        }
+        if (quant_mode == 1) {
+            const float scale = amax * factor;
+            qs[r] = amax == 0.0f ? 0.0f : scale;
+            for (int64_t i = 0; i < I; ++i) {
+                float t = amax == 0.0f ? 0.0f : rintf(v[i] / scale);
+                t = t > 127.0f ? 127.0f : t;
+                t = t < -128.0f ? -128.0f : t;
+                q[r * I + i] = (int8_t)t;
+            }
+        } else {
+            for (int64_t i = 0; i < I; ++i) {
+                float t;
+                if (quant_per_channel)
+                    t = v[i] / quant_scale[g * I + i] + (quant_offset ? quant_offset[g * I + i] : 0.0f);
+                else
+                    t = v[i] * (1.0f / quant_scale[g]) + (quant_offset ? quant_offset[g] : 0.0f);
+                t = rintf(t);
+                t = t > 127.0f ? 127.0f : t;
+                t = t < -128.0f ? -128.0f : t;
+                q[r * I + i] = (int8_t)t;
+            }
+        }
+    }
+    free(v);
     return 0;
 }
 

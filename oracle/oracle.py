@@ -336,6 +336,40 @@ def dequant_swiglu_quant(x_i32, w_scale, a_scale, activate_left=True, clamp_limi
     return q, qs
 
 
+def dequant_swiglu_quant_grouped(x_i32, w_scale, a_scale=None, group_index=None, bias=None, activate_left=True,
+                                 swiglu_mode=0, clamp_limit=0.0, glu_alpha=1.0, glu_bias=0.0, quant_mode=1,
+                                 quant_scale=None, quant_offset=None):
+    """The grouped form: w_scale [G, N] (or [N]), group_index [G] row counts or None, bias [G, N] int32 or float.
+    -> (q int8 [rows, N/2], scale [rows] float32; zeros in static mode)."""
+    x = np.ascontiguousarray(x_i32, dtype=np.int32)
+    rows, N = x.shape
+    ws = np.ascontiguousarray(w_scale, dtype=np.float32).reshape(-1, N)
+    G = ws.shape[0]
+    as_ = None if a_scale is None else np.ascontiguousarray(a_scale, dtype=np.float32).reshape(-1)
+    gi = None if group_index is None else np.ascontiguousarray(group_index, dtype=np.int64).reshape(-1)
+    assert gi is None or gi.size == G
+    kind, b = 0, None
+    if bias is not None:
+        kind = 1 if np.asarray(bias).dtype == np.int32 else 2
+        b = np.ascontiguousarray(bias, dtype=np.int32 if kind == 1 else np.float32).reshape(G, N)
+    qsc = qof = None
+    per_channel = 0
+    if quant_mode == 0:
+        qsc = np.ascontiguousarray(quant_scale, dtype=np.float32).reshape(-1)
+        per_channel = int(qsc.size == G * (N // 2) and N // 2 != 1)
+        assert per_channel or qsc.size == G
+        if quant_offset is not None:
+            qof = np.ascontiguousarray(quant_offset, dtype=np.float32).reshape(-1)
+            assert qof.size == qsc.size
+    q = np.zeros((rows, N // 2), dtype=np.int8)
+    qs = np.zeros((rows,), dtype=np.float32)
+    lib().orc_dequant_swiglu_quant_grouped(_p(x), _p(ws), _p(as_), _p(b), _i32(kind), _p(gi), _i64(G), _i64(rows),
+                                           _i64(N), _i32(int(activate_left)), _i32(swiglu_mode), _f32(clamp_limit),
+                                           _f32(glu_alpha), _f32(glu_bias), _i32(quant_mode), _p(qsc),
+                                           _i32(per_channel), _p(qof), _p(q), _p(qs))
+    return q, qs
+
+
 def dequant_swiglu_quant_static(x_i32, w_scale, a_scale, quant_scale, quant_offset=None, activate_left=True,
                                 clamp_limit=0.0):
     x = np.ascontiguousarray(x_i32, dtype=np.int32)
@@ -437,16 +471,18 @@ def experts_forward(x_bf16, topk_w_bf16, topk_ids, w13, s13, w2, s2, *, keep_acc
     return tr
 
 
-def shared_expert_forward(x_bf16, w13, s13, w2, s2) -> np.ndarray:
+def shared_expert_forward(x_bf16, w13, s13, w2, s2, swiglu_limit=0.0, swiglu_alpha=1.0, swiglu_beta=0.0) -> np.ndarray:
     """Dense W8A8 MLP every token goes through, op for op as the reference's shared expert
     (vllm_ascend/ops/fused_moe/shared_experts.py:254-301): dynamic quant -> int32 matmul ->
-    dequant_swiglu_quant (weight scale first, then activation scale) -> matmul with per-token
+    dequant_swiglu_quant (weight scale first, then activation scale; called with swiglu_mode=1 on int32 x,
+    :272-289, which the reference's tiling sends to its grouped kernel class) -> matmul with per-token
     scale -> bf16.  w13 [2I,H], s13 [2I], w2 [H,I], s2 [H]."""
     T = x_bf16.shape[0]
     one = np.array([T], dtype=np.int64)
     xq, sx = dynamic_quant(x_bf16)
     acc1 = gmm_i32(xq, w13[None], one)
-    q1, s1 = dequant_swiglu_quant(acc1, s13, sx, activate_left=True)
+    q1, s1 = dequant_swiglu_quant_grouped(acc1, s13, sx, activate_left=True, swiglu_mode=1, clamp_limit=swiglu_limit,
+                                          glu_alpha=swiglu_alpha, glu_bias=swiglu_beta)
     acc2 = gmm_i32(q1, w2[None], one)
     return gmm2_dequant(acc2, s1, s2[None], one)
 

@@ -551,6 +551,91 @@ def test_dequant_swiglu_quant_static_mode(K, orc, rows, n, left):
         assert sc.shape == (rows,)
 
 
+# the general form (groups, biases, swiglu_mode 1, both quant modes) and the row kernel behind swiglu_mode 1 calls
+# without groups (the shared expert's call), against the restatement of the reference's grouped kernel class
+@pytest.mark.parametrize("rows,n", [(20, 192), (300, 2048), (5, 8448), (64, 4096)])
+@pytest.mark.parametrize("left", [True, False])
+def test_dequant_swiglu_quant_grouped(K, orc, rows, n, left):
+    g = torch.Generator().manual_seed(rows * 7 + n)
+    G = 7
+    x = torch.randint(-3000, 3000, (rows, n), generator=g, dtype=torch.int32)
+    ws = (torch.rand(G, n, generator=g) * 1.8 + 0.2) * 1e-3
+    a = torch.rand(rows, generator=g) * 1.5 + 0.5
+    bias_i = torch.randint(-50, 50, (G, n), generator=g, dtype=torch.int32)
+    bias_f = torch.randn(G, n, generator=g)
+    cuts = sorted(torch.randint(0, rows, (G - 1,), generator=g).tolist())
+    counts = torch.tensor([b - a_ for a_, b in zip([0] + cuts, cuts + [rows - rows // 5])], dtype=torch.int64).clamp_(min=-1)
+    x[1] = 0                                                        # an all-zero row: scale 0, q 0
+    dev = lambda t: None if t is None else t.to(DEV)
+    npy = lambda t: None if t is None else t.numpy()
+
+    def both(**kw):
+        t = {k: dev(v) if torch.is_tensor(v) else v for k, v in kw.items()}
+        o = {{"weight_scale": "w_scale", "activation_scale": "a_scale"}.get(k, k): npy(v) if torch.is_tensor(v) else v
+             for k, v in kw.items()}
+        got = K.dequant_swiglu_quant_grouped(dev(x), activate_left=left, **t)
+        torch.cuda.synchronize()
+        want = orc.dequant_swiglu_quant_grouped(x.numpy(), activate_left=left, **o)
+        assert np.array_equal(got[0].cpu().numpy(), want[0]), kw.keys()
+        if kw.get("quant_mode", 1) == 1:
+            assert np.array_equal(got[1].cpu().numpy().view(np.uint32), want[1].view(np.uint32)), kw.keys()
+        return want
+
+    m1 = dict(swiglu_mode=1, clamp_limit=1.5, glu_alpha=1.702, glu_bias=1.0)
+    # one group: the row kernel (what the shared expert runs), plain and with every swiglu_mode 1 parameter
+    both(weight_scale=ws[0], activation_scale=a)
+    both(weight_scale=ws[0], activation_scale=a, swiglu_mode=1)
+    both(weight_scale=ws[0], activation_scale=a, **m1)
+    both(weight_scale=ws[0], activation_scale=a, swiglu_mode=1, clamp_limit=0.75)
+    both(weight_scale=ws[0], activation_scale=None, **m1)           # no activation scale: the general kernel
+    # groups
+    w = both(weight_scale=ws, activation_scale=a, group_index=counts)
+    total = int(counts.clamp(min=0).sum())
+    assert total < rows and not w[0][total:].any() and not w[1][total:].any()
+    both(weight_scale=ws, activation_scale=a, group_index=counts, **m1)
+    both(weight_scale=ws, activation_scale=a, group_index=counts, bias=bias_i, **m1)
+    both(weight_scale=ws, activation_scale=a, group_index=counts, bias=bias_f)
+    both(weight_scale=ws, activation_scale=None, group_index=counts, bias=bias_f, **m1)
+    # static quantisation: one scale per group, one per group and channel, with and without offsets
+    qs_g, qo_g = torch.rand(G, generator=g) * 0.04 + 0.01, torch.randn(G, generator=g)
+    qs_c, qo_c = torch.rand(G, n // 2, generator=g) * 0.04 + 0.01, torch.randn(G, n // 2, generator=g)
+    both(weight_scale=ws, activation_scale=a, group_index=counts, quant_mode=0, quant_scale=qs_g, quant_offset=qo_g)
+    both(weight_scale=ws, activation_scale=a, group_index=counts, quant_mode=0, quant_scale=qs_c, quant_offset=qo_c, **m1)
+    both(weight_scale=ws, activation_scale=a, group_index=counts, quant_mode=0, quant_scale=qs_c)
+
+
+def test_npu_dequant_swiglu_quant_operator_routes_like_the_reference(K, orc):
+    """group_index / swiglu_mode 1 -> the grouped kernel class (clamp, alpha, bias, its quantiser); swiglu_mode 0
+    without groups -> the older kernels, which ignore clamp_limit (dequant_swiglu_quant_tiling.cpp:555-571)."""
+    from vllm_ascend_amd import custom_ops
+
+    custom_ops.enable_custom_op()
+    op = torch.ops._C_ascend.npu_dequant_swiglu_quant
+    g = torch.Generator().manual_seed(5)
+    rows, n, G = 48, 512, 4
+    x = torch.randint(-3000, 3000, (rows, n), generator=g, dtype=torch.int32)
+    ws = (torch.rand(G, n, generator=g) * 1.8 + 0.2) * 1e-3
+    a = torch.rand(rows, 1, generator=g) * 1.5 + 0.5
+    counts = torch.tensor([10, 0, 30, 8], dtype=torch.int64)
+    y, s = op(x.to(DEV), weight_scale=ws.to(DEV), activation_scale=a.to(DEV), group_index=counts.to(DEV),
+              activate_left=True, quant_mode=1)                                   # moe_mlp.py:340-359
+    want = orc.dequant_swiglu_quant_grouped(x.numpy(), ws.numpy(), a.numpy(), counts.numpy())
+    assert np.array_equal(y.cpu().numpy(), want[0]) and np.array_equal(s.cpu().numpy(), want[1])
+    kw = dict(activate_left=True, quant_mode=1, swiglu_mode=1, clamp_limit=2.0, glu_alpha=1.702, glu_bias=1.0)
+    y, s = op(x.to(DEV), weight_scale=ws[0].to(DEV), activation_scale=a.to(DEV), **kw)   # shared_experts.py:272-289
+    want = orc.dequant_swiglu_quant_grouped(x.numpy(), ws[0].numpy(), a.numpy(), swiglu_mode=1, clamp_limit=2.0,
+                                            glu_alpha=1.702, glu_bias=1.0)
+    assert np.array_equal(y.cpu().numpy(), want[0]) and np.array_equal(s.cpu().numpy(), want[1])
+    y, s = op(x.to(DEV), weight_scale=ws[0].to(DEV), activation_scale=a.to(DEV), activate_left=True, quant_mode=1,
+              swiglu_mode=0, clamp_limit=2.0)
+    want = orc.dequant_swiglu_quant(x.numpy(), ws[0].numpy(), a.numpy(), True, 0.0)
+    assert np.array_equal(y.cpu().numpy(), want[0]) and np.array_equal(s.cpu().numpy(), want[1])
+    with pytest.raises(NotImplementedError, match="smooth"):
+        op(x.to(DEV), weight_scale=ws[0].to(DEV), activation_scale=a.to(DEV), quant_scale=ws[0, :256].to(DEV), quant_mode=1)
+    with pytest.raises(ValueError, match="group_index"):
+        op(x.to(DEV), weight_scale=ws.to(DEV), activation_scale=a.to(DEV), quant_mode=1, swiglu_mode=1)
+
+
 @pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "swiglustep", "swigluoai"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_act_mul_quant(K, orc, act, dtype):

@@ -611,3 +611,117 @@ def test_layer_with_other_activations_matches_a_dense_float64_rendering():
         got = orc.half_to_f32(tr.out).astype(np.float64)
         err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
         assert err <= 5e-2, (act, err)
+
+
+# ---- the grouped / swiglu_mode 1 form of dequant_swiglu_quant (csrc/moe/dequant_swiglu_quant/op_kernel/
+# dequant_swiglu_quant.h): pinned from outside the C restatement
+def _dsq_inputs(rows, n, groups, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-2000, 2000, (rows, n), dtype=np.int32)
+    ws = (rng.uniform(0.2, 2.0, (groups, n)) * 1e-3).astype(np.float32)
+    a = rng.uniform(0.5, 2.0, rows).astype(np.float32)
+    return rng, x, ws, a
+
+
+def _np_dynamic_quant_of_the_grouped_kernel(v):
+    """scale = max * float32(1 / 127); q = rint(v / scale), every step rounded to float32 (numpy)."""
+    v = v.astype(np.float32)
+    amax = np.abs(v).max(axis=1)
+    s = (amax * np.float32(1.0 / 127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.rint((v / s[:, None]).astype(np.float32))
+    q = np.where(amax[:, None] == 0, 0, np.clip(q, -128, 127)).astype(np.int8)
+    return q, np.where(amax == 0, np.float32(0), s)
+
+
+def test_grouped_dsq_with_one_group_is_the_plain_swiglu_through_its_own_quantiser():
+    rng, x, ws, a = _dsq_inputs(400, 256, 1, 1)
+    q, s = orc.dequant_swiglu_quant_grouped(x, ws, a)
+    # the SwiGLU values of the plain op: same dequant order, same gate function (want_y of the fused epilogue's
+    # restatement takes the dequantised fp32 values)
+    f = ((x.astype(np.float32) * ws[0]).astype(np.float32) * a[:, None]).astype(np.float32)
+    _, _, y = orc.swiglu_quant(f, 0.0, want_y=True)
+    q_np, s_np = _np_dynamic_quant_of_the_grouped_kernel(y)
+    assert np.array_equal(q, q_np) and np.array_equal(s.view(np.uint32), s_np.view(np.uint32))
+    # no activation scale = a scale of ones
+    q1, s1 = orc.dequant_swiglu_quant_grouped(x, ws, None)
+    q2, s2 = orc.dequant_swiglu_quant_grouped(x, ws, np.ones(400, dtype=np.float32))
+    assert np.array_equal(q1, q2) and np.array_equal(s1, s2)
+    # the scale is max * (1/127), not max / 127: a row maximum where the two differ
+    amax = np.abs(y).max(axis=1)
+    differs = (amax * np.float32(1.0 / 127.0)).astype(np.float32) != (amax / np.float32(127.0)).astype(np.float32)
+    assert differs.any()
+    assert np.array_equal(s[differs], (amax * np.float32(1.0 / 127.0)).astype(np.float32)[differs])
+    # right half activated = halves swapped
+    swap = np.r_[128:256, 0:128]
+    q3, s3 = orc.dequant_swiglu_quant_grouped(np.ascontiguousarray(x[:, swap]), ws[:, swap], a, activate_left=False)
+    assert np.array_equal(q3, q) and np.array_equal(s3, s)
+
+
+def test_grouped_dsq_groups_are_row_ranges_with_their_own_scales():
+    counts = np.array([3, 0, 5, -2, 1, 0, 7], dtype=np.int64)     # negative counts are empty groups
+    rows, n = 20, 192                                             # 16 rows in groups, 4 past the last group
+    rng, x, ws, a = _dsq_inputs(rows, n, len(counts), 2)
+    bias_i = rng.integers(-50, 50, (len(counts), n), dtype=np.int32)
+    for kw in ({}, {"swiglu_mode": 1, "clamp_limit": 1.5, "glu_alpha": 1.702, "glu_bias": 1.0}):
+        q, s = orc.dequant_swiglu_quant_grouped(x, ws, a, counts, **kw)
+        qb, sb = orc.dequant_swiglu_quant_grouped(x, ws, a, counts, bias=bias_i, **kw)
+        start = 0
+        for g, c in enumerate(np.maximum(counts, 0)):
+            sl = slice(start, start + c)
+            q1, s1 = orc.dequant_swiglu_quant_grouped(x[sl], ws[g], a[sl], **kw)
+            assert np.array_equal(q[sl], q1) and np.array_equal(s[sl], s1), g
+            # an int32 bias is added to x before anything else
+            q2, s2 = orc.dequant_swiglu_quant_grouped(x[sl] + bias_i[g], ws[g], a[sl], **kw)
+            assert np.array_equal(qb[sl], q2) and np.array_equal(sb[sl], s2), g
+            start += c
+        assert start == 16 and not q[16:].any() and not s[16:].any()
+
+
+def test_grouped_dsq_mode_one_formula_against_float64():
+    rows, n = 64, 128
+    rng, x, ws, a = _dsq_inputs(rows, n, 1, 3)
+    bias_f = rng.standard_normal((1, n)).astype(np.float32)
+    for limit, alpha, beta, bias in ((0.0, 1.0, 0.0, None), (1.25, 1.702, 1.0, None), (0.0, 0.5, -0.75, bias_f),
+                                     (2.0, 1.0, 0.0, bias_f)):
+        q, s = orc.dequant_swiglu_quant_grouped(x, ws, a, bias=bias, swiglu_mode=1, clamp_limit=limit,
+                                                glu_alpha=alpha, glu_bias=beta)
+        f = x.astype(np.float64) * ws[0].astype(np.float64) * a[:, None].astype(np.float64)
+        if bias is not None:
+            f = f + bias[0]
+        act, lin = f[:, :64], f[:, 64:]
+        if limit > 0:
+            act = np.minimum(act, limit)
+            lin = np.clip(lin, -limit, limit)
+        v = (lin + beta) * act / (1.0 + np.exp(-alpha * act))
+        amax = np.abs(v).max(axis=1)
+        assert np.allclose(s, amax / 127.0, rtol=1e-5)
+        assert np.abs(q.astype(np.float64) * s[:, None] - v).max() <= 0.5001 * s.max() + 1e-6, (limit, alpha, beta)
+    # swiglu_mode 1 with alpha 1, beta 0 and no clamp is swiglu_mode 0; swiglu_mode 0 ignores all three
+    base = orc.dequant_swiglu_quant_grouped(x, ws, a)
+    same = orc.dequant_swiglu_quant_grouped(x, ws, a, swiglu_mode=1)
+    ignored = orc.dequant_swiglu_quant_grouped(x, ws, a, swiglu_mode=0, clamp_limit=0.01, glu_alpha=3.0, glu_bias=5.0)
+    for other in (same, ignored):
+        assert np.array_equal(base[0], other[0]) and np.array_equal(base[1], other[1])
+
+
+def test_grouped_dsq_static_mode_per_group_scales():
+    counts = np.array([4, 2, 0, 6], dtype=np.int64)
+    rows, n = 12, 64
+    rng, x, ws, a = _dsq_inputs(rows, n, 4, 4)
+    qs_g = rng.uniform(0.01, 0.05, 4).astype(np.float32)
+    qo_g = rng.standard_normal(4).astype(np.float32)
+    qs_c = rng.uniform(0.01, 0.05, (4, 32)).astype(np.float32)
+    qo_c = rng.standard_normal((4, 32)).astype(np.float32)
+    group_of_row = np.repeat(np.arange(4), counts)
+    f = ((x.astype(np.float32) * ws[group_of_row]).astype(np.float32) * a[:, None]).astype(np.float32)
+    _, _, y = orc.swiglu_quant(f, 0.0, want_y=True)
+    got, _ = orc.dequant_swiglu_quant_grouped(x, ws, a, counts, quant_mode=0, quant_scale=qs_g, quant_offset=qo_g)
+    inv = (np.float32(1.0) / qs_g).astype(np.float32)
+    want = np.clip(np.rint((y * inv[group_of_row][:, None]).astype(np.float32) + qo_g[group_of_row][:, None]), -128, 127)
+    assert np.array_equal(got, want.astype(np.int8))
+    got, _ = orc.dequant_swiglu_quant_grouped(x, ws, a, counts, quant_mode=0, quant_scale=qs_c, quant_offset=qo_c)
+    want = np.clip(np.rint((y / qs_c[group_of_row]).astype(np.float32) + qo_c[group_of_row]), -128, 127)
+    assert np.array_equal(got, want.astype(np.int8))
+    got, _ = orc.dequant_swiglu_quant_grouped(x, ws, a, counts, quant_mode=0, quant_scale=qs_c)
+    assert np.array_equal(got, np.clip(np.rint((y / qs_c[group_of_row]).astype(np.float32)), -128, 127).astype(np.int8))

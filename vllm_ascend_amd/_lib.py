@@ -78,6 +78,9 @@ PROTOTYPES = {
                                c_void_p, c_size_t, c_void_p]),
     "moe355_dequant_swiglu_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p,
                                             c_void_p, c_void_p]),
+    "moe355_dequant_swiglu_quant_grouped": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                                     c_int64, c_int64, c_int, c_int, c_float, c_float, c_float, c_int,
+                                                     c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe355_dequant_swiglu_quant_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                                    c_int64, c_int, c_float, c_void_p, c_void_p]),
     "moe355_act_mul_quant": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int64, c_int64, c_int, c_float,

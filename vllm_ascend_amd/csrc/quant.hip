@@ -123,11 +123,15 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const uint16_t* __re
 // x [rows, n] int32 -> dequant (weight scale, then activation scale) -> SwiGLU -> dynamic int8.
 // NH > 0: a thread keeps its (at most NH) SwiGLU values between the absmax and the rounding pass;
 // NH == 0: any row length, the values are computed again in the second pass.
+// alpha, beta: the SwiGLU of swiglu_mode 1, (u + beta) * g / (1 + exp(-alpha g)) on the clamped values.  form_b: the
+// quantiser of the reference's grouped kernel class, which also runs every swiglu_mode 1 call on int32 x
+// (scale = max * (float)(1.0 / 127.0), q = rint(v / scale)); otherwise scale = max / 127, q = rint(v * (1 / scale)).
 template <int NH>
 __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t* __restrict__ x,
                                                                    const float* __restrict__ w_scale,
                                                                    const float* __restrict__ a_scale, int64_t n,
-                                                                   int activate_left, float limit,
+                                                                   int activate_left, float limit, float alpha,
+                                                                   float beta, int form_b,
                                                                    int8_t* __restrict__ y, float* __restrict__ scale)
 {
     __shared__ float lds4[4];
@@ -137,6 +141,7 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
     const float as = a_scale[row];
     const int64_t goff = activate_left ? 0 : half;
     const int64_t uoff = activate_left ? half : 0;
+    const bool plain = alpha == 1.0f && beta == 0.0f;  // the proven short SiLU covers exactly this case
     auto value = [&](int64_t i) {
         float g = ((float)xr[goff + i] * w_scale[goff + i]) * as;
         float u = ((float)xr[uoff + i] * w_scale[uoff + i]) * as;
@@ -145,7 +150,8 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
             u = u > limit ? limit : u;
             u = u < -limit ? -limit : u;
         }
-        return m_silu(g) * u;
+        if (plain) return m_silu(g) * u;
+        return (u + beta) * (g / (1.0f + m_expf(g * -alpha)));
     };
     float held[NH > 0 ? NH : 1];
     float a = 0.0f;
@@ -164,19 +170,19 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_kernel(const int32_t
         }
     }
     a = block_max_256(a, lds4);
-    const float s = a / 127.0f;
+    const float s = form_b ? a * (float)(1.0 / 127.0) : a / 127.0f;
     const float inv = 1.0f / s;
     if (threadIdx.x == 0) scale[row] = (a == 0.0f) ? 0.0f : s;
     int8_t* yr = y + row * half;
+    auto quantise = [&](float v) { return (a == 0.0f) ? (int8_t)0 : sat_rint_i8(form_b ? v / s : v * inv); };
     if constexpr (NH > 0) {
 #pragma unroll
         for (int j = 0; j < NH; ++j) {
             const int64_t i = threadIdx.x + 256 * j;
-            if (i < half) yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(held[j] * inv);
+            if (i < half) yr[i] = quantise(held[j]);
         }
     } else {
-        for (int64_t i = threadIdx.x; i < half; i += 256)
-            yr[i] = (a == 0.0f) ? (int8_t)0 : sat_rint_i8(value(i) * inv);
+        for (int64_t i = threadIdx.x; i < half; i += 256) yr[i] = quantise(value(i));
     }
 }
 
@@ -207,6 +213,139 @@ __global__ __launch_bounds__(256) void dequant_swiglu_quant_static_kernel(
         if (per_channel) t = v / q_scale[i] + (q_offset ? q_offset[i] : 0.0f);
         else t = v * inv0 + (q_offset ? q_offset[0] : 0.0f);
         y[row * half + i] = sat_rint_i8(t);
+    }
+}
+
+// The general form of the op above: rows in groups (group_index = row counts) with a weight scale, bias and quant
+// scale per group, an int32 bias added to x or a float bias added after the scales, no activation scale, and the
+// clamped / scaled SwiGLU of swiglu_mode 1 (csrc/moe/dequant_swiglu_quant/op_kernel/dequant_swiglu_quant.h:211-242,
+// 380-424, 627-677).  Its dynamic quantiser multiplies the row maximum by (float)(1.0 / 127.0) and divides the
+// values by that scale (:681-738).  One workgroup per row; the first wavefront finds the row's group from the
+// counts.  Rows past the last group get y = 0 and scale = 0.
+struct DsqArgs {
+    const int32_t* x;
+    const float* w_scale;
+    const float* a_scale;
+    const void* bias;
+    int bias_kind;  // 0 none, 1 int32, 2 float
+    const int64_t* group_index;
+    int num_groups;
+    int64_t n;
+    int activate_left, swiglu_mode;
+    float limit, alpha, beta;
+    int quant_mode;
+    const float* q_scale;
+    int q_per_channel;
+    const float* q_offset;
+    int8_t* y;
+    float* scale;
+};
+
+__global__ __launch_bounds__(256) void dequant_swiglu_quant_grouped_kernel(DsqArgs a)
+{
+    __shared__ float lds4[4];
+    __shared__ int s_group;
+    const int64_t row = blockIdx.x;
+    const int64_t half = a.n >> 1;
+    int g = 0;
+    if (a.group_index) {
+        if (threadIdx.x < 64) {
+            const int lane = threadIdx.x;
+            const int per = (a.num_groups + 63) / 64;
+            int64_t local = 0;
+            for (int j = 0; j < per; ++j) {
+                const int gg = lane * per + j;
+                const int64_t c = gg < a.num_groups ? a.group_index[gg] : 0;
+                local += c < 0 ? 0 : c;
+            }
+            int64_t incl = local;
+            for (int off = 1; off < 64; off <<= 1) {
+                const int64_t t = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += t;
+            }
+            int64_t start = incl - local;
+            if (row >= start && row < incl) {
+                for (int j = 0; j < per; ++j) {
+                    const int gg = lane * per + j;
+                    const int64_t c = gg < a.num_groups ? a.group_index[gg] : 0;
+                    const int64_t cc = c < 0 ? 0 : c;
+                    if (row < start + cc) {
+                        s_group = gg;
+                        break;
+                    }
+                    start += cc;
+                }
+            }
+            if (lane == 63 && row >= incl) s_group = -1;
+        }
+        __syncthreads();
+        g = s_group;
+    }
+    int8_t* yr = a.y + row * half;
+    if (g < 0) {
+        for (int64_t i = threadIdx.x; i < half; i += 256) yr[i] = 0;
+        if (threadIdx.x == 0 && a.scale) a.scale[row] = 0.0f;
+        return;
+    }
+    const int32_t* xr = a.x + row * a.n;
+    const float* ws = a.w_scale + (int64_t)g * a.n;
+    const int64_t aoff = a.activate_left ? 0 : half;
+    const int64_t loff = a.activate_left ? half : 0;
+    const float as = a.a_scale ? a.a_scale[row] : 1.0f;
+    auto value = [&](int64_t i) {
+        int32_t xa = xr[aoff + i], xl = xr[loff + i];
+        if (a.bias_kind == 1) {
+            const int32_t* b = (const int32_t*)a.bias + (int64_t)g * a.n;
+            xa = (int32_t)((uint32_t)xa + (uint32_t)b[aoff + i]);
+            xl = (int32_t)((uint32_t)xl + (uint32_t)b[loff + i]);
+        }
+        float act = (float)xa * ws[aoff + i], lin = (float)xl * ws[loff + i];
+        if (a.a_scale) {
+            act = act * as;
+            lin = lin * as;
+        }
+        if (a.bias_kind == 2) {
+            const float* b = (const float*)a.bias + (int64_t)g * a.n;
+            act = act + b[aoff + i];
+            lin = lin + b[loff + i];
+        }
+        float e;
+        if (a.swiglu_mode == 1) {
+            if (a.limit > 0.0f) {
+                lin = lin > a.limit ? a.limit : lin;
+                lin = lin < -a.limit ? -a.limit : lin;
+            }
+            lin = lin + a.beta;
+            if (a.limit > 0.0f) act = act > a.limit ? a.limit : act;
+            e = m_expf(act * -a.alpha);
+        } else {
+            e = m_expf(act * -1.0f);
+        }
+        return lin * (act / (1.0f + e));
+    };
+    if (a.quant_mode == 1) {
+        float amax = 0.0f;
+        for (int64_t i = threadIdx.x; i < half; i += 256) {
+            const float v = __builtin_fabsf(value(i));
+            amax = v > amax ? v : amax;
+        }
+        amax = block_max_256(amax, lds4);
+        const float s = amax * (float)(1.0 / 127.0);
+        if (threadIdx.x == 0) a.scale[row] = (amax == 0.0f) ? 0.0f : s;
+        for (int64_t i = threadIdx.x; i < half; i += 256)
+            yr[i] = (amax == 0.0f) ? (int8_t)0 : sat_rint_i8(value(i) / s);
+    } else {
+        for (int64_t i = threadIdx.x; i < half; i += 256) {
+            const float v = value(i);
+            float t;
+            if (a.q_per_channel) {
+                const int64_t c = (int64_t)g * half + i;
+                t = v / a.q_scale[c] + (a.q_offset ? a.q_offset[c] : 0.0f);
+            } else {
+                t = v * (1.0f / a.q_scale[g]) + (a.q_offset ? a.q_offset[g] : 0.0f);
+            }
+            yr[i] = sat_rint_i8(t);
+        }
     }
 }
 
@@ -359,6 +498,20 @@ extern "C" int moe355_dynamic_quant_form(const void* x, int x_dtype, int64_t row
     return dynamic_quant_impl(x, x_dtype, rows, cols, q, scale, form, stream);
 }
 
+static void launch_dsq(const int32_t* x, const float* weight_scale, const float* activation_scale, int64_t rows,
+                       int64_t n, int activate_left, float limit, float alpha, float beta, int form_b, int8_t* y,
+                       float* scale, void* stream)
+{
+#define MOE355_DSQ(NH_)                                                                                         \
+    hipLaunchKernelGGL(dequant_swiglu_quant_kernel<NH_>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x, \
+                       weight_scale, activation_scale, n, activate_left, limit, alpha, beta, form_b, y, scale)
+    const int64_t half = n / 2;
+    if (half <= 4 * 256) MOE355_DSQ(4);
+    else if (half <= 16 * 256) MOE355_DSQ(16);
+    else MOE355_DSQ(0);
+#undef MOE355_DSQ
+}
+
 extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight_scale, const float* activation_scale,
                                            int64_t rows, int64_t n, int activate_left, float clamp_limit, int8_t* y,
                                            float* scale, void* stream)
@@ -367,14 +520,7 @@ extern "C" int moe355_dequant_swiglu_quant(const int32_t* x, const float* weight
     if (rows == 0) return MOE355_OK;
     if (!x || !weight_scale || !activation_scale || !y || !scale) return MOE355_E_ARG;
     if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
-#define MOE355_DSQ(NH_)                                                                                         \
-    hipLaunchKernelGGL(dequant_swiglu_quant_kernel<NH_>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x, \
-                       weight_scale, activation_scale, n, activate_left, clamp_limit, y, scale)
-    const int64_t half = n / 2;
-    if (half <= 4 * 256) MOE355_DSQ(4);
-    else if (half <= 16 * 256) MOE355_DSQ(16);
-    else MOE355_DSQ(0);
-#undef MOE355_DSQ
+    launch_dsq(x, weight_scale, activation_scale, rows, n, activate_left, clamp_limit, 1.0f, 0.0f, 0, y, scale, stream);
     return launch_status();
 }
 
@@ -392,6 +538,60 @@ extern "C" int moe355_dequant_swiglu_quant_static(const int32_t* x, const float*
     hipLaunchKernelGGL(dequant_swiglu_quant_static_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x,
                        weight_scale, activation_scale, quant_scale, quant_scale_len != 1 ? 1 : 0,
                        quant_offset, n, activate_left, clamp_limit, y);
+    return launch_status();
+}
+
+extern "C" int moe355_dequant_swiglu_quant_grouped(const int32_t* x, const float* weight_scale,
+                                                   const float* activation_scale, const void* bias, int bias_kind,
+                                                   const int64_t* group_index, int num_groups, int64_t rows, int64_t n,
+                                                   int activate_left, int swiglu_mode, float clamp_limit,
+                                                   float glu_alpha, float glu_bias, int quant_mode,
+                                                   const float* quant_scale, int64_t quant_scale_len,
+                                                   const float* quant_offset, int8_t* y, float* scale, void* stream)
+{
+    if (rows < 0 || n <= 0 || (n & 1) || num_groups < 1) return MOE355_E_ARG;
+    if (bias_kind < 0 || bias_kind > 2 || (bias_kind != 0) != (bias != nullptr)) return MOE355_E_ARG;
+    if ((swiglu_mode != 0 && swiglu_mode != 1) || (quant_mode != 0 && quant_mode != 1)) return MOE355_E_ARG;
+    if (!group_index && num_groups != 1) return MOE355_E_ARG;
+    int per_channel = 0;
+    if (quant_mode == 0) {
+        if (!quant_scale) return MOE355_E_ARG;
+        if (quant_scale_len == (int64_t)num_groups * (n / 2) && n / 2 != 1) per_channel = 1;
+        else if (quant_scale_len != num_groups) return MOE355_E_SHAPE;
+    } else if (quant_scale || quant_offset) {
+        return MOE355_E_UNSUPPORTED;  // the smooth scale of the dynamic mode
+    }
+    if (rows == 0) return MOE355_OK;
+    if (!x || !weight_scale || !y || (quant_mode == 1 && !scale)) return MOE355_E_ARG;
+    if (rows > 0x7fffffffLL) return MOE355_E_SHAPE;
+    if (!group_index && bias_kind == 0 && activation_scale && quant_mode == 1) {
+        // the common call (shared expert): the row kernel that keeps its values in registers
+        const bool m1 = swiglu_mode == 1;
+        launch_dsq(x, weight_scale, activation_scale, rows, n, activate_left, m1 ? clamp_limit : 0.0f,
+                   m1 ? glu_alpha : 1.0f, m1 ? glu_bias : 0.0f, 1, y, scale, stream);
+        return launch_status();
+    }
+    DsqArgs a;
+    a.x = x;
+    a.w_scale = weight_scale;
+    a.a_scale = activation_scale;
+    a.bias = bias;
+    a.bias_kind = bias_kind;
+    a.group_index = group_index;
+    a.num_groups = num_groups;
+    a.n = n;
+    a.activate_left = activate_left;
+    a.swiglu_mode = swiglu_mode;
+    a.limit = clamp_limit;
+    a.alpha = glu_alpha;
+    a.beta = glu_bias;
+    a.quant_mode = quant_mode;
+    a.q_scale = quant_scale;
+    a.q_per_channel = per_channel;
+    a.q_offset = quant_offset;
+    a.y = y;
+    a.scale = scale;
+    hipLaunchKernelGGL(dequant_swiglu_quant_grouped_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, a);
     return launch_status();
 }
 

@@ -199,27 +199,36 @@ def _gmm_swiglu_quant_v2_meta(x, weight, weight_scale, x_scale, group_list, smoo
 def _npu_dequant_swiglu_quant(x, *, weight_scale=None, activation_scale=None, bias=None, quant_scale=None,
                               quant_offset=None, group_index=None, activate_left=True, quant_mode=0, swiglu_mode=0,
                               clamp_limit=0.0, glu_alpha=1.0, glu_bias=0.0):
+    """The reference runs two kernel families behind this op (csrc/moe/dequant_swiglu_quant/op_host/
+    dequant_swiglu_quant_tiling.cpp:555-571): calls with ``group_index``, and calls with ``swiglu_mode=1`` on int32
+    x, take the grouped class (``op_kernel/dequant_swiglu_quant.h``: clamp, ``glu_alpha``, ``glu_bias``, its own
+    dynamic quantiser); the others the older per-mode kernels, which know neither clamp nor alpha."""
     if quant_mode not in (0, 1):
         raise NotImplementedError("npu_dequant_swiglu_quant: quant_mode must be 0 (static) or 1 (dynamic)")
-    for name, val in (("bias", bias), ("group_index", group_index)):
-        if val is not None:
-            raise NotImplementedError(f"npu_dequant_swiglu_quant: `{name}` is not supported")
-    if glu_alpha != 1.0 or glu_bias != 0.0:
-        raise NotImplementedError("npu_dequant_swiglu_quant: glu_alpha / glu_bias variants are not supported")
-    if x.dtype != torch.int32 or weight_scale is None or activation_scale is None:
-        raise RuntimeError("npu_dequant_swiglu_quant expects int32 x with weight_scale and activation_scale")
+    if swiglu_mode not in (0, 1):
+        raise NotImplementedError("npu_dequant_swiglu_quant: swiglu_mode must be 0 or 1")
+    if x.dtype != torch.int32 or weight_scale is None:
+        raise RuntimeError("npu_dequant_swiglu_quant expects int32 x with weight_scale")
+    if quant_mode == 1:
+        for name, val in (("quant_scale", quant_scale), ("quant_offset", quant_offset)):
+            if val is not None:
+                raise NotImplementedError(f"npu_dequant_swiglu_quant: `{name}` (smooth scale) is not supported "
+                                          "in quant_mode=1")
+    elif quant_scale is None:
+        raise RuntimeError("npu_dequant_swiglu_quant: quant_mode=0 needs quant_scale")
+    if group_index is not None and group_index.dim() != 1:
+        raise NotImplementedError("npu_dequant_swiglu_quant: group_index must hold one row count per group")
+    if group_index is not None or swiglu_mode == 1 or bias is not None or activation_scale is None:
+        return kernels.dequant_swiglu_quant_grouped(
+            x, weight_scale, activation_scale, group_index, bias, activate_left, swiglu_mode, clamp_limit, glu_alpha,
+            glu_bias, quant_mode, quant_scale, quant_offset)
     ws = weight_scale.to(torch.float32).reshape(-1)
     as_ = activation_scale.to(torch.float32).reshape(-1)
     if quant_mode == 0:
         # static: q = rint(y / quant_scale + quant_offset); the scale output carries nothing (zeros here)
-        if quant_scale is None:
-            raise RuntimeError("npu_dequant_swiglu_quant: quant_mode=0 needs quant_scale")
-        y = kernels.dequant_swiglu_quant_static(x, ws, as_, quant_scale, quant_offset, activate_left, clamp_limit)
+        y = kernels.dequant_swiglu_quant_static(x, ws, as_, quant_scale, quant_offset, activate_left, 0.0)
         return y, torch.zeros(x.shape[:-1], dtype=torch.float32, device=x.device)
-    for name, val in (("quant_scale", quant_scale), ("quant_offset", quant_offset)):
-        if val is not None:
-            raise NotImplementedError(f"npu_dequant_swiglu_quant: `{name}` belongs to quant_mode=0")
-    return kernels.dequant_swiglu_quant(x, ws, as_, activate_left, clamp_limit)
+    return kernels.dequant_swiglu_quant(x, ws, as_, activate_left, 0.0)
 
 
 def _npu_dequant_swiglu_quant_meta(x, *, weight_scale=None, activation_scale=None, bias=None, quant_scale=None,

@@ -25,7 +25,8 @@ def shared_experts_calculation_stream() -> torch.cuda.Stream:
 
 class AscendSharedExperts(torch.nn.Module):
     def __init__(self, gate_up_weight: torch.Tensor, gate_up_scale: torch.Tensor, down_weight: torch.Tensor,
-                 down_scale: torch.Tensor, swiglu_limit: float = 0.0, multistream_overlap: bool = False):
+                 down_scale: torch.Tensor, swiglu_limit: float = 0.0, multistream_overlap: bool = False,
+                 swiglu_alpha: float = 1.0, swiglu_beta: float = 0.0):
         """gate_up_weight int8 [2I, H], down_weight int8 [H, I] (checkpoint order, one row per output
         channel); scales [2I] / [H]."""
         super().__init__()
@@ -37,6 +38,8 @@ class AscendSharedExperts(torch.nn.Module):
         self.gate_up_scale_fp32 = gate_up_scale.reshape(-1).to(torch.float32).contiguous()
         self.down_scale_fp32 = down_scale.reshape(-1).to(torch.float32).contiguous()
         self.swiglu_limit = swiglu_limit
+        self.swiglu_alpha = swiglu_alpha
+        self.swiglu_beta = swiglu_beta
         self.multistream_overlap = multistream_overlap
 
     def _mlp(self, hidden_states: torch.Tensor, quantized=None) -> torch.Tensor:
@@ -49,7 +52,7 @@ class AscendSharedExperts(torch.nn.Module):
         quantized_x, swiglu_out_scale = torch.ops._C_ascend.npu_dequant_swiglu_quant(
             x=acc, weight_scale=self.gate_up_scale_fp32, activation_scale=pertoken_scale, bias=None,
             quant_scale=None, quant_offset=None, group_index=None, activate_left=True, quant_mode=1,
-            swiglu_mode=1, clamp_limit=self.swiglu_limit)
+            swiglu_mode=1, clamp_limit=self.swiglu_limit, glu_alpha=self.swiglu_alpha, glu_bias=self.swiglu_beta)
         return npu_ops.npu_quant_matmul(quantized_x, self.down_weight, self.down_scale_fp32,
                                         pertoken_scale=swiglu_out_scale, bias=None, output_dtype=original_dtype)
 

@@ -403,6 +403,61 @@ def dequant_swiglu_quant(x, weight_scale, activation_scale, activate_left=True, 
     return y, s
 
 
+def dequant_swiglu_quant_grouped(x, weight_scale, activation_scale=None, group_index=None, bias=None,
+                                 activate_left=True, swiglu_mode=0, clamp_limit=0.0, glu_alpha=1.0, glu_bias=0.0,
+                                 quant_mode=1, quant_scale=None, quant_offset=None):
+    """The general form of npu_dequant_swiglu_quant: weight_scale [G, n] (or [n]), group_index [G] row counts,
+    bias [G, n] int32 or floating, swiglu_mode 1 with clamp_limit / glu_alpha / glu_bias, quant_mode 0 with
+    quant_scale [G] or [G, n/2].  -> (y int8, scale fp32; zeros in quant_mode 0)."""
+    x = _dev(x, "x")
+    if x.dtype != torch.int32:
+        raise TypeError(f"x: int32 tensor expected but got {x.dtype}")
+    lib = _lib.load()
+    n = x.shape[-1]
+    rows = x.numel() // n if n else 0
+    ws = _dev(weight_scale, "weight_scale").to(torch.float32).contiguous()
+    if ws.numel() % n:
+        raise ValueError(f"weight_scale has {ws.numel()} elements, x {n} columns")
+    groups = ws.numel() // n
+    gi = None
+    if group_index is not None:
+        gi = _dev(group_index, "group_index").to(torch.int64).contiguous()
+        if gi.dim() != 1 or gi.numel() != groups:
+            raise ValueError(f"group_index must hold one row count per group of weight_scale ({groups}), "
+                             f"got shape {tuple(gi.shape)}")
+    elif groups != 1:
+        raise ValueError("weight_scale with several groups needs group_index")
+    a = None
+    if activation_scale is not None:
+        a = _dev(activation_scale, "activation_scale").to(torch.float32).reshape(-1).contiguous()
+        if a.numel() != rows:
+            raise ValueError(f"activation_scale has {a.numel()} elements for {rows} rows")
+    kind = 0
+    if bias is not None:
+        bias = _dev(bias, "bias")
+        kind = 1 if bias.dtype == torch.int32 else 2
+        bias = (bias if kind == 1 else bias.to(torch.float32)).contiguous()
+        if bias.numel() != groups * n:
+            raise ValueError(f"bias must have {groups} x {n} elements, got {bias.numel()}")
+    qs = qo = None
+    if quant_mode == 0:
+        if quant_scale is None:
+            raise RuntimeError("quant_mode=0 needs quant_scale")
+        qs = _dev(quant_scale, "quant_scale").to(torch.float32).reshape(-1).contiguous()
+        if quant_offset is not None:
+            qo = _dev(quant_offset, "quant_offset").to(torch.float32).reshape(-1).contiguous()
+            if qo.numel() != qs.numel():
+                raise ValueError("quant_offset must have as many elements as quant_scale")
+    y = torch.empty(x.shape[:-1] + (n // 2,), dtype=torch.int8, device=x.device)
+    s = (torch.empty if quant_mode == 1 else torch.zeros)(x.shape[:-1], dtype=torch.float32, device=x.device)
+    check(lib.moe355_dequant_swiglu_quant_grouped(
+        _ptr(x), _ptr(ws), _ptr(a), _ptr(bias), kind, _ptr(gi), groups, rows, n, int(bool(activate_left)),
+        int(swiglu_mode), float(clamp_limit), float(glu_alpha), float(glu_bias), int(quant_mode), _ptr(qs),
+        qs.numel() if qs is not None else 0, _ptr(qo), _ptr(y), _ptr(s), _stream(x)),
+        "moe355_dequant_swiglu_quant_grouped")
+    return y, s
+
+
 def dequant_swiglu_quant_static(x, weight_scale, activation_scale, quant_scale, quant_offset=None,
                                 activate_left=True, clamp_limit=0.0):
     """quant_mode 0 of npu_dequant_swiglu_quant: one scale (and offset) per output channel or per tensor."""
