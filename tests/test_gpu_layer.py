@@ -235,7 +235,7 @@ def test_force_load_balance_with_log2phy_keeps_the_random_ids_unmapped():
     assert torch.isfinite(res.routed_out.float()).all()
 
 
-@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "swiglustep", "swigluoai"])
+@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "swiglustep", "swigluoai_uninterleave"])
 @pytest.mark.parametrize("name", ["c2_small", "c3_small"])
 def test_layer_with_other_activations(name, act):
     """Activations without a fused op take the unfused branch (vllm_ascend/ops/fused_moe/moe_mlp.py:484-569):
@@ -248,7 +248,7 @@ def test_layer_with_other_activations(name, act):
     print(f"layer {name} activation={act}", flush=True)
     d = make_layer(cfg, seed=2)
     layer = build_layer(cfg, d, DEV)
-    limit, alpha, beta = (0.0, 1.0, 0.0) if act != "swigluoai" else (7.0, 1.702, 1.0)
+    limit, alpha, beta = (0.0, 1.0, 0.0) if act != "swigluoai_uninterleave" else (7.0, 1.702, 1.0)
     layer.activation = act
     layer.moe_config = dataclasses.replace(layer.moe_config, activation=act, swiglu_limit=limit, swiglu_alpha=alpha,
                                            swiglu_beta=beta)
@@ -259,12 +259,23 @@ def test_layer_with_other_activations(name, act):
     kw = dict(k_group=1, group_count=1, group_select_mode=1, renorm=1, norm_type=0, x_dtype="f32")
     y, ids, _ = orc.gating_top_k(d["logits"].numpy(), cfg.k, **kw)
     tr = orc.experts_forward(bits(d["x"]), orc.f32_to_half(y), ids, d["w13"].numpy(), d["s13"].numpy(),
-                             d["w2"].numpy(), d["s2"].numpy(), activation=act, swiglu_limit=limit,
-                             swiglu_alpha=alpha, swiglu_beta=beta)
+                             d["w2"].numpy(), d["s2"].numpy(), activation=act.replace("_uninterleave", ""),
+                             swiglu_limit=limit, swiglu_alpha=alpha, swiglu_beta=beta)
     assert np.array_equal(res.expert_tokens.cpu().numpy(), tr.expert_tokens)
     assert np.array_equal(bits(res.routed_out), tr.out)
     silu = oracle_layer(cfg, d)
     assert not np.array_equal(tr.out, silu.out)  # the activation is really a different one
+    if act == "swigluoai_uninterleave":
+        # the interleaved name is not known to the reference's quantised MLP (moe_mlp.py:213): it takes the default
+        # branch there, the fused SwiGLU with the limit, and so it does here
+        layer.activation = "swigluoai"
+        layer.moe_config = dataclasses.replace(layer.moe_config, activation="swigluoai")
+        layer.moe_comm_method.moe_config = layer.moe_config
+        res = layer.forward_impl(x, logits)
+        torch.cuda.synchronize()
+        tr = orc.experts_forward(bits(d["x"]), orc.f32_to_half(y), ids, d["w13"].numpy(), d["s13"].numpy(),
+                                 d["w2"].numpy(), d["s2"].numpy(), swiglu_limit=limit)
+        assert np.array_equal(bits(res.routed_out), tr.out)
 
 
 def test_layer_with_per_expert_weight_lists():

@@ -52,9 +52,14 @@ def quant_apply_mlp(hidden_states, w1, w1_scale, w2, w2_scale, group_list, group
     act_name = getattr(activation, "value", activation) or "silu"
     from ..kernels import ACTIVATIONS
 
+    if act_name == "swigluoai":
+        # The reference's quantised MLP asks only for "swigluoai_uninterleave" (moe_mlp.py:213, 522-538); the
+        # interleaved name takes its default branch, the fused SwiGLU with swiglu_limit, alpha and beta unused.
+        act_name, swiglu_alpha, swiglu_beta = "silu", 1.0, 0.0
+
     if act_name != "silu" and act_name not in ACTIVATIONS:
         raise NotImplementedError(f"activation {act_name!r}: supported are 'silu' and {sorted(ACTIVATIONS)}")
-    if act_name not in ("swigluoai", "swigluoai_uninterleave") and (swiglu_alpha != 1.0 or swiglu_beta != 0.0):
+    if act_name != "swigluoai_uninterleave" and (swiglu_alpha != 1.0 or swiglu_beta != 0.0):
         raise NotImplementedError("swiglu_alpha / swiglu_beta belong to the swigluoai activation")
     if w1_offset is not None or w2_offset is not None:
         raise NotImplementedError("asymmetric weight offsets are not supported")
