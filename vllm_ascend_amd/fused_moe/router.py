@@ -41,7 +41,24 @@ class AscendFusedTopKRouter:
             topk_ids = torch.argsort(random_matrix, dim=1)[:, : topk_ids.size(1)].to(topk_ids.dtype)
         return topk_weights.to(weights_dtype), topk_ids
 
+    def is_fused_supported(self, hidden_states: torch.Tensor) -> bool:
+        """The reference's guard in front of the fused gating op, taken over as it stands (it measures the last
+        dimension of the hidden states, ``fused_topk_router.py:66-82``)."""
+        topk_group = self.topk_group if self.topk_group is not None else 1
+        num_expert_group = self.num_expert_group if self.num_expert_group is not None else 1
+        last = hidden_states.shape[-1]
+        if not (num_expert_group > 0 and last % num_expert_group == 0 and last // num_expert_group > 2):
+            return False
+        if self.top_k > (last / (num_expert_group * topk_group)):
+            return False
+        return not topk_group * last / num_expert_group < self.top_k
+
     def _compute_routing(self, hidden_states, router_logits, indices_type=None, weights_dtype=None):
+        if not self.is_fused_supported(hidden_states):
+            # the reference falls back to its torch-native grouped top-k here, whose group score (max instead of the
+            # sum of the top two) and tie order differ from the fused op's (grouped_topk_router.py:51-67)
+            raise NotImplementedError("router: shapes the fused gating op refuses take the torch-native router in "
+                                      "the reference, which this build does not have")
         bias = self.e_score_correction_bias
         if bias is not None and bias.dtype != router_logits.dtype:
             bias = self.e_score_correction_bias = bias.to(router_logits.dtype)
