@@ -215,6 +215,7 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const void* __restrict
         if constexpr (KW == 1) {
             total = total + p[ps];
         } else {
+            __syncthreads();  // nobody is still reading the results posted during the last stages
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 px[wave][q][lane] = (v4f){p[ps][4 * q], p[ps][4 * q + 1], p[ps][4 * q + 2], p[ps][4 * q + 3]};
