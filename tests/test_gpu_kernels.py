@@ -856,6 +856,52 @@ def test_grouped_gemms_on_skewed_histograms(K, orc, name, gl_type):
     assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
+@pytest.mark.parametrize("Kd,N", [(4096, 1024), (2048, 2048)])
+def test_split_grouped_gemms_on_random_histograms(K, orc, Kd, N):
+    """The two-launch forms (experts of at most 32 rows streamed, the others on tiles) on random histograms of 12 to
+    23 rows per expert: uniform, Zipf-skewed, and with experts set exactly on the borders."""
+    from vllm_ascend_amd._lib import W_ENK, load
+
+    E = 256
+    lib = load()
+    g = torch.Generator().manual_seed(Kd + N)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    w_np, sw_np = w.numpy(), sw.numpy()
+    for seed in range(3):
+        r = np.random.default_rng(seed)
+        avg = int(r.integers(12, 24))
+        if seed == 0:
+            cnt = r.multinomial(avg * E, np.full(E, 1.0 / E))
+        else:
+            p = 1.0 / np.arange(1, E + 1) ** r.uniform(0.6, 1.2)
+            cnt = r.multinomial(avg * E, r.permutation(p / p.sum()))
+        for e, c in zip(r.choice(E, 8, replace=False), (0, 31, 32, 33, 64, 65, 256, 257)):
+            cnt[e] = c
+        while cnt.sum() // E < 12:
+            cnt[int(r.integers(E))] += 40
+        while cnt.sum() // E > 23:
+            cnt[int(np.argmax(cnt))] //= 2
+        cnt = torch.from_numpy(cnt.astype(np.int64))
+        R = int(cnt.sum())
+        cum = torch.cumsum(cnt, 0)
+        print(f"split gemm K={Kd} N={N} seed={seed}: R={R} max={int(cnt.max())} empty={int((cnt == 0).sum())}", flush=True)
+        assert " + " in lib.moe355_gmm_kernel_name(1, R, Kd, N, E).decode()
+        x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+        sx = torch.rand(R, generator=g) * 0.05 + 0.001
+        ref = orc.gmm_i32(x.numpy(), w_np, cum.numpy())
+        want = orc.gmm2_dequant(ref, sx.numpy(), sw_np, cum.numpy())
+        got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt.to(DEV), 1, N, Kd)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(got.cpu()), want)
+        q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw_np, cum.numpy()))
+        q, s_ = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd)
+        torch.cuda.synchronize()
+        assert np.array_equal(q.cpu().numpy(), q_want)
+        assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
 def test_w4_scales_of_every_magnitude(K, orc):
     """Subnormal scales, scales near the bottom of the normal range, zero and negative scales next to ordinary
     ones give the checker's bits (a token scale of 2^90 brings the tiny products into bf16 range)."""
