@@ -80,13 +80,18 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     __shared__ int32_t red[(KSPLIT > 1) ? 32 * 64 : 1];
     __shared__ uint16_t plist[PAIRS ? kPairMax : 1];
     __shared__ int32_t pcount[4];
+    __shared__ uint32_t pmap[PAIRS ? 64 : 1];  // one bit per expert (at most 2048) that has pairs
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int NB = a.N >> 5, KB = a.K >> 5;
     const int upe = NB >> 1;  // units per expert
     const int64_t unit = (KSPLIT == 1) ? (int64_t)blockIdx.x * 4 + wave : (int64_t)blockIdx.x;
-    if (unit >= (int64_t)a.E * upe) return;  // KSPLIT == 1: no barriers below; KSPLIT == 4: whole workgroup leaves
-    const int e = (int)(unit / upe);
+    // pair order with fewer pairs than experts: the grid has a slot per pair instead of a place per expert (most
+    // experts are idle, and a workgroup that only finds that out still costs its dispatch: 28,000 of them are
+    // 150 us), and slot s belongs to the s-th expert that has pairs at all
+    const int places = (PAIRS && a.pair_slots > 0) ? a.pair_slots : a.E;
+    if (unit >= (int64_t)places * upe) return;  // KSPLIT == 1: no barriers below; KSPLIT == 4: whole workgroup leaves
+    int e = (int)(unit / upe);
     const int p = (int)(unit % upe);
     const int nb0 = (EPI == EPI_SWIGLU) ? p : 2 * p;
     const int nb1 = (EPI == EPI_SWIGLU) ? p + upe : 2 * p + 1;
@@ -103,6 +108,46 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     const int kb_begin = slab_begin + ((slab_end - slab_begin) * ks) / KSPLIT;
     const int kb_end = slab_begin + ((slab_end - slab_begin) * (ks + 1)) / KSPLIT;
 
+    // pair order: wavefront w scans pairs [w Q, (w + 1) Q), Q a multiple of 64 and at most 256.  The ids are
+    // requested in front of the weights: answers come back in the order of the requests, and the list of the
+    // expert's pairs (which the token loads wait for) should not queue behind the first weight tiles from HBM.
+    const int Q = PAIRS ? (((int)a.R + 255) >> 8) << 6 : 0;
+    int pid[PAIRS ? 4 : 1];
+    if constexpr (PAIRS) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int f = wave * Q + c * 64 + lane;
+            pid[c] = (c * 64 < Q && f < (int)a.R) ? a.pair_ids[f] : -1;
+        }
+    }
+    if constexpr (PAIRS) {
+        if (a.pair_slots > 0) {
+            // the experts that have pairs, as a bit map in LDS; every wavefront then finds the expert of the
+            // workgroup's slot by itself: a count of the bits in front of each word, and the word's bit
+            if (threadIdx.x < 64) pmap[threadIdx.x] = 0u;
+            __syncthreads();
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (pid[c] >= 0 && pid[c] < a.E) atomicOr(&pmap[pid[c] >> 5], 1u << (pid[c] & 31));
+            __syncthreads();
+            const uint32_t bits = pmap[lane];
+            const int cnt = __popc(bits);
+            int incl = cnt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int t = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += t;
+            }
+            const int excl = incl - cnt;
+            const bool has = e >= excl && e < incl;
+            const unsigned long long holder = __ballot(has);
+            if (holder == 0ull) return;  // fewer experts with pairs than slots (the same answer in all four wavefronts)
+            uint32_t t = bits;
+            for (int i = has ? e - excl : 0; i > 0; --i) t &= t - 1;
+            const int mine = lane * 32 + (t ? __builtin_ctz(t) : 0);
+            e = __shfl(mine, __builtin_ctzll(holder), 64);
+        }
+    }
     const int8_t* we = expert_weights(a, e);
     const int8_t* w0 = we + ((int64_t)nb0 * KB) * 1024 + lane * 16;
     const int8_t* w1 = we + ((int64_t)nb1 * KB) * 1024 + lane * 16;
@@ -123,18 +168,6 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
             }
         }
     };
-    // pair order: wavefront w scans pairs [w Q, (w + 1) Q), Q a multiple of 64 and at most 256.  The ids are
-    // requested in front of the weights: answers come back in the order of the requests, and the list of the
-    // expert's pairs (which the token loads wait for) should not queue behind the first weight tiles from HBM.
-    const int Q = PAIRS ? (((int)a.R + 255) >> 8) << 6 : 0;
-    int pid[PAIRS ? 4 : 1];
-    if constexpr (PAIRS) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int f = wave * Q + c * 64 + lane;
-            pid[c] = (c * 64 < Q && f < (int)a.R) ? a.pair_ids[f] : -1;
-        }
-    }
     if constexpr (EARLY) load_weights(kb_begin);
 
     int64_t row0 = 0, row1 = 0;
@@ -881,6 +914,21 @@ extern "C" int moe355_gmm_pairs_supported(int64_t num_tokens, int top_k, int64_t
     return num_tokens > 0 && top_k > 0 && num_tokens * top_k <= kPairMax && n > 0 && k > 0 && n % 64 == 0 && k % 32 == 0;
 }
 
+// pair order: how many places the grid gets.  A place per expert makes every idle expert cost the dispatch of its
+// workgroups (about 5 ns each: at one token of the DeepSeek-V3 shape 28,000 of them, 150 us); with few pairs the grid
+// gets a slot per pair instead (at most one per expert) and the kernel looks up which expert a slot belongs to.
+// Measured (whole layer, graph replay): DeepSeek-V3 shape 1 / 8 / 32 / 64 tokens 307 -> 104, 567 -> 403,
+// 1174 -> 1114, 1492 -> 1475 us; Qwen3 shape 1 / 4 / 16 tokens 48 -> 38, 62 -> 42, 91 -> 86 us, and from 24 tokens
+// on (more pairs than experts, 24 or 32 units per expert) the lookup costs what the few idle experts saved.  The
+// bit map of the lookup holds 2048 experts.
+static int pair_places(GmmArgs& a)
+{
+    const int64_t places = a.R < (int64_t)a.E ? a.R : (int64_t)a.E;
+    const bool few = a.R <= (int64_t)a.E || (a.R <= 2 * (int64_t)a.E && a.N / 64 >= 48);
+    a.pair_slots = (few && a.E <= 2048) ? (int)places : 0;
+    return (int)(a.pair_slots > 0 ? places : a.E);
+}
+
 extern "C" size_t moe355_gmm1_swiglu_quant_pairs_workspace(int64_t num_tokens, int top_k, int64_t n)
 {
     if (num_tokens <= 0 || top_k <= 0 || n <= 0) return 256;
@@ -922,7 +970,7 @@ extern "C" int moe355_gmm1_swiglu_quant_pairs(const int8_t* x, const float* x_sc
     a.pair_gather = 1;
     hipEvent_t ev0, ev1;
     take_profile_events(ev0, ev1);
-    const int64_t units = (int64_t)num_experts * (n / 64);
+    const int64_t units = (int64_t)pair_places(a) * (n / 64);
     launch_gemm(gmm_stream_kernel<EPI_SWIGLU, 4, 4, 3, false, true, true>, dim3((unsigned)units), st, a, ev0, ev1);
     launch_swiglu_requant(a.y, nullptr, 0, num_experts, rows, I, out, out_scale, st);
     return launch_status();
@@ -958,7 +1006,7 @@ extern "C" int moe355_gmm2_dequant_pairs(const int8_t* x, const int8_t* weight_n
     a.pair_gather = 0;
     hipEvent_t ev0, ev1;
     take_profile_events(ev0, ev1);
-    const int64_t units = (int64_t)num_experts * (n / 64);
+    const int64_t units = (int64_t)pair_places(a) * (n / 64);
     // as the sorted form chooses: a wavefront per unit when there are enough units and K is short, and the units
     // of an expert come in fours (a workgroup collects the pairs of one expert)
     if (units >= 2048 && k < 2048 && (n / 64) % 4 == 0)
@@ -998,7 +1046,7 @@ extern "C" int moe355_gmm1_swiglu_pairs(const int8_t* x, const float* x_scale, c
     a.pair_gather = 1;
     hipEvent_t ev0, ev1;
     take_profile_events(ev0, ev1);
-    const int64_t units = (int64_t)num_experts * (n / 64);
+    const int64_t units = (int64_t)pair_places(a) * (n / 64);
     launch_gemm(gmm_stream_kernel<EPI_SWIGLU, 4, 4, 3, false, true, true>, dim3((unsigned)units), (hipStream_t)stream, a,
                 ev0, ev1);
     return launch_status();
@@ -1043,7 +1091,7 @@ extern "C" int moe355_gmm2_requant_dequant_pairs(const float* y, const int8_t* w
     a.pair_gather = 0;
     hipEvent_t ev0, ev1;
     take_profile_events(ev0, ev1);
-    const int64_t units = (int64_t)num_experts * (n / 64);
+    const int64_t units = (int64_t)pair_places(a) * (n / 64);
     const unsigned lds = (unsigned)(32 * (k + 16));
     auto kernel = gmm_stream_kernel<EPI_DEQUANT, 1, 4, 2, false, true, true, true>;
     const dim3 grid((unsigned)((units + 3) / 4));

@@ -38,6 +38,9 @@ struct GmmArgs {
     // order) or in row f, and its result goes to row f.
     const int32_t* pair_ids;
     int pair_k, pair_gather;
+    // > 0: the grid has pair_slots places instead of E, and place s works on the s-th expert that has pairs (fewer
+    // pairs than experts: most experts are idle)
+    int pair_slots;
     // pair order, down GEMM with the re-quantisation inside (REQ): the SwiGLU values [R, K] fp32 that the gate_up
     // GEMM wrote; the workgroup quantises the rows of its expert itself (x and row_scale are not read)
     const float* y_in;
