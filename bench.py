@@ -172,8 +172,6 @@ def run_workload(name, args, lib, torch, np):
     dev = "cuda:0"
     cfg = CONFIGS[name]
     if args.tokens:
-        import dataclasses
-
         cfg = dataclasses.replace(cfg, T=args.tokens)  # the same layer on a batch of another size
     t_start = time.perf_counter()
     dg = make_layer(cfg, seed=0, gen_device=dev)
