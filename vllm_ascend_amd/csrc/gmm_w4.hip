@@ -427,7 +427,10 @@ __global__ __launch_bounds__(256, 2) void gmm_w4_stream_kernel(W4Args p)
 // list) times the groups of four tile pairs
 static int64_t w4_blocks(int64_t rows, int num_experts, int64_t n)
 {
-    return (rows / kW4Chunk + num_experts) * ((n / 64 + 3) / 4);
+    // a chunk has at least one row: a decode batch of a few rows has a few chunks, not one per expert (a workgroup
+    // that only finds its chunk missing still costs its dispatch)
+    const int64_t by_experts = rows / kW4Chunk + num_experts;
+    return (rows < by_experts ? rows : by_experts) * ((n / 64 + 3) / 4);
 }
 
 template <int EPI>
