@@ -60,6 +60,27 @@ __global__ __launch_bounds__(256) void format_cast_nz_kernel(const int8_t* __res
 // one expert (KSPLIT == 1: four units of it; the host picks that form only when the units of an expert come in
 // fours), scan a quarter of the ids each and leave the expert's pairs, in ascending order, in LDS.  The routing
 // launch in front of the GEMM then is gating and quantisation only: no sort, no hand-off between workgroups.
+// the n-th expert (counting from 0) whose group has rows, or -1: every lane of the wavefront calls it and gets the
+// same answer (64 experts per step: one load per lane, a ballot, a count of bits)
+__device__ __forceinline__ int nth_expert_with_rows(const int64_t* gl, int gl_type, int E, int n, int lane)
+{
+    int seen = 0;
+    for (int base = 0; base < E; base += 64) {
+        const int e = base + lane;
+        int64_t c = 0;
+        if (e < E) c = (gl_type == 1) ? gl[e] : gl[e] - (e ? gl[e - 1] : 0);
+        const unsigned long long m = __ballot(c > 0);
+        const int pc = __popcll(m);
+        if (n < seen + pc) {
+            unsigned long long t = m;
+            for (int i = n - seen; i > 0; --i) t &= t - 1;
+            return base + __builtin_ctzll(t);
+        }
+        seen += pc;
+    }
+    return -1;
+}
+
 constexpr int kPairMax = 1024;
 
 // REQ (pair order, down GEMM): the activation is still the fp32 SwiGLU output; the workgroup re-quantises the rows
@@ -89,7 +110,7 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
     // pair order with fewer pairs than experts: the grid has a slot per pair instead of a place per expert (most
     // experts are idle, and a workgroup that only finds that out still costs its dispatch: 28,000 of them are
     // 150 us), and slot s belongs to the s-th expert that has pairs at all
-    const int places = (PAIRS && a.pair_slots > 0) ? a.pair_slots : a.E;
+    const int places = (PAIRS && a.pair_slots > 0) ? a.pair_slots : (!PAIRS && !EARLY && a.gl_slots > 0) ? a.gl_slots : a.E;
     if (unit >= (int64_t)places * upe) return;  // KSPLIT == 1: no barriers below; KSPLIT == 4: whole workgroup leaves
     int e = (int)(unit / upe);
     const int p = (int)(unit % upe);
@@ -146,6 +167,12 @@ __global__ __launch_bounds__(256, OCC) void gmm_stream_kernel(GmmArgs a)
             for (int i = has ? e - excl : 0; i > 0; --i) t &= t - 1;
             const int mine = lane * 32 + (t ? __builtin_ctz(t) : 0);
             e = __shfl(mine, __builtin_ctzll(holder), 64);
+        }
+    }
+    if constexpr (!PAIRS && !EARLY) {
+        if (a.gl_slots > 0) {  // few rows over many experts: the workgroup's place is a slot, not an expert
+            e = nth_expert_with_rows(a.gl, a.gl_type, a.E, e, lane);
+            if (e < 0) return;
         }
     }
     const int8_t* we = expert_weights(a, e);
@@ -665,6 +692,13 @@ static int launch_gemm_auto(const GmmArgs& a_in, void* tile_ws, hipStream_t st, 
         // itself (no K split, no LDS reduction); otherwise the four wavefronts of a workgroup split K (from
         // K = 2048 on that measured 1.5 % faster on the whole layer, below it the same or slower).
         if (done) {
+        } else if (plan.split == 0 && a.gl && a.R < (int64_t)a.E) {
+            // fewer rows than experts (a decode batch of a few tokens on the sorted path): a slot per row instead
+            // of a place per expert, so that the idle experts cost no dispatch; the workgroup looks up the expert
+            // of its slot in the group list, so nothing is requested before that
+            a.gl_slots = (int)a.R;
+            launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, false, false>, dim3((unsigned)(a.R * (a.N / 64))), st, a, ev0,
+                        first_stop);
         } else if (plan.split > 0) {
             launch_gemm(gmm_stream_kernel<EPI, 4, 4, 3, false, false>, dim3((unsigned)units), st, a, ev0, first_stop);
         } else if (EPI != EPI_SWIGLU && units >= 2048 && a.K < 2048) {

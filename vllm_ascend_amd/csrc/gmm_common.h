@@ -41,6 +41,9 @@ struct GmmArgs {
     // > 0: the grid has pair_slots places instead of E, and place s works on the s-th expert that has pairs (fewer
     // pairs than experts: most experts are idle)
     int pair_slots;
+    // the same for a sorted activation with fewer rows than experts: place s works on the s-th expert whose group
+    // is not empty
+    int gl_slots;
     // pair order, down GEMM with the re-quantisation inside (REQ): the SwiGLU values [R, K] fp32 that the gate_up
     // GEMM wrote; the workgroup quantises the rows of its expert itself (x and row_scale are not read)
     const float* y_in;
