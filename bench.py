@@ -173,6 +173,8 @@ def run_workload(name, args, lib, torch, np):
     cfg = CONFIGS[name]
     if args.tokens:
         cfg = dataclasses.replace(cfg, T=args.tokens)  # the same layer on a batch of another size
+    if args.zipf is not None:
+        cfg = dataclasses.replace(cfg, zipf=args.zipf)  # ... with another skew of the expert popularity
     t_start = time.perf_counter()
     dg = make_layer(cfg, seed=0, gen_device=dev)
     layer = build_layer(cfg, dg, dev, shared=cfg.shared, overlap=False)
@@ -299,7 +301,7 @@ def run_workload(name, args, lib, torch, np):
                 kernel = "gmm_w4_stream_kernel"
             else:
                 kernel = lib.moe355_gmm_kernel_name(1, R, cfg.H, 2 * cfg.I, cfg.E).decode()
-            traffic = None if args.tokens else TRAFFIC_FROM_PROFILES.get(name)
+            traffic = None if (args.tokens or args.zipf is not None) else TRAFFIC_FROM_PROFILES.get(name)
             roofline.update({
                 "traffic": traffic[0] if traffic else None,
                 "traffic_source": (traffic[1] + " (rocprofv3 --pmc of an earlier run of this command, not measured "
@@ -409,6 +411,8 @@ def main() -> int:
                     help="one workload or a comma-separated list; default: all of " + ", ".join(WORKLOADS))
     ap.add_argument("--tokens", type=int, default=0,
                     help="run the named workload(s) on a batch of this many tokens instead of their own")
+    ap.add_argument("--zipf", type=float, default=None,
+                    help="expert popularity ~ rank^-S for the named workload(s) instead of their own (0: uniform)")
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--with-gate", action="store_true",
                     help="start the step one operator earlier: the fp32 router gate GEMM (hidden states -> logits, "

@@ -948,18 +948,24 @@ extern "C" int moe355_gmm_pairs_supported(int64_t num_tokens, int top_k, int64_t
     return num_tokens > 0 && top_k > 0 && num_tokens * top_k <= kPairMax && n > 0 && k > 0 && n % 64 == 0 && k % 32 == 0;
 }
 
-// pair order: how many places the grid gets.  A place per expert makes every idle expert cost the dispatch of its
-// workgroups (about 5 ns each: at one token of the DeepSeek-V3 shape 28,000 of them, 150 us); with few pairs the grid
-// gets a slot per pair instead (at most one per expert) and the kernel looks up which expert a slot belongs to.
-// Measured (whole layer, graph replay): DeepSeek-V3 shape 1 / 8 / 32 / 64 tokens 307 -> 104, 567 -> 403,
-// 1174 -> 1114, 1492 -> 1475 us; Qwen3 shape 1 / 4 / 16 tokens 48 -> 38, 62 -> 42, 91 -> 86 us, and from 24 tokens
-// on (more pairs than experts, 24 or 32 units per expert) the lookup costs what the few idle experts saved.  The
-// bit map of the lookup holds 2048 experts.
+// pair order: how many places the grid gets.  A place per expert lets a workgroup request its first weight tiles
+// before it has seen a single id, which is the fastest form when nearly every expert has pairs -- and makes every
+// idle expert cost the dispatch of its workgroups plus 32 KiB of weights requested for nothing.  A slot per pair
+// (at most one per expert; the kernel looks up which expert a slot belongs to, and requests nothing before) costs
+// every launch one exposed lookup, and nothing for idle experts.  Measured, whole layer under graph replay:
+//   DeepSeek-V3 shape, uniform routing, 1 / 8 / 32 / 64 / 128 tokens: 307 -> 104, 567 -> 403, 1174 -> 1114,
+//     1492 -> 1475, 1641 -> 1639 us; Zipf(1.1) routing, 96 / 128 tokens: 719 -> 599, 839 -> 731 us
+//   Qwen3 shape, uniform, 1 / 4 / 16 / 64 / 128 tokens: 48 -> 38, 62 -> 42, 91 -> 86, 111.7 -> 114.3, 116 -> 120 us;
+//     Zipf(1.1), 24 / 64 / 128 tokens: 80.5 -> 63.3, 108.9 -> 83.0, 169.6 -> 127.4 us
+// The host cannot know the skew.  Slots wherever uniform routing loses nothing by them: up to two pairs per expert,
+// and at any number of pairs when an expert has 48 units and more (the DeepSeek-V3 shape); with more pairs over
+// experts of few units (the Qwen3 shape from 40 tokens on) a place per expert, which is the faster form on uniform
+// routing and the slower one on skewed routing.  The bit map of the lookup holds 2048 experts.
 static int pair_places(GmmArgs& a)
 {
     const int64_t places = a.R < (int64_t)a.E ? a.R : (int64_t)a.E;
-    const bool few = a.R <= (int64_t)a.E || (a.R <= 2 * (int64_t)a.E && a.N / 64 >= 48);
-    a.pair_slots = (few && a.E <= 2048) ? (int)places : 0;
+    const bool slots = a.R <= 2 * (int64_t)a.E || a.N / 64 >= 48;
+    a.pair_slots = (slots && a.E <= 2048) ? (int)places : 0;
     return (int)(a.pair_slots > 0 ? places : a.E);
 }
 
