@@ -811,6 +811,9 @@ SKEWED = {
     "stream+wide": (_HOT + [12] * 240, 4096, 1024),
     "stream+wide, nothing above the border": ([16] * 224 + [32] * 32, 4096, 1024),
     "stream+tiled": (_HOT + [12] * 240, 2048, 2048),
+    # a decode batch (fewer than 1024 rows, most experts idle) on a product of a GiB: split from one row per expert on
+    "stream+wide, decode batch": ([0] * 200 + [1] * 40 + [2] * 8 + [300, 40, 33, 32, 31, 0, 5, 65], 4096, 1024),
+    "stream+tiled, decode batch": ([0] * 200 + [1] * 40 + [2] * 8 + [300, 40, 33, 32, 31, 0, 5, 65], 2048, 2048),
     "tiled": (_HOT + [12] * 240, 256, 256),
     "wide": ([255, 256, 257, 511, 513, 1, 0, 33, 128, 160, 161, 192, 193, 40, 90, 100], 1024, 256),
     "wide, K 4096": ([300, 20, 256, 257, 47, 150, 0, 90], 4096, 256),

@@ -570,7 +570,8 @@ static int tiled_bm(const GmmArgs& a)
 
 // What one operator call launches: the family chosen from the mean rows per expert, restricted to the experts it
 // is good at, and (split > 0) the 128-row tiles for the experts above that range.
-//   mean < 24 (12..23 for products of a GiB of weights and more, see tiled_bm) and at least 1024 rows: streaming
+//   mean < 24 (12..23 for products of a GiB of weights and more, see tiled_bm; such products from one row per
+//     expert on, smaller ones from 1024 rows on): streaming
 //     for experts of at most 32 rows (one pass over their weights, and no request before the group list says that
 //     the expert is theirs), tiles for the others -- a 500-row expert would otherwise stream its weights 16 times
 //     while the units of the cold experts have long finished.  Measured at the DeepSeek-V3 shape with Zipf(1.1)
@@ -601,8 +602,12 @@ static GemmPlan gemm_plan(const GmmArgs& a, bool have_tile_ws)
         return p;
     }
 #endif
-    // a large product (a GiB of weights and more) over many experts with few rows on average
-    if (p.bm == 0 && a.R >= 1024 && (int64_t)a.E * a.N * a.K >= (1ll << 30)) {
+    // a large product (a GiB of weights and more) over many experts with few rows on average.  Decode batches
+    // too, from one row per expert on: on uniform routing the second launch finds nothing to do and costs 3 to 8 us,
+    // on skewed routing the hot experts leave the streaming kernel (which also requests nothing for an idle expert
+    // in this form).  DeepSeek-V3 shape through the sorted path, 32 / 64 / 112 tokens: uniform 1216 -> 1159,
+    // 1500 -> 1490, 1648 -> 1656 us; Zipf(1.1) 529 -> 391, 640 -> 533, 796 -> 625 us.
+    if (p.bm == 0 && a.R >= 128 && a.R >= (int64_t)a.E && (int64_t)a.E * a.N * a.K >= (1ll << 30)) {
         p.split = 32;
         // the experts above the border: weight-streaming tiles when K is long (an expert of up to 256 rows fetches
         // its weights once), 128-row tiles otherwise.  Measured on 512 tokens of Zipf(1.1) routing at the
