@@ -220,6 +220,11 @@ class AscendW8A8DynamicFusedMoEMethod(AscendMoEScheme):
         experts = layer.w13_weight.shape[0]  # physical experts (more than E with redundant copies behind log2phy)
         if not kernels.gate_quant_supported(T, k, E) or experts > 2048:
             return False
+        if experts * w13.shape[1] * w13.shape[2] >= 1 << 30 and T * k > 768:
+            # A product of a GiB and more has a second kernel family for hot experts on the sorted path (csrc/gmm.hip:
+            # gemm_plan), pair order streams every expert: DeepSeek-V3 shape under Zipf(1.1) routing, 112 / 128 tokens
+            # 668 / 742 us in pair order, 625 / 641 us sorted; on uniform routing pair order leads by 1 % there.
+            return False
         return T * k < 1024 or (T * k) // experts < 12  # where the sorted form streams as well (csrc/gmm.hip: tiled_bm)
 
     def _experts_in_pair_order(self, layer, x, router_logits, router, shared_experts, shared_experts_input,
