@@ -49,12 +49,12 @@ WORKLOADS = ["c4_dsv3_prefill", "c2_qwen3_decode", "c3_qwen3_prefill", "c5_w4a8_
 # kernel of known size), taken from the committed summaries: NOT measured in this run.
 TRAFFIC_FROM_PROFILES = {
     "c2_qwen3_decode": (401_500_000, "profiles/moe_layer_qwen3_decode_kernel_trace.md"),
-    "c3_qwen3_prefill": (952_500_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
+    "c3_qwen3_prefill": (952_400_000, "profiles/moe_layer_qwen3_prefill_kernel_trace.md"),
     "c4_dsv3_prefill": (8_030_700_000, "profiles/moe_layer_dsv3_prefill_kernel_trace.md"),
     "c5_w4a8_zipf": (1_662_500_000, "profiles/moe_layer_w4a8_zipf_kernel_trace.md"),
-    "c6_dsv3_decode": (6_611_000_000, "profiles/moe_layer_dsv3_decode_kernel_trace.md"),
-    "c7_w8a8_zipf": (2_892_000_000, "profiles/moe_layer_w8a8_zipf_kernel_trace.md"),
-    "c7_w8a8_zipf_4096": (8_313_700_000, "profiles/moe_layer_w8a8_zipf_4096_kernel_trace.md"),
+    "c6_dsv3_decode": (6_600_600_000, "profiles/moe_layer_dsv3_decode_kernel_trace.md"),
+    "c7_w8a8_zipf": (2_892_100_000, "profiles/moe_layer_w8a8_zipf_kernel_trace.md"),
+    "c7_w8a8_zipf_4096": (8_314_400_000, "profiles/moe_layer_w8a8_zipf_4096_kernel_trace.md"),
 }
 
 
