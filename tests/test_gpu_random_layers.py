@@ -29,6 +29,9 @@ def _draw(seed: int) -> LayerCfg:
             topk_group = int(r.integers(1, n_group + 1))
             if k > topk_group * (E // n_group):
                 k = topk_group * (E // n_group)
+            # the router's guard in front of the fused gating op (it measures the hidden size, as the reference's does)
+            if k > H / (n_group * topk_group) or H // n_group <= 2:
+                n_group = topk_group = 1
     # mostly decode-sized batches, some with enough rows for the tiled kernels; bounded checker time
     T = int(r.choice([1, 3, 17, 64, 130, 257, 700, 1500, 2600]))
     while T * k * H * I > 1.2e10 and T > 1:

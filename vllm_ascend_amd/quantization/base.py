@@ -61,6 +61,9 @@ def fused_front_supported(layer, x: torch.Tensor, router_logits: torch.Tensor, r
         return False
     if getattr(layer, "enable_force_load_balance", False):
         return False
+    guard = getattr(router, "is_fused_supported", None)
+    if guard is not None and not guard(x):
+        return False  # the router's own guard decides (and refuses) on the operator-by-operator path
     if getattr(layer, "log2phy", None) is not None:  # the ids are remapped between gating and dispatch
         return kernels.gate_quant_supported(x.shape[0], router.top_k, router_logits.shape[1])
     return (kernels.route_quant_small_supported(x.shape[0], router.top_k, router_logits.shape[1])
