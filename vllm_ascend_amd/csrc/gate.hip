@@ -422,6 +422,8 @@ extern "C" int moe355_router_gate(const void* x, int x_dtype, const float* weigh
             }
         }
     }
+    // the plan never puts four wavefronts on a tile of fp32 tokens (no such kernel is built)
+    if (x_dtype == MOE355_DT_F32 && (first.kw == 4 || rest.kw == 4)) return MOE355_E_UNSUPPORTED;
     launch(first, 0, main_tokens);
     if (main_tokens < num_tokens) launch(rest, main_tokens, num_tokens - main_tokens);
     if (g.split) {
