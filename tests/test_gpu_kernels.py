@@ -1099,6 +1099,44 @@ def test_grouped_gemms_on_random_problems(K, orc, seed):
     assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
 
 
+# Fewer rows than experts (a decode batch of a few tokens on the sorted path): the grid has a slot per row and a
+# workgroup looks up the expert of its slot in the group list.  Random histograms with most experts empty.
+@pytest.mark.parametrize("seed", range(10))
+def test_grouped_gemms_with_fewer_rows_than_experts(K, orc, seed):
+    from vllm_ascend_amd._lib import W_ENK
+
+    rng = np.random.default_rng(500 + seed)
+    E = int(rng.integers(2, 320))
+    R = int(rng.integers(1, E))
+    Kd = int(rng.choice([64, 128, 192, 512, 1024, 2048]))
+    N = int(rng.choice([64, 128, 320, 576]))
+    cnt = np.zeros(E, dtype=np.int64)
+    for _ in range(R):
+        cnt[int(rng.integers(E)) if rng.random() < 0.7 else int(rng.integers(min(E, 4)))] += 1
+    print(f"few rows seed={seed} E={E} R={R} K={Kd} N={N} experts with rows={int((cnt > 0).sum())}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randint(-128, 128, (R, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (E, N, Kd), generator=g, dtype=torch.int8)
+    sw = torch.rand(E, N, generator=g) * 0.009 + 0.001
+    sx = torch.rand(R, generator=g) * 0.05 + 0.001
+    cnt_t = torch.from_numpy(cnt)
+    cum = torch.cumsum(cnt_t, 0)
+    wnz = K.format_cast_nz(w.to(DEV), W_ENK)
+    ref = orc.gmm_i32(x.numpy(), w.numpy(), cum.numpy())
+    acc = K.gmm_i32(x.to(DEV), wnz, cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+    want = orc.gmm2_dequant(ref, sx.numpy(), sw.numpy(), cum.numpy())
+    got = K.gmm2_dequant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cnt_t.to(DEV), 1, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got.cpu()), want)
+    q_want, s_want = orc.swiglu_quant(orc.dequant_acc(ref, sx.numpy(), sw.numpy(), cum.numpy()))
+    q, s_ = K.gmm1_swiglu_quant(x.to(DEV), wnz, sw.to(DEV), sx.to(DEV), cum.to(DEV), 0, N, Kd)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_want)
+    assert np.array_equal(s_.cpu().numpy().view(np.uint32), s_want.view(np.uint32))
+
+
 # The expert MLP of a decode batch in pair order (no sort): every stage against the sorted form of the checker,
 # rows moved to pair order through the checker's own expanded_row_idx.
 @pytest.mark.parametrize("T,k,E,H,I", [(64, 8, 128, 2048, 768), (8, 8, 128, 2048, 768), (48, 8, 128, 2048, 768),
